@@ -1,0 +1,124 @@
+/*
+ * libjitnn_hip.so - MI355X (gfx950) implementation of jitNN's GGUF quantised-weight linear path.
+ *
+ * Plain C ABI: opaque handles, raw pointers and sizes; no C++ or torch types.  Every function returns
+ * an int status (JITNN_HIP_OK or a negative JITNN_HIP_E* code) unless stated otherwise, never throws and
+ * never aborts the process; jitnn_hip_last_error() gives the message of the calling thread's last failure.
+ *
+ * Each entry point names the reference interface it stands in for (paths relative to the reference
+ * root; "core/" = jitnn-core/src/main/java/ai/beestream/jitnn/, "gguf/" =
+ * jitnn-gguf/src/main/java/ai/beestream/jitnn/gguf/).
+ *
+ * Conventions
+ *  - fmt is the ggml type id stored in GGUF files (gguf/GgmlType.java:27-65):
+ *    Q4_0=2 Q4_1=3 Q8_0=8 Q4_K=12 Q5_K=13 Q6_K=14.
+ *  - A weight is [n, k] row-major rows of k/block_values blocks, byte-for-byte as in the GGUF file
+ *    (core/Tensor.java:249-278); it stays in that layout in HBM.
+ *  - Activations and outputs are FP32 row-major: x [rows, k], y [rows, n], bias [n].
+ *  - "_dev" entry points take device pointers and a hipStream_t passed as void* (NULL = the null stream);
+ *    they only enqueue work.  Entry points without "_dev" take host pointers and are synchronous.
+ *  - Thread safety: weights are immutable after upload and may be shared by any number of threads;
+ *    each call uses only its arguments and per-call stream order; the last-error string is thread-local.
+ */
+#ifndef JITNN_HIP_H
+#define JITNN_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JITNN_HIP_API __attribute__((visibility("default")))
+
+#define JITNN_HIP_OK 0
+#define JITNN_HIP_EINVAL (-1)   /* bad argument: unknown format, k not a multiple of the block, size mismatch, NULL */
+#define JITNN_HIP_EDEVICE (-2)  /* a HIP runtime call failed */
+#define JITNN_HIP_ENODEVICE (-3) /* no gfx950 device / library not initialised */
+#define JITNN_HIP_ENOMEM (-4)
+
+#define JITNN_HIP_Q4_0 2
+#define JITNN_HIP_Q4_1 3
+#define JITNN_HIP_Q8_0 8
+#define JITNN_HIP_Q4_K 12
+#define JITNN_HIP_Q5_K 13
+#define JITNN_HIP_Q6_K 14
+
+typedef struct jitnn_hip_weight jitnn_hip_weight;
+
+/* ---- library and device ------------------------------------------------------------------------ */
+
+/* Selects the device and prepares the kernels; idempotent.  The counterpart of binding an optional native
+ * library at start-up (core/cpu/Blas.java:59-104): on failure the caller keeps its own path. */
+JITNN_HIP_API int jitnn_hip_init(int device_ordinal);
+
+/* Device name (NUL-terminated, truncated to cap), compute units and HBM bytes. */
+JITNN_HIP_API int jitnn_hip_device_info(char *name, int cap, int *compute_units, long long *hbm_bytes);
+
+/* Message of the calling thread's last failed call; never NULL.  Failures surface in Java as
+ * JitnnException("calling ... failed", cause) (core/cpu/Blas.java:195-200, core/JitnnException.java:18-25). */
+JITNN_HIP_API const char *jitnn_hip_last_error(void);
+
+JITNN_HIP_API int jitnn_hip_sync(void);
+
+/* ---- block formats (no device needed) ------------------------------------------------------------ */
+
+/* Values per block / bytes per block of a format, 0 when fmt is not one of the six
+ * (core/DType.java:75-98, gguf/GgmlType.java:113-118). */
+JITNN_HIP_API int jitnn_hip_block_values(int fmt);
+JITNN_HIP_API int jitnn_hip_block_bytes(int fmt);
+
+/* Bytes an [n, k] weight takes, or JITNN_HIP_EINVAL (unknown fmt, n < 1, k < 1, k not a multiple of the block):
+ * the check of Tensor.persistent (core/Tensor.java:266-276). */
+JITNN_HIP_API long long jitnn_hip_weight_nbytes(int fmt, long long n, long long k);
+
+/* ---- weights ------------------------------------------------------------------------------------ */
+
+/* Copies raw blocks from host memory to HBM unchanged.  Stands in for the upload of a persistent
+ * block-quantised storage (Tensor.quantized / Tensor.persistent, core/Tensor.java:249-278; the bytes come
+ * from GgufFile.tensor / raw, gguf/GgufFile.java:329-366).  nbytes must equal jitnn_hip_weight_nbytes. */
+JITNN_HIP_API int jitnn_hip_weight_upload(int fmt, const void *blocks_host, long long nbytes, int n, int k, jitnn_hip_weight **out);
+
+/* Wraps blocks that are already in device memory (not copied, not owned: the caller keeps them alive).
+ * dev_blocks must be 16-byte aligned. */
+JITNN_HIP_API int jitnn_hip_weight_wrap_dev(int fmt, const void *dev_blocks, long long nbytes, int n, int k, jitnn_hip_weight **out);
+
+JITNN_HIP_API int jitnn_hip_weight_free(jitnn_hip_weight *w);
+
+/* Shape and format of a weight; any out pointer may be NULL. */
+JITNN_HIP_API int jitnn_hip_weight_info(const jitnn_hip_weight *w, int *fmt, int *n, int *k, long long *nbytes);
+
+/* ---- dequantise --------------------------------------------------------------------------------- */
+
+/* y[i] = value(w, i), i < n*k, bit-identical to the reference's per-value decode:
+ * Gguf.dequantize / op gguf_dequantize (core/ops/Gguf.java:68-73,127-133), Quant.dequantize / op
+ * dequantize_q8_0 (core/ops/Quant.java:53-60,137-144), Tensor.toFloatArray on block tensors
+ * (core/Tensor.java:539-555). */
+JITNN_HIP_API int jitnn_hip_dequantize(const jitnn_hip_weight *w, float *y_host);
+JITNN_HIP_API int jitnn_hip_dequantize_dev(const jitnn_hip_weight *w, float *y_dev, void *stream);
+
+/* ---- linear ------------------------------------------------------------------------------------- */
+
+/* y = x W^T (+ bias): Gguf.linear (core/ops/Gguf.java:76-98; ops gguf_matvec :136-205 and
+ * gguf_dequantize + matmul) and, for Q8_0, F.linearQ8 / Quant.linear (core/F.java:1049-1051,
+ * core/ops/Quant.java:66-80,147-187).  rows >= 1; bias may be NULL.
+ * rows <= 8 run the GEMV kernels (FP32 accumulation); more rows run the dequantise-to-LDS MFMA kernel. */
+JITNN_HIP_API int jitnn_hip_linear(const jitnn_hip_weight *w, const float *x_host, int rows, const float *bias_host, float *y_host);
+JITNN_HIP_API int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, void *stream);
+
+/* ---- Q8_0 quantiser ----------------------------------------------------------------------------- */
+
+/* FP32 -> Q8_0 blocks (34 bytes per 32 values) with the reference quantiser's arithmetic: F.quantizeQ8 /
+ * op quantize_q8_0 (core/F.java:1039-1041, core/ops/Quant.java:42-50,102-118).  numel % 32 == 0. */
+JITNN_HIP_API int jitnn_hip_quantize_q8_0(const float *x_host, long long numel, void *blocks_host);
+JITNN_HIP_API int jitnn_hip_quantize_q8_0_dev(const float *x_dev, long long numel, void *blocks_dev, void *stream);
+
+/* ---- device memory for callers that have no HIP binding of their own (the Java side) ------------- */
+
+JITNN_HIP_API int jitnn_hip_malloc(long long nbytes, void **dev);
+JITNN_HIP_API int jitnn_hip_free(void *dev);
+JITNN_HIP_API int jitnn_hip_memcpy_h2d(void *dev, const void *host, long long nbytes);
+JITNN_HIP_API int jitnn_hip_memcpy_d2h(void *host, const void *dev, long long nbytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JITNN_HIP_H */

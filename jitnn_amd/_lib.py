@@ -1,0 +1,87 @@
+"""ctypes binding of libjitnn_hip.so (the C ABI in include/jitnn_hip.h).
+
+The library is the only implementation of the path: if it is missing or cannot be loaded this module
+raises, there is no other code path to fall back to.  It is built in-tree by jitnn_amd/csrc/Makefile
+(see __graft_entry__.build).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libjitnn_hip.so"
+
+OK, EINVAL, EDEVICE, ENODEVICE, ENOMEM = 0, -1, -2, -3, -4
+
+
+class JitnnError(RuntimeError):
+    """A native call failed (the reference's JitnnException, core/JitnnException.java:18-25)."""
+
+
+def _bind() -> C.CDLL:
+    if not LIB_PATH.exists():
+        raise JitnnError(f"{LIB_PATH} is not built: run `make -C jitnn_amd/csrc` (or __graft_entry__.build())")
+    lib = C.CDLL(str(LIB_PATH))
+    vp, i, ll, fp = C.c_void_p, C.c_int, C.c_longlong, C.POINTER(C.c_float)
+    sig = {
+        "jitnn_hip_init": (i, [i]),
+        "jitnn_hip_device_info": (i, [C.c_char_p, i, C.POINTER(i), C.POINTER(ll)]),
+        "jitnn_hip_last_error": (C.c_char_p, []),
+        "jitnn_hip_sync": (i, []),
+        "jitnn_hip_block_values": (i, [i]),
+        "jitnn_hip_block_bytes": (i, [i]),
+        "jitnn_hip_weight_nbytes": (ll, [i, ll, ll]),
+        "jitnn_hip_weight_upload": (i, [i, vp, ll, i, i, C.POINTER(vp)]),
+        "jitnn_hip_weight_wrap_dev": (i, [i, vp, ll, i, i, C.POINTER(vp)]),
+        "jitnn_hip_weight_free": (i, [vp]),
+        "jitnn_hip_weight_info": (i, [vp, C.POINTER(i), C.POINTER(i), C.POINTER(i), C.POINTER(ll)]),
+        "jitnn_hip_dequantize": (i, [vp, vp]),
+        "jitnn_hip_dequantize_dev": (i, [vp, vp, vp]),
+        "jitnn_hip_linear": (i, [vp, vp, i, vp, vp]),
+        "jitnn_hip_linear_dev": (i, [vp, vp, i, vp, vp, vp]),
+        "jitnn_hip_quantize_q8_0": (i, [vp, ll, vp]),
+        "jitnn_hip_quantize_q8_0_dev": (i, [vp, ll, vp, vp]),
+        "jitnn_hip_malloc": (i, [ll, C.POINTER(vp)]),
+        "jitnn_hip_free": (i, [vp]),
+        "jitnn_hip_memcpy_h2d": (i, [vp, vp, ll]),
+        "jitnn_hip_memcpy_d2h": (i, [vp, vp, ll]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.restype, fn.argtypes = res, args
+    lib._signatures = sig
+    return lib
+
+
+lib = _bind()
+_initialised = False
+
+
+def last_error() -> str:
+    return lib.jitnn_hip_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int, what: str) -> None:
+    """0 passes; EINVAL is the caller's misuse (ValueError, the reference's IllegalArgumentException);
+    anything else is a failed native call (JitnnError)."""
+    if rc == OK:
+        return
+    msg = f"calling {what} failed: {last_error()}"
+    if rc == EINVAL:
+        raise ValueError(msg)
+    raise JitnnError(msg)
+
+
+def init(device: int = 0) -> None:
+    global _initialised
+    if not _initialised:
+        check(lib.jitnn_hip_init(device), "jitnn_hip_init")
+        _initialised = True
+
+
+def device_info() -> dict:
+    init()
+    name = C.create_string_buffer(256)
+    cus, hbm = C.c_int(), C.c_longlong()
+    check(lib.jitnn_hip_device_info(name, 256, C.byref(cus), C.byref(hbm)), "jitnn_hip_device_info")
+    return {"name": name.value.decode(), "compute_units": cus.value, "hbm_bytes": hbm.value}

@@ -1,0 +1,121 @@
+// Bit-exact dequantisation of raw GGUF blocks to FP32 and the Q8_0 quantiser.
+//
+// The arithmetic follows the reference's per-value decode operation by operation in binary32 with no fused
+// multiply-add (this translation unit is built with -ffp-contract=off): the integer fields are unpacked
+// with shifts and masks, which give the same integers as the reference's division/remainder form, and the
+// float expression is evaluated left to right exactly as written there
+// (reference: core/kernels/GgufKernels.java:61-140, core/ops/Quant.java:137-144).
+#pragma once
+#include "common.h"
+
+namespace jitnn {
+
+// 6-bit scale (part 0) or min (part 1) of sub-block j from the 12 scale bytes at s (GgufKernels.java:74-83).
+__device__ __forceinline__ int k4_scale_min(const uint8_t *s, int j, int part) {
+    if (j < 4) return s[j + 4 * part] & 63;
+    int low = part == 0 ? (s[j + 4] & 15) : (s[j + 4] >> 4);
+    return low | ((s[j - 4 + 4 * part] >> 6) << 4);
+}
+
+// Four consecutive values i..i+3 (i % 4 == 0) of a tensor: they share block, sub-block, nibble half and scale.
+template <int FMT>
+__device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
+    float o[4];
+    if constexpr (FMT == F_Q4_0) {
+        const uint8_t *b = w + (i >> 5) * 18;
+        const int e = (int)(i & 31);
+        const float d = h2f(ld16(b));
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            int v = b[2 + ((e + t) & 15)];
+            int q = e < 16 ? (v & 15) : (v >> 4);
+            o[t] = (float)(q - 8) * d;
+        }
+    } else if constexpr (FMT == F_Q4_1) {
+        const uint8_t *b = w + (i >> 5) * 20;
+        const int e = (int)(i & 31);
+        const float d = h2f(ld16(b)), m = h2f(ld16(b + 2));
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            int v = b[4 + ((e + t) & 15)];
+            int q = e < 16 ? (v & 15) : (v >> 4);
+            float p = (float)q * d;
+            o[t] = p + m;
+        }
+    } else if constexpr (FMT == F_Q8_0) {
+        const uint8_t *b = w + (i >> 5) * 34;
+        const int e = (int)(i & 31);
+        const float d = h2f(ld16(b));
+#pragma unroll
+        for (int t = 0; t < 4; ++t) o[t] = d * (float)(int)(int8_t)b[2 + e + t];
+    } else if constexpr (FMT == F_Q4_K || FMT == F_Q5_K) {
+        constexpr int NB = FMT == F_Q4_K ? 144 : 176, QS = FMT == F_Q4_K ? 16 : 48;
+        const uint8_t *b = w + (i >> 8) * NB;
+        const int e = (int)(i & 255);
+        const int j = e >> 6, half = (e & 63) >> 5, l = e & 31, sub = 2 * j + half;
+        const float ds = h2f(ld16(b)) * (float)k4_scale_min(b + 4, sub, 0);
+        const float m = h2f(ld16(b + 2)) * (float)k4_scale_min(b + 4, sub, 1);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            int v = b[QS + 32 * j + l + t];
+            int q = half == 0 ? (v & 15) : (v >> 4);
+            if constexpr (FMT == F_Q5_K) q += 16 * ((b[16 + l + t] >> sub) & 1);
+            float a = ds * (float)q;
+            o[t] = a - m;
+        }
+    } else {  // F_Q6_K
+        const uint8_t *b = w + (i >> 8) * 210;
+        const int e = (int)(i & 255);
+        const int n = e >> 7, k = (e & 127) >> 5, l = e & 31;
+        const int sc = (int)(int8_t)b[192 + 8 * n + (l >> 4) + 2 * k];
+        const float a = h2f(ld16(b + 208)) * (float)sc;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            int lb = b[64 * n + l + t + (k & 1) * 32];
+            int low = k < 2 ? (lb & 15) : (lb >> 4);
+            int hb = (b[128 + 32 * n + l + t] >> (2 * k)) & 3;
+            o[t] = a * (float)(low + 16 * hb - 32);
+        }
+    }
+    return make_float4(o[0], o[1], o[2], o[3]);
+}
+
+template <int FMT>
+__global__ void __launch_bounds__(256) dequant_kernel(const uint8_t *__restrict__ w, float *__restrict__ y, size_t quads) {
+    for (size_t f = (size_t)blockIdx.x * blockDim.x + threadIdx.x; f < quads; f += (size_t)gridDim.x * blockDim.x) {
+        reinterpret_cast<float4 *>(y)[f] = dequant4<FMT>(w, f * 4);
+    }
+}
+
+// FP32 -> Q8_0, one thread per block of 32 values, in the reference quantiser's arithmetic
+// (core/ops/Quant.java:102-118): amax in double, d = (float)(amax / 127.0) stored as binary16 (round to
+// nearest even), quants = round-half-away(x / (double)d) with the unrounded float d, clamped to +-127.
+__global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restrict__ x, uint8_t *__restrict__ q, size_t blocks) {
+    for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < blocks; b += (size_t)gridDim.x * blockDim.x) {
+        const float *xb = x + b * 32;
+        float v[32];
+#pragma unroll
+        for (int l = 0; l < 8; ++l) {
+            float4 t = reinterpret_cast<const float4 *>(xb)[l];
+            v[4 * l] = t.x; v[4 * l + 1] = t.y; v[4 * l + 2] = t.z; v[4 * l + 3] = t.w;
+        }
+        double amax = 0;
+#pragma unroll
+        for (int l = 0; l < 32; ++l) {
+            double a = fabs((double)v[l]);
+            amax = a > amax ? a : amax;
+        }
+        const float d = (float)(amax / 127.0);
+        uint8_t *o = q + b * 34;
+        *reinterpret_cast<uint16_t *>(o) = __half_as_ushort(__float2half_rn(d));
+#pragma unroll
+        for (int l = 0; l < 32; ++l) {
+            double s = d > 0 ? (double)v[l] / (double)d : 0.0;
+            long long r = s >= 0 ? (long long)(s + 0.5) : -(long long)(-s + 0.5);
+            r = r < -127 ? -127 : (r > 127 ? 127 : r);
+            o[2 + l] = (uint8_t)(int8_t)r;
+        }
+    }
+}
+
+}  // namespace jitnn

@@ -1,0 +1,404 @@
+// C-ABI entry points of libjitnn_hip.so (declared in include/jitnn_hip.h): argument validation, weight
+// handles, kernel selection and launch.  Host side of the path in C++; every kernel is in the headers
+// included below.
+#include "../../include/jitnn_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+
+#include "dequant.h"
+#include "gemv.h"
+
+using namespace jitnn;
+
+struct jitnn_hip_weight {
+    int fmt;
+    int n, k;
+    long long nbytes;
+    uint8_t *dev;
+    bool owned;
+};
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                                       \
+    do {                                                                                                    \
+        hipError_t e_ = (expr);                                                                             \
+        if (e_ != hipSuccess) return fail(JITNN_HIP_EDEVICE, "%s: %s", #expr, hipGetErrorString(e_));       \
+    } while (0)
+
+struct State {
+    bool ready = false;
+    int device = -1;
+    int cus = 0;
+    long long hbm = 0;
+    char name[256] = "";
+    float nib = 0.f;  // 1 / (value of E4M3 byte 0x01): 512 for OCP, 1024 for FNUZ
+    size_t max_lds = 0;
+};
+State g;
+std::mutex g_mu;
+
+__global__ void fp8_probe_kernel(float *out) {
+    f32x2 p = __builtin_amdgcn_cvt_pk_f32_fp8(0x00000f01, false);
+    out[0] = p.x;
+    out[1] = p.y;
+}
+
+bool known(int fmt) { return block_values(fmt) != 0; }
+
+int check_ready() {
+    if (!g.ready) return fail(JITNN_HIP_ENODEVICE, "jitnn_hip_init has not succeeded in this process");
+    return JITNN_HIP_OK;
+}
+
+// ------------------------------------------------------------------------------------------ launch tables
+
+typedef void (*gemv_fn)(const uint8_t *, const float *, const float *, float *, int, int, int, int, float);
+
+struct GemvVariant {
+    gemv_fn fn;
+    int B, R;
+    size_t lds_per_step;  // LDS bytes per staged wave step
+};
+
+template <int FMT, int B, int R>
+GemvVariant variant() {
+    // the fp8 nibble conversion only applies to the 4-bit formats; the others ignore CV
+    constexpr int CV = (FMT == F_Q4_K || FMT == F_Q4_0 || FMT == F_Q4_1) ? 1 : 0;
+    return GemvVariant{gemv_lds_kernel<FMT, B, R, CV>, B, R, gemv_lds_bytes<FMT>(B, 1)};
+}
+
+template <int FMT>
+GemvVariant pick_fmt(int rows) {
+    if (rows <= 1) return variant<FMT, 1, 4>();
+    if (rows <= 2) return variant<FMT, 2, 4>();
+    if (rows <= 4) return variant<FMT, 4, 2>();
+    return variant<FMT, 8, 2>();
+}
+
+GemvVariant pick(int fmt, int rows) {
+    switch (fmt) {
+    case F_Q4_0: return pick_fmt<F_Q4_0>(rows);
+    case F_Q4_1: return pick_fmt<F_Q4_1>(rows);
+    case F_Q8_0: return pick_fmt<F_Q8_0>(rows);
+    case F_Q4_K: return pick_fmt<F_Q4_K>(rows);
+    case F_Q5_K: return pick_fmt<F_Q5_K>(rows);
+    default: return pick_fmt<F_Q6_K>(rows);
+    }
+}
+
+int unit_values(int fmt) { return block_values(fmt) == 256 ? 64 : 32; }
+
+int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    GemvVariant v = pick(w->fmt, rows);
+    const int units = w->k / unit_values(w->fmt);
+    const int steps = (units + 63) / 64;
+    // stage as many steps as fit in 64 KiB (keeps several workgroups per CU); one step may need more
+    int itc = (int)(65536 / v.lds_per_step);
+    if (itc < 1) itc = 1;
+    if (itc > steps) itc = steps;
+    const size_t lds = v.lds_per_step * itc;
+    if (lds > g.max_lds) return fail(JITNN_HIP_EINVAL, "GEMV needs %zu bytes of LDS, the device offers %zu", lds, g.max_lds);
+    if (lds > 65536) HIP_TRY(hipFuncSetAttribute((const void *)v.fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    const int threads = 256, waves = threads / 64;
+    const int groups = (w->n + v.R - 1) / v.R;
+    int blocks = (groups + waves - 1) / waves;
+    const int cap = g.cus * 8;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(v.fn, dim3(blocks), dim3(threads), lds, stream, w->dev, x, bias, y, w->n, w->k, rows, itc, g.nib);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+template <int FMT>
+void launch_dequant(const jitnn_hip_weight *w, float *y, hipStream_t stream) {
+    const size_t quads = (size_t)w->n * w->k / 4;
+    size_t blocks = (quads + 255) / 256;
+    const size_t cap = (size_t)g.cus * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(dequant_kernel<FMT>, dim3((unsigned)blocks), dim3(256), 0, stream, w->dev, y, quads);
+}
+
+int check_weight_args(int fmt, long long nbytes, int n, int k, const void *blocks, jitnn_hip_weight **out) {
+    if (!out) return fail(JITNN_HIP_EINVAL, "out is NULL");
+    *out = nullptr;
+    if (!blocks) return fail(JITNN_HIP_EINVAL, "blocks is NULL");
+    long long need = jitnn_hip_weight_nbytes(fmt, n, k);
+    if (need < 0) return (int)need;
+    if (nbytes != need)
+        return fail(JITNN_HIP_EINVAL, "format %d weight of shape [%d, %d] needs %lld bytes, got %lld", fmt, n, k, need, nbytes);
+    return JITNN_HIP_OK;
+}
+
+}  // namespace
+
+// ================================================================================================ C ABI
+
+extern "C" {
+
+const char *jitnn_hip_last_error(void) { return g_err; }
+
+int jitnn_hip_block_values(int fmt) { return block_values(fmt); }
+int jitnn_hip_block_bytes(int fmt) { return block_bytes(fmt); }
+
+long long jitnn_hip_weight_nbytes(int fmt, long long n, long long k) {
+    if (!known(fmt)) return fail(JITNN_HIP_EINVAL, "ggml type id %d is not one of Q4_0, Q4_1, Q8_0, Q4_K, Q5_K, Q6_K", fmt);
+    if (n < 1 || k < 1) return fail(JITNN_HIP_EINVAL, "weight shape [%lld, %lld] is empty", n, k);
+    if (k % block_values(fmt) != 0)
+        return fail(JITNN_HIP_EINVAL, "format %d weight of shape [%lld, %lld]: last axis not a multiple of its block of %d", fmt, n, k,
+                    block_values(fmt));
+    if (n > 0x7fffffffLL || k > 0x7fffffffLL || n * k > 0x7fffffffLL)  // the reference's tensors hold at most Integer.MAX_VALUE values
+        return fail(JITNN_HIP_EINVAL, "weight shape [%lld, %lld] holds more than 2^31-1 values", n, k);
+    return n * (k / block_values(fmt)) * block_bytes(fmt);
+}
+
+int jitnn_hip_init(int device_ordinal) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g.ready) {
+        if (device_ordinal != g.device) return fail(JITNN_HIP_EINVAL, "already initialised on device %d", g.device);
+        return JITNN_HIP_OK;
+    }
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) return fail(JITNN_HIP_ENODEVICE, "no HIP device: %s", hipGetErrorString(e));
+    if (device_ordinal < 0 || device_ordinal >= count) return fail(JITNN_HIP_EINVAL, "device %d of %d", device_ordinal, count);
+    HIP_TRY(hipSetDevice(device_ordinal));
+    hipDeviceProp_t p;
+    HIP_TRY(hipGetDeviceProperties(&p, device_ordinal));
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+        return fail(JITNN_HIP_ENODEVICE, "device %d is %s; this library holds gfx950 code only", device_ordinal, p.gcnArchName);
+    snprintf(g.name, sizeof g.name, "%s (%s)", p.name, p.gcnArchName);
+    g.cus = p.multiProcessorCount;
+    g.hbm = (long long)p.totalGlobalMem;
+    int optin = 0;
+    if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, device_ordinal) != hipSuccess || optin <= 0)
+        optin = (int)p.sharedMemPerBlock;
+    g.max_lds = (size_t)optin;
+    float *probe = nullptr;
+    HIP_TRY(hipMalloc(&probe, 2 * sizeof(float)));
+    hipLaunchKernelGGL(fp8_probe_kernel, dim3(1), dim3(1), 0, 0, probe);
+    float h[2] = {0, 0};
+    hipError_t ce = hipMemcpy(h, probe, sizeof h, hipMemcpyDeviceToHost);
+    (void)hipFree(probe);
+    if (ce != hipSuccess) return fail(JITNN_HIP_EDEVICE, "fp8 probe: %s", hipGetErrorString(ce));
+    if (!(h[0] > 0.f) || h[1] != 15.f * h[0])
+        return fail(JITNN_HIP_EDEVICE, "fp8 probe: E4M3 bytes 0x01, 0x0f decode to %g, %g; expected q * 2^-9 or q * 2^-10", h[0], h[1]);
+    g.nib = 1.f / h[0];
+    g.device = device_ordinal;
+    g.ready = true;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_device_info(char *name, int cap, int *compute_units, long long *hbm_bytes) {
+    if (int rc = check_ready()) return rc;
+    if (name && cap > 0) {
+        strncpy(name, g.name, (size_t)cap - 1);
+        name[cap - 1] = 0;
+    }
+    if (compute_units) *compute_units = g.cus;
+    if (hbm_bytes) *hbm_bytes = g.hbm;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_sync(void) {
+    if (int rc = check_ready()) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_weight_upload(int fmt, const void *blocks_host, long long nbytes, int n, int k, jitnn_hip_weight **out) {
+    if (int rc = check_weight_args(fmt, nbytes, n, k, blocks_host, out)) return rc;
+    if (int rc = check_ready()) return rc;
+    uint8_t *dev = nullptr;
+    hipError_t e = hipMalloc(&dev, (size_t)nbytes);
+    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc of %lld bytes: %s", nbytes, hipGetErrorString(e));
+    e = hipMemcpy(dev, blocks_host, (size_t)nbytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return fail(JITNN_HIP_EDEVICE, "hipMemcpy of %lld bytes: %s", nbytes, hipGetErrorString(e));
+    }
+    jitnn_hip_weight *w = new (std::nothrow) jitnn_hip_weight{fmt, n, k, nbytes, dev, true};
+    if (!w) {
+        (void)hipFree(dev);
+        return fail(JITNN_HIP_ENOMEM, "out of host memory");
+    }
+    *out = w;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_weight_wrap_dev(int fmt, const void *dev_blocks, long long nbytes, int n, int k, jitnn_hip_weight **out) {
+    if (int rc = check_weight_args(fmt, nbytes, n, k, dev_blocks, out)) return rc;
+    if (((uintptr_t)dev_blocks & 15) != 0) return fail(JITNN_HIP_EINVAL, "device blocks must be 16-byte aligned");
+    jitnn_hip_weight *w = new (std::nothrow) jitnn_hip_weight{fmt, n, k, nbytes, (uint8_t *)dev_blocks, false};
+    if (!w) return fail(JITNN_HIP_ENOMEM, "out of host memory");
+    *out = w;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_weight_free(jitnn_hip_weight *w) {
+    if (!w) return JITNN_HIP_OK;
+    int rc = JITNN_HIP_OK;
+    if (w->owned && w->dev) {
+        hipError_t e = hipFree(w->dev);
+        if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipFree: %s", hipGetErrorString(e));
+    }
+    delete w;
+    return rc;
+}
+
+int jitnn_hip_weight_info(const jitnn_hip_weight *w, int *fmt, int *n, int *k, long long *nbytes) {
+    if (!w) return fail(JITNN_HIP_EINVAL, "weight is NULL");
+    if (fmt) *fmt = w->fmt;
+    if (n) *n = w->n;
+    if (k) *k = w->k;
+    if (nbytes) *nbytes = w->nbytes;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_dequantize_dev(const jitnn_hip_weight *w, float *y_dev, void *stream) {
+    if (!w || !y_dev) return fail(JITNN_HIP_EINVAL, "weight or output is NULL");
+    if (int rc = check_ready()) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (w->fmt) {
+    case F_Q4_0: launch_dequant<F_Q4_0>(w, y_dev, s); break;
+    case F_Q4_1: launch_dequant<F_Q4_1>(w, y_dev, s); break;
+    case F_Q8_0: launch_dequant<F_Q8_0>(w, y_dev, s); break;
+    case F_Q4_K: launch_dequant<F_Q4_K>(w, y_dev, s); break;
+    case F_Q5_K: launch_dequant<F_Q5_K>(w, y_dev, s); break;
+    default: launch_dequant<F_Q6_K>(w, y_dev, s); break;
+    }
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_dequantize(const jitnn_hip_weight *w, float *y_host) {
+    if (!w || !y_host) return fail(JITNN_HIP_EINVAL, "weight or output is NULL");
+    if (int rc = check_ready()) return rc;
+    const size_t bytes = (size_t)w->n * w->k * sizeof(float);
+    float *y = nullptr;
+    hipError_t e = hipMalloc(&y, bytes);
+    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc of %zu bytes: %s", bytes, hipGetErrorString(e));
+    int rc = jitnn_hip_dequantize_dev(w, y, nullptr);
+    if (rc == JITNN_HIP_OK) {
+        e = hipMemcpy(y_host, y, bytes, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(y);
+    return rc;
+}
+
+int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, void *stream) {
+    if (!w || !x_dev || !y_dev) return fail(JITNN_HIP_EINVAL, "weight, input or output is NULL");
+    if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
+    if (int rc = check_ready()) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    for (int r0 = 0; r0 < rows; r0 += 8) {
+        const int nb = rows - r0 < 8 ? rows - r0 : 8;
+        if (int rc = launch_gemv(w, x_dev + (size_t)r0 * w->k, nb, bias_dev, y_dev + (size_t)r0 * w->n, s)) return rc;
+    }
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_linear(const jitnn_hip_weight *w, const float *x_host, int rows, const float *bias_host, float *y_host) {
+    if (!w || !x_host || !y_host) return fail(JITNN_HIP_EINVAL, "weight, input or output is NULL");
+    if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
+    if (int rc = check_ready()) return rc;
+    const size_t xb = (size_t)rows * w->k * 4, yb = (size_t)rows * w->n * 4, bb = bias_host ? (size_t)w->n * 4 : 0;
+    uint8_t *buf = nullptr;
+    const size_t xo = 0, yo = (xb + 255) & ~(size_t)255, bo = yo + ((yb + 255) & ~(size_t)255);
+    hipError_t e = hipMalloc(&buf, bo + bb + 256);
+    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc: %s", hipGetErrorString(e));
+    int rc = JITNN_HIP_OK;
+    e = hipMemcpy(buf + xo, x_host, xb, hipMemcpyHostToDevice);
+    if (e == hipSuccess && bias_host) e = hipMemcpy(buf + bo, bias_host, bb, hipMemcpyHostToDevice);
+    if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    if (rc == JITNN_HIP_OK)
+        rc = jitnn_hip_linear_dev(w, (const float *)(buf + xo), rows, bias_host ? (const float *)(buf + bo) : nullptr, (float *)(buf + yo), nullptr);
+    if (rc == JITNN_HIP_OK) {
+        e = hipMemcpy(y_host, buf + yo, yb, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(buf);
+    return rc;
+}
+
+int jitnn_hip_quantize_q8_0_dev(const float *x_dev, long long numel, void *blocks_dev, void *stream) {
+    if (!x_dev || !blocks_dev) return fail(JITNN_HIP_EINVAL, "input or output is NULL");
+    if (numel < 0 || numel % 32 != 0) return fail(JITNN_HIP_EINVAL, "Q8_0 needs a multiple of 32 values, got %lld", numel);
+    if (int rc = check_ready()) return rc;
+    if (numel == 0) return JITNN_HIP_OK;
+    const size_t blocks = (size_t)numel / 32;
+    size_t grid = (blocks + 255) / 256;
+    if (grid > (size_t)g.cus * 16) grid = (size_t)g.cus * 16;
+    hipLaunchKernelGGL(quantize_q8_0_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, x_dev, (uint8_t *)blocks_dev, blocks);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_quantize_q8_0(const float *x_host, long long numel, void *blocks_host) {
+    if (!x_host || !blocks_host) return fail(JITNN_HIP_EINVAL, "input or output is NULL");
+    if (numel < 0 || numel % 32 != 0) return fail(JITNN_HIP_EINVAL, "Q8_0 needs a multiple of 32 values, got %lld", numel);
+    if (int rc = check_ready()) return rc;
+    if (numel == 0) return JITNN_HIP_OK;
+    const size_t xb = (size_t)numel * 4, qb = (size_t)numel / 32 * 34;
+    uint8_t *buf = nullptr;
+    hipError_t e = hipMalloc(&buf, xb + qb);
+    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc: %s", hipGetErrorString(e));
+    int rc = JITNN_HIP_OK;
+    e = hipMemcpy(buf, x_host, xb, hipMemcpyHostToDevice);
+    if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    if (rc == JITNN_HIP_OK) rc = jitnn_hip_quantize_q8_0_dev((const float *)buf, numel, buf + xb, nullptr);
+    if (rc == JITNN_HIP_OK) {
+        e = hipMemcpy(blocks_host, buf + xb, qb, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    }
+    (void)hipFree(buf);
+    return rc;
+}
+
+int jitnn_hip_malloc(long long nbytes, void **dev) {
+    if (!dev || nbytes < 0) return fail(JITNN_HIP_EINVAL, "bad arguments");
+    *dev = nullptr;
+    if (int rc = check_ready()) return rc;
+    hipError_t e = hipMalloc(dev, (size_t)(nbytes > 0 ? nbytes : 1));
+    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc of %lld bytes: %s", nbytes, hipGetErrorString(e));
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_free(void *dev) {
+    if (!dev) return JITNN_HIP_OK;
+    HIP_TRY(hipFree(dev));
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_memcpy_h2d(void *dev, const void *host, long long nbytes) {
+    if (!dev || !host || nbytes < 0) return fail(JITNN_HIP_EINVAL, "bad arguments");
+    if (int rc = check_ready()) return rc;
+    HIP_TRY(hipMemcpy(dev, host, (size_t)nbytes, hipMemcpyHostToDevice));
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_memcpy_d2h(void *host, const void *dev, long long nbytes) {
+    if (!dev || !host || nbytes < 0) return fail(JITNN_HIP_EINVAL, "bad arguments");
+    if (int rc = check_ready()) return rc;
+    HIP_TRY(hipMemcpy(host, dev, (size_t)nbytes, hipMemcpyDeviceToHost));
+    return JITNN_HIP_OK;
+}
+
+}  // extern "C"

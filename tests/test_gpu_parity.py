@@ -1,0 +1,187 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle, the reference's golden vectors and its
+GgufChecks recipe.  Bars: dequantised weights bit-exact; GEMV max|y-ref| / max|ref| <= 1e-4 (the
+normalisation of GgufChecks.close, GgufChecks.java:110-120) and the goldens' own rtol 1e-4 / atol 1e-3
+(Golden.java:483-498)."""
+import numpy as np
+import pytest
+
+import ggml_numpy
+from helpers import (GGML_ID, GGML_NAMES, GOLDEN_CODE_TO_GGML, HOT_FORMATS, JavaRandom, checks_close, java_string_hash, norm_err,
+                     random_valid_blocks)
+
+pytestmark = pytest.mark.gpu
+
+GEMV_BAR = 1e-4
+
+
+@pytest.fixture(scope="module")
+def jn():
+    import jitnn_amd
+    jitnn_amd.init()
+    return jitnn_amd
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def weight(jn, fmt, raw, n, k):
+    return jn.Tensor.quantized(jn.DType[fmt], raw, n, k)
+
+
+# ------------------------------------------------------------------------------------------ dequantise
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
+def test_dequant_fixture_bit_exact(jn, gguf_fixture, fmt):
+    """GgufChecks.check 'values' and 'dequantize' (GgufChecks.java:75-80) - here bit for bit."""
+    w = weight(jn, fmt, gguf_fixture.raw(f"w.{fmt}"), 3, 512)
+    expect = gguf_fixture.f32(f"expect.{fmt}").reshape(-1)
+    assert np.array_equal(bits(w.to_float_array()), bits(expect))
+    d = jn.Quant.dequantize(w) if fmt == "Q8_0" else jn.Gguf.dequantize(w)
+    assert np.array_equal(bits(d.numpy().reshape(-1)), bits(expect))
+
+
+@pytest.mark.parametrize("code", [0, 1, 2, 3, 4])
+def test_dequant_goldens_bit_exact(jn, goldens, code):
+    fmt = GGML_NAMES[GOLDEN_CODE_TO_GGML[code]]
+    case = goldens[f"gguf_dequant_{fmt.lower()}"]
+    w = weight(jn, fmt, case.arrays["in0"].astype(np.uint8), 3, 512)
+    assert np.array_equal(bits(w.to_float_array()), bits(case.arrays["out"].reshape(-1)))
+
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
+def test_dequant_random_blocks_vs_oracle(jn, fmt):
+    from oracle import oracle
+    rng = np.random.default_rng(100 + GGML_ID[fmt])
+    n, k = 33, 1024
+    raw = random_valid_blocks(rng, fmt, n, k, lo=1e-6, hi=4.0)  # includes FP16-subnormal scales
+    got = weight(jn, fmt, raw, n, k).to_float_array()
+    assert np.array_equal(bits(got), bits(oracle.dequantize(GGML_ID[fmt], raw, n * k)))
+
+
+# ------------------------------------------------------------------------------------------ linear, reference fixtures
+
+@pytest.mark.parametrize("code", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("rows", [1, 5, 40])
+def test_linear_goldens(jn, goldens, code, rows):
+    fid = GOLDEN_CODE_TO_GGML[code]
+    fmt = GGML_NAMES[fid]
+    case = goldens[f"gguf_linear_{fmt.lower()}_r{rows}"]
+    x, raw, bias, out = case.arrays["in0"], case.arrays["in1"].astype(np.uint8), case.arrays["in2"], case.arrays["out"]
+    n = int(case.attrs[1])
+    y = jn.Gguf.linear(jn.Tensor.of(x), weight(jn, fmt, raw, n, 512), jn.Tensor.of(bias)).numpy()
+    assert y.shape == out.shape
+    assert checks_close(y, out, 1e-4, 1e-3)
+    assert norm_err(y, out) <= GEMV_BAR
+
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
+def test_linear_ggufchecks_recipe(jn, gguf_fixture, fmt):
+    """GgufChecks.check (GgufChecks.java:82-103): 1, 5 and 40 rows from one java.util.Random, bias, 2e-4 * max."""
+    from oracle import oracle
+    raw = gguf_fixture.raw(f"w.{fmt}")
+    expect = gguf_fixture.f32(f"expect.{fmt}").astype(np.float64)
+    w = weight(jn, fmt, raw, 3, 512)
+    rnd = JavaRandom(java_string_hash(fmt))
+    bias = np.array([0.25, -0.5, 1.0], dtype=np.float32)
+    for rows in (1, 5, 40):
+        x = np.array([rnd.next_float() * np.float32(2) - np.float32(1) for _ in range(rows * 512)], dtype=np.float32).reshape(rows, 512)
+        ref = (bias.astype(np.float64)[None, :] + x.astype(np.float64) @ expect.T).astype(np.float32)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias)).numpy()
+        assert norm_err(y, ref) <= 2e-4
+        assert norm_err(y, oracle.gguf_linear(GGML_ID[fmt], x, raw, bias, 3, 512)) <= GEMV_BAR
+
+
+# ------------------------------------------------------------------------------------------ linear, seeded inputs vs oracle
+
+SHAPES = [  # (n, k): ragged row counts, one block, several wave steps, K past one LDS chunk
+    (1, 256), (7, 512), (37, 1024), (64, 4096), (131, 4096), (29, 14336), (5, 8192 + 256),
+]
+
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
+@pytest.mark.parametrize("n,k", SHAPES)
+def test_gemv_vs_oracle(jn, fmt, n, k):
+    from oracle import oracle
+    rng = np.random.default_rng(n * 100003 + k + GGML_ID[fmt])
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    for rows in (1, 2, 3, 4, 8):
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, bias if rows % 2 else None, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias) if rows % 2 else None).numpy()
+        assert y.shape == (rows, n)
+        assert norm_err(y, ref) <= GEMV_BAR, (fmt, n, k, rows, norm_err(y, ref))
+
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
+def test_small_k_32_blocks_and_many_rows(jn, fmt):
+    """K of a single block for the 32-value formats; rows beyond one batch of 8 (9, 17, 40)."""
+    from oracle import oracle
+    rng = np.random.default_rng(77)
+    k = 32 * 3 if fmt in ("Q8_0", "Q4_0", "Q4_1") else 256
+    n = 19
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    for rows in (9, 17, 40):
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, None, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, None).numpy()
+        assert norm_err(y, ref) <= GEMV_BAR, (fmt, rows)
+
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
+def test_unit_vectors_give_columns(jn, fmt):
+    """x = e_j reduces the GEMV to column j of the dequantised matrix: catches any misplaced value."""
+    rng = np.random.default_rng(11)
+    n, k = 9, 1024
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    wd = ggml_numpy.dequant(fmt, raw).reshape(n, k)
+    cols = np.concatenate([np.arange(0, 64), np.arange(250, 262), np.arange(500, 520), np.array([767, 768, 1023])])
+    for c0 in range(0, len(cols), 8):
+        cc = cols[c0:c0 + 8]
+        x = np.zeros((len(cc), k), dtype=np.float32)
+        x[np.arange(len(cc)), cc] = 1.0
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, None).numpy()
+        exp = wd[:, cc].T
+        assert np.allclose(y, exp, rtol=3e-7, atol=1e-9), (fmt, cc)
+
+
+def test_batched_leading_axes(jn):
+    """x [2, 3, K] -> y [2, 3, N] (Gguf.linear keeps the leading axes, Gguf.java:86-93)."""
+    from oracle import oracle
+    rng = np.random.default_rng(5)
+    n, k = 24, 512
+    raw = random_valid_blocks(rng, "Q5_K", n, k)
+    x = rng.standard_normal((2, 3, k)).astype(np.float32)
+    y = jn.Gguf.linear(jn.Tensor.of(x), weight(jn, "Q5_K", raw, n, k), None).numpy()
+    assert y.shape == (2, 3, n)
+    assert norm_err(y.reshape(6, n), oracle.gguf_linear(13, x.reshape(6, k), raw, None, n, k)) <= GEMV_BAR
+
+
+# ------------------------------------------------------------------------------------------ Q8_0 quantiser
+
+def test_quantize_q8_0_bit_exact_vs_oracle(jn):
+    """Same bytes as the oracle's restatement of Quant.Quantize.reference (exact bytes on .5 ties are not pinned by
+    any reference-held vector; both sides share the closed form)."""
+    from oracle import oracle
+    rng = np.random.default_rng(21)
+    x = (rng.standard_normal((64, 256)) * rng.uniform(1e-3, 50, size=(64, 1))).astype(np.float32)
+    x[0, :32] = 0
+    x[1, :32] = np.linspace(-3, 3, 32)
+    x[2, :32] = 1e-7   # scale below the FP16 normal range
+    x[3, :32] = np.arange(32) * 0.5  # exact .5 ties after scaling by a power-of-two-friendly d
+    q = jn.Quant.quantize_q8(jn.Tensor.of(x))
+    assert q.shape() == (64, 256) and q.dtype() == jn.DType.Q8_0
+    exp = oracle.quantize_q8_0(x)
+    got = q.to_float_array()
+    assert np.array_equal(bits(got), bits(oracle.dequantize(8, exp, x.size)))
+    # round trip within one step, the reference's own bar (OpsAccelTest.java:261-267)
+    assert np.abs(got - x.reshape(-1)).max() <= np.abs(x).max() * (1 / 127.0) + 1e-6
+    # and the linear on it agrees with the reference's FP64 host loop
+    xin = rng.standard_normal((3, 256)).astype(np.float32)
+    b = rng.standard_normal(64).astype(np.float32)
+    y = jn.F.linear_q8(jn.Tensor.of(xin), q, jn.Tensor.of(b)).numpy()
+    assert norm_err(y, oracle.gguf_linear(8, xin, exp, b, 64, 256)) <= 1e-5
