@@ -57,6 +57,17 @@ __device__ __forceinline__ float ub1(uint32_t v) { return (float)((v >> 8) & 0xf
 __device__ __forceinline__ float ub2(uint32_t v) { return (float)((v >> 16) & 0xffu); }
 __device__ __forceinline__ float ub3(uint32_t v) { return (float)(v >> 24); }
 
+// Sum over aligned groups of G = 4 or 8 neighbouring lanes (every lane of a group receives the group's total):
+// quad swaps, then for G = 8 the mirror within each half row - DPP moves inside the VALU, no LDS traffic.
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+    static_assert(G == 4 || G == 8, "groups of 4 or 8 lanes");
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+    if constexpr (G == 8) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    return v;
+}
+
 // Sum over the 64 lanes of a wavefront; every lane receives the total.  Four DPP steps fold each row of
 // 16 lanes (quad swaps, then the two mirrors), then the four row totals are read through scalar lanes.
 __device__ __forceinline__ float wave_sum(float v) {

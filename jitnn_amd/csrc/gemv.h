@@ -41,6 +41,23 @@ __device__ __forceinline__ float dot4(float a, float b, float c, float d, const 
     return acc;
 }
 
+// Where a lane finds the activations of its unit: quad g (values 4g..4g+3 in unit order) and partial sum i of
+// batch row b.  XLds reads them from the staged LDS copy; XReg holds them in registers (batch 1).
+struct XLds {
+    const float4 *xu;
+    const float *su;
+    int bs, ss;
+    __device__ __forceinline__ float4 q(int b, int g) const { return xu[b * bs + g]; }
+    __device__ __forceinline__ float s(int b, int i) const { return su[b * ss + i]; }
+};
+template <int UQ, int NS>
+struct XReg {
+    float4 x[UQ];
+    float sm[NS];
+    __device__ __forceinline__ float4 q(int, int g) const { return x[g]; }
+    __device__ __forceinline__ float s(int, int i) const { return sm[i]; }
+};
+
 template <int FMT>
 struct Unit;
 
@@ -52,28 +69,31 @@ template <>
 struct Unit<F_Q4_K> {
     static constexpr int UV = 64, NS = 2, SG = 8;
     struct Raw { u32x4 h, q0, q1; };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *sb = row + (size_t)(u >> 2) * 144;
-        r.h = ld128<16>(sb);
-        r.q0 = ld128<16>(sb + 16 + (u & 3) * 32);
-        r.q1 = ld128<16>(sb + 32 + (u & 3) * 32);
+    static constexpr int NOFF = 2;
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) {
+        o[0] = (uint32_t)(u >> 2) * 144u;
+        o[1] = o[0] + 16u + (uint32_t)(u & 3) * 32u;
+    }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.h = ld128<16>(row + o[0]);
+        r.q0 = ld128<16>(row + o[1]);
+        r.q1 = ld128<16>(row + o[1] + 16);
     }
     __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 4; g = f & 15; }
 
-    // scale and min of sub-blocks 2j and 2j+1 as packed byte pairs
+    // scale and min of sub-blocks 2j and 2j+1 as packed byte pairs (ggml's get_scale_min_k4 on two sub-blocks at
+    // once): for j < 2 the low six bits of scale bytes 2j.. and 4+2j..; for j >= 2 a nibble of bytes 8+2(j-2)..
+    // with the top two bits of bytes 2(j-2).. / 4+2(j-2)..  The three masks select the case without a branch.
     __device__ static __forceinline__ void scale_min(const u32x4 &h, int j, uint32_t &sc2, uint32_t &mn2) {
-        int sh = (j & 1) * 16;
-        uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
-        uint32_t sc_lo = a & 0x3f3fu, mn_lo = b & 0x3f3fu;
-        uint32_t sc_hi = (c & 0x0f0fu) | (((a >> 6) & 0x0303u) << 4);
-        uint32_t mn_hi = ((c >> 4) & 0x0f0fu) | (((b >> 6) & 0x0303u) << 4);
-        sc2 = j < 2 ? sc_lo : sc_hi;
-        mn2 = j < 2 ? mn_lo : mn_hi;
+        const int sh = (j & 1) * 16;
+        const uint32_t m1 = j < 2 ? 0x3f3fu : 0u, m2 = j < 2 ? 0u : 0x0f0fu, m3 = j < 2 ? 0u : 0x3030u;
+        const uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
+        sc2 = (a & m1) | (c & m2) | ((a >> 2) & m3);
+        mn2 = (b & m1) | ((c >> 4) & m2) | ((b >> 2) & m3);
     }
 
-    template <int B, int R, int CV>
-    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const float4 *xu, int bs, const float *su, int ss,
-                                               float (&acc)[R][B], float nib) {
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
         float sl[R][B], sh[R][B];
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -84,8 +104,8 @@ struct Unit<F_Q4_K> {
             float4 xa[B], xb[B];
 #pragma unroll
             for (int b = 0; b < B; ++b) {
-                xa[b] = xu[b * bs + d];
-                xb[b] = xu[b * bs + d + 8];
+                xa[b] = xs.q(b, d);
+                xb[b] = xs.q(b, d + 8);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -110,7 +130,7 @@ struct Unit<F_Q4_K> {
 #pragma unroll
             for (int b = 0; b < B; ++b) {
                 float t = __builtin_fmaf(d0, sl[r][b], d1 * sh[r][b]);
-                float m = __builtin_fmaf(m0, su[b * ss], m1 * su[b * ss + 1]);
+                float m = __builtin_fmaf(m0, xs.s(b, 0), m1 * xs.s(b, 1));
                 acc[r][b] += t - m;
             }
         }
@@ -124,19 +144,22 @@ template <>
 struct Unit<F_Q5_K> {
     static constexpr int UV = 64, NS = 2, SG = 8;
     struct Raw { u32x4 h, qh0, qh1, q0, q1; };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *sb = row + (size_t)(u >> 2) * 176;
-        r.h = ld128<16>(sb);
-        r.qh0 = ld128<16>(sb + 16);
-        r.qh1 = ld128<16>(sb + 32);
-        r.q0 = ld128<16>(sb + 48 + (u & 3) * 32);
-        r.q1 = ld128<16>(sb + 64 + (u & 3) * 32);
+    static constexpr int NOFF = 2;
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) {
+        o[0] = (uint32_t)(u >> 2) * 176u;
+        o[1] = o[0] + 48u + (uint32_t)(u & 3) * 32u;
+    }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.h = ld128<16>(row + o[0]);
+        r.qh0 = ld128<16>(row + o[0] + 16);
+        r.qh1 = ld128<16>(row + o[0] + 32);
+        r.q0 = ld128<16>(row + o[1]);
+        r.q1 = ld128<16>(row + o[1] + 16);
     }
     __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 4; g = f & 15; }
 
-    template <int B, int R, int CV>
-    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const float4 *xu, int bs, const float *su, int ss,
-                                               float (&acc)[R][B], float nib) {
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
         (void)nib;
         const int j2 = (u & 3) * 2;
         float sl[R][B], sh[R][B];
@@ -149,8 +172,8 @@ struct Unit<F_Q5_K> {
             float4 xa[B], xb[B];
 #pragma unroll
             for (int b = 0; b < B; ++b) {
-                xa[b] = xu[b * bs + d];
-                xb[b] = xu[b * bs + d + 8];
+                xa[b] = xs.q(b, d);
+                xb[b] = xs.q(b, d + 8);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -175,7 +198,7 @@ struct Unit<F_Q5_K> {
 #pragma unroll
             for (int b = 0; b < B; ++b) {
                 float t = __builtin_fmaf(d0, sl[r][b], d1 * sh[r][b]);
-                float m = __builtin_fmaf(m0, su[b * ss], m1 * su[b * ss + 1]);
+                float m = __builtin_fmaf(m0, xs.s(b, 0), m1 * xs.s(b, 1));
                 acc[r][b] += t - m;
             }
         }
@@ -192,14 +215,20 @@ template <>
 struct Unit<F_Q6_K> {
     static constexpr int UV = 64, NS = 4, SG = 4;
     struct Raw { u32x4 ql0, ql1, qh; u32x2 sc; uint32_t d; };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *sb = row + (size_t)(u >> 2) * 210;
-        const int n = (u >> 1) & 1, l0 = (u & 1) * 16;
-        r.ql0 = ld128<2>(sb + 64 * n + l0);
-        r.ql1 = ld128<2>(sb + 64 * n + 32 + l0);
-        r.qh = ld128<2>(sb + 128 + 32 * n + l0);
-        r.sc = ld64<2>(sb + 192 + 8 * n);
-        r.d = ld16(sb + 208);
+    static constexpr int NOFF = 4;
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) {
+        const uint32_t sb = (uint32_t)(u >> 2) * 210u, n = (u >> 1) & 1, l0 = (u & 1) * 16;
+        o[0] = sb + 64u * n + l0;  // ql (second half of the nibbles 32 bytes on)
+        o[1] = sb + 32u * n + l0;  // qh, 128 bytes on
+        o[2] = sb + 8u * n;        // scales, 192 bytes on
+        o[3] = sb;                 // d, 208 bytes on
+    }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.ql0 = ld128<2>(row + o[0]);
+        r.ql1 = ld128<2>(row + o[0] + 32);
+        r.qh = ld128<2>(row + o[1] + 128);
+        r.sc = ld64<2>(row + o[2] + 192);
+        r.d = ld16(row + o[3] + 208);
     }
     // x quad f (values 4f..4f+3 of the row) -> unit and quad within the unit (quad 4k + (l%16)/4)
     __device__ static __forceinline__ void slot(int f, int &u, int &g) {
@@ -209,9 +238,8 @@ struct Unit<F_Q6_K> {
         g = 4 * k + ((l & 15) >> 2);
     }
 
-    template <int B, int R, int CV>
-    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const float4 *xu, int bs, const float *su, int ss,
-                                               float (&acc)[R][B], float nib) {
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
         (void)nib;
         float s[R][B][4];
 #pragma unroll
@@ -225,10 +253,10 @@ struct Unit<F_Q6_K> {
             float4 x0[B], x1[B], x2[B], x3[B];
 #pragma unroll
             for (int b = 0; b < B; ++b) {
-                x0[b] = xu[b * bs + p];
-                x1[b] = xu[b * bs + 4 + p];
-                x2[b] = xu[b * bs + 8 + p];
-                x3[b] = xu[b * bs + 12 + p];
+                x0[b] = xs.q(b, p);
+                x1[b] = xs.q(b, 4 + p);
+                x2[b] = xs.q(b, 8 + p);
+                x3[b] = xs.q(b, 12 + p);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -256,11 +284,10 @@ struct Unit<F_Q6_K> {
             float c3 = (float)(int)(int8_t)(w[r].sc.y >> (sh + 16));
 #pragma unroll
             for (int b = 0; b < B; ++b) {
-                const float *sb = su + b * ss;
-                float t = c0 * __builtin_fmaf(-32.f, sb[0], s[r][b][0]);
-                t = __builtin_fmaf(c1, __builtin_fmaf(-32.f, sb[1], s[r][b][1]), t);
-                t = __builtin_fmaf(c2, __builtin_fmaf(-32.f, sb[2], s[r][b][2]), t);
-                t = __builtin_fmaf(c3, __builtin_fmaf(-32.f, sb[3], s[r][b][3]), t);
+                float t = c0 * __builtin_fmaf(-32.f, xs.s(b, 0), s[r][b][0]);
+                t = __builtin_fmaf(c1, __builtin_fmaf(-32.f, xs.s(b, 1), s[r][b][1]), t);
+                t = __builtin_fmaf(c2, __builtin_fmaf(-32.f, xs.s(b, 2), s[r][b][2]), t);
+                t = __builtin_fmaf(c3, __builtin_fmaf(-32.f, xs.s(b, 3), s[r][b][3]), t);
                 acc[r][b] = __builtin_fmaf(d, t, acc[r][b]);
             }
         }
@@ -274,16 +301,16 @@ template <>
 struct Unit<F_Q4_0> {
     static constexpr int UV = 32, NS = 1, SG = 8;
     struct Raw { u32x4 q; uint32_t d; };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *b = row + (size_t)u * 18;
-        r.d = ld16(b);
-        r.q = ld128<2>(b + 2);
+    static constexpr int NOFF = 1;
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) { o[0] = (uint32_t)u * 18u; }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.d = ld16(row + o[0]);
+        r.q = ld128<2>(row + o[0] + 2);
     }
     __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 3; g = f & 7; }
 
-    template <int B, int R, int CV>
-    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const float4 *xu, int bs, const float *su, int ss,
-                                               float (&acc)[R][B], float nib) {
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
         (void)u;
         float s[R][B];
 #pragma unroll
@@ -295,8 +322,8 @@ struct Unit<F_Q4_0> {
             float4 xa[B], xb[B];
 #pragma unroll
             for (int b = 0; b < B; ++b) {
-                xa[b] = xu[b * bs + p];
-                xb[b] = xu[b * bs + p + 4];
+                xa[b] = xs.q(b, p);
+                xb[b] = xs.q(b, p + 4);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -316,7 +343,7 @@ struct Unit<F_Q4_0> {
             float d = h2f(w[r].d);
 #pragma unroll
             for (int b = 0; b < B; ++b)
-                acc[r][b] = __builtin_fmaf(d, __builtin_fmaf(nib, s[r][b], -8.f * su[b * ss]), acc[r][b]);
+                acc[r][b] = __builtin_fmaf(d, __builtin_fmaf(nib, s[r][b], -8.f * xs.s(b, 0)), acc[r][b]);
         }
     }
 };
@@ -328,16 +355,16 @@ template <>
 struct Unit<F_Q4_1> {
     static constexpr int UV = 32, NS = 1, SG = 8;
     struct Raw { u32x4 q; uint32_t dm; };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *b = row + (size_t)u * 20;
-        r.dm = ld32<4>(b);
-        r.q = ld128<4>(b + 4);
+    static constexpr int NOFF = 1;
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) { o[0] = (uint32_t)u * 20u; }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.dm = ld32<4>(row + o[0]);
+        r.q = ld128<4>(row + o[0] + 4);
     }
     __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 3; g = f & 7; }
 
-    template <int B, int R, int CV>
-    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const float4 *xu, int bs, const float *su, int ss,
-                                               float (&acc)[R][B], float nib) {
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
         (void)u;
         float s[R][B];
 #pragma unroll
@@ -349,8 +376,8 @@ struct Unit<F_Q4_1> {
             float4 xa[B], xb[B];
 #pragma unroll
             for (int b = 0; b < B; ++b) {
-                xa[b] = xu[b * bs + p];
-                xb[b] = xu[b * bs + p + 4];
+                xa[b] = xs.q(b, p);
+                xb[b] = xs.q(b, p + 4);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -369,7 +396,7 @@ struct Unit<F_Q4_1> {
         for (int r = 0; r < R; ++r) {
             float d = h2f(w[r].dm) * nib, m = h2f(w[r].dm >> 16);
 #pragma unroll
-            for (int b = 0; b < B; ++b) acc[r][b] += __builtin_fmaf(d, s[r][b], m * su[b * ss]);
+            for (int b = 0; b < B; ++b) acc[r][b] += __builtin_fmaf(d, s[r][b], m * xs.s(b, 0));
         }
     }
 };
@@ -382,17 +409,17 @@ template <>
 struct Unit<F_Q8_0> {
     static constexpr int UV = 32, NS = 1, SG = 8;
     struct Raw { u32x4 q0, q1; uint32_t d; };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, int u) {
-        const uint8_t *b = row + (size_t)u * 34;
-        r.d = ld16(b);
-        r.q0 = ld128<2>(b + 2);
-        r.q1 = ld128<2>(b + 18);
+    static constexpr int NOFF = 1;
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) { o[0] = (uint32_t)u * 34u; }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.d = ld16(row + o[0]);
+        r.q0 = ld128<2>(row + o[0] + 2);
+        r.q1 = ld128<2>(row + o[0] + 18);
     }
     __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 3; g = f & 7; }
 
-    template <int B, int R, int CV>
-    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const float4 *xu, int bs, const float *su, int ss,
-                                               float (&acc)[R][B], float nib) {
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
         (void)u;
         (void)nib;
         float s[R][B];
@@ -404,7 +431,7 @@ struct Unit<F_Q8_0> {
         for (int p = 0; p < 8; ++p) {
             float4 xa[B];
 #pragma unroll
-            for (int b = 0; b < B; ++b) xa[b] = xu[b * bs + p];
+            for (int b = 0; b < B; ++b) xa[b] = xs.q(b, p);
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 uint32_t v = (p < 4 ? w[r].q0[p & 3] : w[r].q1[p & 3]) ^ 0x80808080u;
@@ -416,10 +443,118 @@ struct Unit<F_Q8_0> {
         for (int r = 0; r < R; ++r) {
             float d = h2f(w[r].d);
 #pragma unroll
-            for (int b = 0; b < B; ++b) acc[r][b] = __builtin_fmaf(d, __builtin_fmaf(-128.f, su[b * ss], s[r][b]), acc[r][b]);
+            for (int b = 0; b < B; ++b) acc[r][b] = __builtin_fmaf(d, __builtin_fmaf(-128.f, xs.s(b, 0), s[r][b]), acc[r][b]);
         }
     }
 };
+
+// Batch-1 GEMV for rows of at most 4096 values: the activations live in registers.
+//
+// The vector is staged through LDS once per workgroup (coalesced global read, unit-order write), each lane
+// then pulls the 64 floats of its own units (STEPS units of UV values, STEPS * UV = 64) and their partial
+// sums into VGPRs and never touches LDS again.  Every wave walks the rows gw, gw + W, gw + 2W, ... (W = waves
+// in the grid), one row per iteration, through a ring of PF + 1 register buffers: while one row is decoded
+// the loads of the next PF rows are in flight, and a buffer is refilled as soon as its row is done.  The
+// loads are unconditional (rows past the end re-read the last row) so that the hardware's in-order load
+// counter can be waited on exactly; only the decode and the store are skipped for rows that do not exist.
+// The first rows' loads are issued before the staging barrier, so HBM latency overlaps the staging too.
+constexpr int XREG_THREADS = 256;  // workgroup size of gemv_xreg_kernel (compile-time: the staging is fully unrolled)
+
+template <int FMT, int STEPS, int CV, int PF, bool BIAS>
+__global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
+                                                         const float *__restrict__ bias, float *__restrict__ y, int n, int k, float nib) {
+    using U = Unit<FMT>;
+    constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG, NB = PF + 1;
+    static_assert(STEPS * U::UV == 64, "a lane keeps 64 activations");
+    __shared__ float4 xl[STEPS * 64 * (UQ + 1)];
+    __shared__ float sums[STEPS * 64 * NS];
+    constexpr int nwaves = XREG_THREADS / 64;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: row numbers, row pointers and the loop run on the SALU
+    const int units = k / U::UV;
+    const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
+    const int stride = gridDim.x * nwaves;
+    const int row0 = blockIdx.x * nwaves + wave;
+    int uc[STEPS];
+    uint32_t off[STEPS][U::NOFF];  // byte offsets of this lane's fields within a row: the same for every row
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        uc[s] = min(s * 64 + lane, units - 1);  // lanes past the row end: last unit, zeroed x
+        U::offsets(uc[s], off[s]);
+    }
+    // loads of buffer b for row r; a row past the end is "loaded" from the first bytes of the matrix by every lane
+    // (one cache line, no traffic) so that the number of loads in flight never depends on the data
+    auto fill = [&](typename U::Raw(&dst)[STEPS], float &bdst, int r) {
+        const bool live = r < n;
+        const uint8_t *rp = W + (live ? (size_t)r * rowbytes : 0);
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            uint32_t o[U::NOFF];
+#pragma unroll
+            for (int i = 0; i < U::NOFF; ++i) o[i] = live ? off[s][i] : 0u;
+            U::load(dst[s], rp, o);
+        }
+        if (BIAS) bdst = bias[live ? r : 0];
+    };
+
+    // ---- activations first: their loads (L2 hits) are issued ahead of the weight loads because the hardware counts
+    // returning loads in order - waiting for x must not mean waiting for the first weight rows from HBM
+    constexpr int QUADS = STEPS * 64 * UQ, PER = QUADS / XREG_THREADS;
+    static_assert(QUADS % XREG_THREADS == 0, "whole passes");
+    float4 xv[PER];
+    {
+        const int kq = k >> 2;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int f = tid + i * XREG_THREADS;
+            xv[i] = f < kq ? reinterpret_cast<const float4 *>(x)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    typename U::Raw buf[NB][STEPS];
+    float bv[NB];  // the bias of each buffered row rides with its loads, so waiting for it never drains younger loads
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        bv[b] = 0.f;
+        fill(buf[b], bv[b], row0 + b * stride);
+    }
+    // ---- stage x (and the partial sums) in unit order
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int f = tid + i * XREG_THREADS;
+        int u, g;
+        U::slot(f, u, g);
+        xl[u * (UQ + 1) + g] = xv[i];
+        const float sm = group_sum<SG>((xv[i].x + xv[i].y) + (xv[i].z + xv[i].w));
+        if ((f & (SG - 1)) == 0) sums[u * NS + g / SG] = sm;
+    }
+    __syncthreads();
+    XReg<UQ, NS> xs[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+        for (int g = 0; g < UQ; ++g) xs[s].x[g] = xl[(s * 64 + lane) * (UQ + 1) + g];
+#pragma unroll
+        for (int i = 0; i < NS; ++i) xs[s].sm[i] = sums[(s * 64 + lane) * NS + i];
+    }
+
+    for (int base = row0; base < n; base += NB * stride) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int row = base + b * stride;
+            if (row < n) {  // wave-uniform
+                float acc[1][1] = {{0.f}};
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    const typename U::Raw(&w1)[1] = reinterpret_cast<const typename U::Raw(&)[1]>(buf[b][s]);
+                    U::template dot<1, 1, CV>(w1, uc[s], xs[s], acc, nib);
+                }
+                float t = wave_sum(acc[0][0]);
+                if (lane == 0) y[row] = BIAS ? t + bv[b] : t;
+            }
+            fill(buf[b], bv[b], row + NB * stride);
+        }
+    }
+}
 
 // LDS bytes one staged K-chunk of `itc` wave steps takes for batch B.
 template <int FMT>
@@ -462,9 +597,7 @@ __global__ void __launch_bounds__(512) gemv_lds_kernel(const uint8_t *__restrict
                 U::slot(f, u, g);
                 u -= c0 * 64;
                 xl[(size_t)b * bs + (size_t)u * (UQ + 1) + g] = v;
-                float s = (v.x + v.y) + (v.z + v.w);
-#pragma unroll
-                for (int m = 1; m < SG; m <<= 1) s += __shfl_xor(s, m);
+                const float s = group_sum<SG>((v.x + v.y) + (v.z + v.w));
                 if ((f & (SG - 1)) == 0) sums[(size_t)b * ss + u * NS + g / SG] = s;
             }
         }
@@ -480,9 +613,12 @@ __global__ void __launch_bounds__(512) gemv_lds_kernel(const uint8_t *__restrict
                 const int u = (c0 + it) * 64 + lane;
                 const int uc = min(u, units - 1);  // lanes past the row end re-read the last unit against zeroed x
                 typename U::Raw w[R];
+                uint32_t off[U::NOFF];
+                U::offsets(uc, off);
 #pragma unroll
-                for (int r = 0; r < R; ++r) U::load(w[r], W + (size_t)min(rg * R + r, n - 1) * rowbytes, uc);
-                U::template dot<B, R, CV>(w, uc, xl + (size_t)(it * 64 + lane) * (UQ + 1), bs, sums + (it * 64 + lane) * NS, ss, acc, nib);
+                for (int r = 0; r < R; ++r) U::load(w[r], W + (size_t)min(rg * R + r, n - 1) * rowbytes, off);
+                const XLds xs{xl + (size_t)(it * 64 + lane) * (UQ + 1), sums + (it * 64 + lane) * NS, bs, ss};
+                U::template dot<B, R, CV>(w, uc, xs, acc, nib);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {

@@ -7,6 +7,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -50,6 +51,9 @@ struct State {
     char name[256] = "";
     float nib = 0.f;  // 1 / (value of E4M3 byte 0x01): 512 for OCP, 1024 for FNUZ
     size_t max_lds = 0;
+    int xreg_blocks_per_cu = 0;  // JITNN_HIP_XREG_BLOCKS: override of the workgroups per CU (0 = built-in choice)
+    int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1..3 (0 = built-in choice)
+    bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
 };
 State g;
 std::mutex g_mu;
@@ -105,7 +109,46 @@ GemvVariant pick(int fmt, int rows) {
 
 int unit_values(int fmt) { return block_values(fmt) == 256 ? 64 : 32; }
 
+typedef void (*gemv1_fn)(const uint8_t *, const float *, const float *, float *, int, int, float);
+
+template <int PF, bool BIAS>
+gemv1_fn pick_xreg_pf(int fmt) {
+    switch (fmt) {
+    case F_Q4_0: return gemv_xreg_kernel<F_Q4_0, 2, 1, PF, BIAS>;
+    case F_Q4_1: return gemv_xreg_kernel<F_Q4_1, 2, 1, PF, BIAS>;
+    case F_Q8_0: return gemv_xreg_kernel<F_Q8_0, 2, 0, PF, BIAS>;
+    case F_Q4_K: return gemv_xreg_kernel<F_Q4_K, 1, 1, PF, BIAS>;
+    case F_Q5_K: return gemv_xreg_kernel<F_Q5_K, 1, 0, PF, BIAS>;
+    default: return gemv_xreg_kernel<F_Q6_K, 1, 0, PF, BIAS>;
+    }
+}
+
+gemv1_fn pick_xreg(int fmt, bool bias, int pf) {
+    switch (pf) {
+    case 1: return bias ? pick_xreg_pf<1, true>(fmt) : pick_xreg_pf<1, false>(fmt);
+    case 3: return bias ? pick_xreg_pf<3, true>(fmt) : pick_xreg_pf<3, false>(fmt);
+    default: return bias ? pick_xreg_pf<2, true>(fmt) : pick_xreg_pf<2, false>(fmt);
+    }
+}
+
+// Batch 1, rows of at most 4096 values: activations in registers, one row per wave iteration.
+int launch_gemv_xreg(const jitnn_hip_weight *w, const float *x, const float *bias, float *y, hipStream_t stream) {
+    const int threads = XREG_THREADS, waves = threads / 64;
+    int blocks = (w->n + waves - 1) / waves;
+    // Two workgroups (eight waves) per CU measured best for streaming: fewer, longer row streams keep HBM pages
+    // open.  A wave that sees many rows needs one row of prefetch; when it sees only a handful (a 14336-row
+    // matrix gives a wave seven rows) a second row in flight covers the start-up latency.
+    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : 2);
+    if (blocks > cap) blocks = cap;
+    const int rows_per_wave = (w->n + blocks * waves - 1) / (blocks * waves);
+    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
+    hipLaunchKernelGGL(pick_xreg(w->fmt, bias != nullptr, pf), dim3(blocks), dim3(threads), 0, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    if (rows == 1 && w->k <= 4096 && !g.force_lds) return launch_gemv_xreg(w, x, bias, y, stream);
     GemvVariant v = pick(w->fmt, rows);
     const int units = w->k / unit_values(w->fmt);
     const int steps = (units + 63) / 64;
@@ -200,6 +243,15 @@ int jitnn_hip_init(int device_ordinal) {
     if (!(h[0] > 0.f) || h[1] != 15.f * h[0])
         return fail(JITNN_HIP_EDEVICE, "fp8 probe: E4M3 bytes 0x01, 0x0f decode to %g, %g; expected q * 2^-9 or q * 2^-10", h[0], h[1]);
     g.nib = 1.f / h[0];
+    if (const char *e = getenv("JITNN_HIP_XREG_BLOCKS")) {
+        int v = atoi(e);
+        if (v >= 1 && v <= 32) g.xreg_blocks_per_cu = v;
+    }
+    if (const char *e = getenv("JITNN_HIP_XREG_PF")) {
+        int v = atoi(e);
+        if (v >= 1 && v <= 3) g.xreg_pf = v;
+    }
+    if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     g.device = device_ordinal;
     g.ready = true;
     return JITNN_HIP_OK;
