@@ -556,6 +556,131 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *
     }
 }
 
+// Batch-1 GEMV for rows longer than 4096 values: the row is cut into slices of 4096 values, one per wave of
+// the workgroup (a 14336-value row takes four waves, the last one half full), and each wave keeps the
+// activations of its slice in registers exactly as gemv_xreg_kernel does.  All waves of a workgroup walk the
+// same rows (blockIdx.x, + gridDim.x, ...) with the same prefetch ring; each leaves its partial sum of a row in
+// LDS, and every KS_FLUSH rows (and at the end) the workgroup meets at a barrier where one thread per row adds
+// the slices in slice order and writes y: a fixed summation order, no atomics.
+//   launch: blockDim.x = 64 * slices, dynamic LDS = gemv_ksplit_lds_bytes<FMT>(slices).
+constexpr int KS_FLUSH = 32;
+
+template <int FMT>
+__host__ __device__ constexpr size_t gemv_ksplit_lds_bytes(int slices) {
+    constexpr int STEPS = 64 / Unit<FMT>::UV;
+    return (size_t)slices * STEPS * 64 * ((Unit<FMT>::UV / 4 + 1) * 16 + Unit<FMT>::NS * 4);
+}
+
+template <int FMT, int STEPS, int CV, int PF>
+__global__ void __launch_bounds__(512) gemv_ksplit_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
+                                                            const float *__restrict__ bias, float *__restrict__ y, int n, int k, float nib) {
+    using U = Unit<FMT>;
+    constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG, NB = PF + 1;
+    static_assert(STEPS * U::UV == 64, "a lane keeps 64 activations");
+    extern __shared__ float4 smem[];
+    __shared__ float part[KS_FLUSH][8];  // at most 8 slices: rows of up to 32768 values
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slices = blockDim.x >> 6;
+    float4 *xl = smem + (size_t)wave * STEPS * 64 * (UQ + 1);
+    float *sums = reinterpret_cast<float *>(smem + (size_t)slices * STEPS * 64 * (UQ + 1)) + (size_t)wave * STEPS * 64 * NS;
+    const int units = k / U::UV;
+    const int ubase = wave * STEPS * 64;  // first unit of this wave's slice
+    const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
+    const int stride = gridDim.x;
+    const int row0 = blockIdx.x;
+    int uc[STEPS];
+    uint32_t off[STEPS][U::NOFF];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        uc[s] = min(ubase + s * 64 + lane, units - 1);  // lanes past the row end: last unit, zeroed x
+        U::offsets(uc[s], off[s]);
+    }
+    auto fill = [&](typename U::Raw(&dst)[STEPS], int r) {
+        const bool live = r < n;
+        const uint8_t *rp = W + (live ? (size_t)r * rowbytes : 0);
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            uint32_t o[U::NOFF];
+#pragma unroll
+            for (int i = 0; i < U::NOFF; ++i) o[i] = live ? off[s][i] : 0u;
+            U::load(dst[s], rp, o);
+        }
+    };
+
+    // ---- each wave stages its own slice of x: 16 quads per lane, issued ahead of the weight loads
+    constexpr int PER = STEPS * UQ;  // quads per lane
+    float4 xv[PER];
+    {
+        const int kq = k >> 2, fbase = ubase * UQ;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int f = fbase + i * 64 + lane;
+            xv[i] = f < kq ? reinterpret_cast<const float4 *>(x)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    typename U::Raw buf[NB][STEPS];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) fill(buf[b], row0 + b * stride);
+    {
+        const int fbase = ubase * UQ;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int f = fbase + i * 64 + lane;
+            int u, g;
+            U::slot(f, u, g);
+            u -= ubase;
+            xl[u * (UQ + 1) + g] = xv[i];
+            const float sm = group_sum<SG>((xv[i].x + xv[i].y) + (xv[i].z + xv[i].w));
+            if ((f & (SG - 1)) == 0) sums[u * NS + g / SG] = sm;
+        }
+    }
+    __syncthreads();
+    XReg<UQ, NS> xs[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+#pragma unroll
+        for (int g = 0; g < UQ; ++g) xs[s].x[g] = xl[(s * 64 + lane) * (UQ + 1) + g];
+#pragma unroll
+        for (int i = 0; i < NS; ++i) xs[s].sm[i] = sums[(s * 64 + lane) * NS + i];
+    }
+
+    int done = 0;       // rows of this workgroup finished so far
+    int flushed = 0;    // ... of which already written to y
+    auto flush = [&]() {
+        __syncthreads();
+        const int cnt = done - flushed;
+        if (tid < cnt) {
+            const int row = row0 + (flushed + tid) * stride;
+            float t = 0.f;
+            for (int w = 0; w < slices; ++w) t += part[tid][w];
+            y[row] = bias ? t + bias[row] : t;
+        }
+        __syncthreads();
+        flushed = done;
+    };
+    for (int base = row0; base < n; base += NB * stride) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int row = base + b * stride;
+            if (row < n) {  // workgroup-uniform
+                float acc[1][1] = {{0.f}};
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    const typename U::Raw(&w1)[1] = reinterpret_cast<const typename U::Raw(&)[1]>(buf[b][s]);
+                    U::template dot<1, 1, CV>(w1, uc[s], xs[s], acc, nib);
+                }
+                float t = wave_sum(acc[0][0]);
+                if (lane == 0) part[done - flushed][wave] = t;
+                ++done;
+                if (done - flushed == KS_FLUSH) flush();
+            }
+            fill(buf[b], row + NB * stride);
+        }
+    }
+    if (done > flushed) flush();
+}
+
 // LDS bytes one staged K-chunk of `itc` wave steps takes for batch B.
 template <int FMT>
 __host__ __device__ constexpr size_t gemv_lds_bytes(int B, int itc) {

@@ -50,7 +50,8 @@ struct State {
     long long hbm = 0;
     char name[256] = "";
     float nib = 0.f;  // 1 / (value of E4M3 byte 0x01): 512 for OCP, 1024 for FNUZ
-    size_t max_lds = 0;
+    size_t max_lds = 0;      // LDS one workgroup may ask for
+    size_t lds_per_cu = 0;   // LDS of a compute unit
     int xreg_blocks_per_cu = 0;  // JITNN_HIP_XREG_BLOCKS: override of the workgroups per CU (0 = built-in choice)
     int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1..3 (0 = built-in choice)
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
@@ -147,8 +148,53 @@ int launch_gemv_xreg(const jitnn_hip_weight *w, const float *x, const float *bia
     return JITNN_HIP_OK;
 }
 
+template <int PF>
+gemv1_fn pick_ksplit_pf(int fmt) {
+    switch (fmt) {
+    case F_Q4_0: return gemv_ksplit_kernel<F_Q4_0, 2, 1, PF>;
+    case F_Q4_1: return gemv_ksplit_kernel<F_Q4_1, 2, 1, PF>;
+    case F_Q8_0: return gemv_ksplit_kernel<F_Q8_0, 2, 0, PF>;
+    case F_Q4_K: return gemv_ksplit_kernel<F_Q4_K, 1, 1, PF>;
+    case F_Q5_K: return gemv_ksplit_kernel<F_Q5_K, 1, 0, PF>;
+    default: return gemv_ksplit_kernel<F_Q6_K, 1, 0, PF>;
+    }
+}
+
+size_t ksplit_lds(int fmt, int slices) {
+    switch (fmt) {
+    case F_Q4_0: return gemv_ksplit_lds_bytes<F_Q4_0>(slices);
+    case F_Q4_1: return gemv_ksplit_lds_bytes<F_Q4_1>(slices);
+    case F_Q8_0: return gemv_ksplit_lds_bytes<F_Q8_0>(slices);
+    case F_Q4_K: return gemv_ksplit_lds_bytes<F_Q4_K>(slices);
+    case F_Q5_K: return gemv_ksplit_lds_bytes<F_Q5_K>(slices);
+    default: return gemv_ksplit_lds_bytes<F_Q6_K>(slices);
+    }
+}
+
+// Batch 1, rows of 4097..32768 values: one wave per 4096-value slice of the row, partial sums joined in LDS.
+int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *bias, float *y, hipStream_t stream) {
+    const int slices = (w->k + 4095) / 4096;
+    const size_t lds = ksplit_lds(w->fmt, slices);
+    int per_cu = (int)((g.lds_per_cu - 4096) / lds);  // workgroups of one CU by LDS
+    if (per_cu < 1) per_cu = 1;
+    const int waves_cap = 16 / slices > 0 ? 16 / slices : 1;  // at most 16 waves (4 per SIMD: the kernels use ~128 VGPRs)
+    if (per_cu > waves_cap) per_cu = waves_cap;
+    if (g.xreg_blocks_per_cu > 0 && per_cu > g.xreg_blocks_per_cu) per_cu = g.xreg_blocks_per_cu;
+    int blocks = w->n < g.cus * per_cu ? w->n : g.cus * per_cu;
+    const int rows_per_block = (w->n + blocks - 1) / blocks;
+    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_block >= 16 ? 1 : 2);
+    gemv1_fn fn = pf == 1 ? pick_ksplit_pf<1>(w->fmt) : pf == 3 ? pick_ksplit_pf<3>(w->fmt) : pick_ksplit_pf<2>(w->fmt);
+    if (lds > 65536) HIP_TRY(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(fn, dim3(blocks), dim3(64 * slices), lds, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
-    if (rows == 1 && w->k <= 4096 && !g.force_lds) return launch_gemv_xreg(w, x, bias, y, stream);
+    if (rows == 1 && !g.force_lds) {
+        if (w->k <= 4096) return launch_gemv_xreg(w, x, bias, y, stream);
+        if (w->k <= 32768 && ksplit_lds(w->fmt, (w->k + 4095) / 4096) <= g.max_lds) return launch_gemv_ksplit(w, x, bias, y, stream);
+    }
     GemvVariant v = pick(w->fmt, rows);
     const int units = w->k / unit_values(w->fmt);
     const int steps = (units + 63) / 64;
@@ -233,6 +279,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (hipDeviceGetAttribute(&optin, hipDeviceAttributeSharedMemPerBlockOptin, device_ordinal) != hipSuccess || optin <= 0)
         optin = (int)p.sharedMemPerBlock;
     g.max_lds = (size_t)optin;
+    g.lds_per_cu = p.maxSharedMemoryPerMultiProcessor > 0 ? (size_t)p.maxSharedMemoryPerMultiProcessor : g.max_lds;
     float *probe = nullptr;
     HIP_TRY(hipMalloc(&probe, 2 * sizeof(float)));
     hipLaunchKernelGGL(fp8_probe_kernel, dim3(1), dim3(1), 0, 0, probe);
