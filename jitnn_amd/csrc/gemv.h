@@ -67,6 +67,7 @@ struct Unit;
 // (reference: core/kernels/GgufKernels.java:101-111, 6-bit scale/min unpack :74-83).
 template <>
 struct Unit<F_Q4_K> {
+    static constexpr int FMT = F_Q4_K;
     static constexpr int UV = 64, NS = 2, SG = 8;
     struct Raw { u32x4 h, q0, q1; };
     static constexpr int NOFF = 2;
@@ -142,6 +143,7 @@ struct Unit<F_Q4_K> {
 // (2j + half) of qh[e%32] as the fifth bit (reference: core/kernels/GgufKernels.java:113-125).
 template <>
 struct Unit<F_Q5_K> {
+    static constexpr int FMT = F_Q5_K;
     static constexpr int UV = 64, NS = 2, SG = 8;
     struct Raw { u32x4 h, qh0, qh1, q0, q1; };
     static constexpr int NOFF = 2;
@@ -213,6 +215,7 @@ struct Unit<F_Q5_K> {
 // Unit u = 4*sb + 2*n + l0/16 covers l in [l0, l0+16) for the four k: 64 values in four runs of 16.
 template <>
 struct Unit<F_Q6_K> {
+    static constexpr int FMT = F_Q6_K;
     static constexpr int UV = 64, NS = 4, SG = 4;
     struct Raw { u32x4 ql0, ql1, qh; u32x2 sc; uint32_t d; };
     static constexpr int NOFF = 4;
@@ -299,6 +302,7 @@ struct Unit<F_Q6_K> {
 // nibble of qs[e-16] otherwise (reference: core/kernels/GgufKernels.java:85-91).
 template <>
 struct Unit<F_Q4_0> {
+    static constexpr int FMT = F_Q4_0;
     static constexpr int UV = 32, NS = 1, SG = 8;
     struct Raw { u32x4 q; uint32_t d; };
     static constexpr int NOFF = 1;
@@ -353,6 +357,7 @@ struct Unit<F_Q4_0> {
 // core/kernels/GgufKernels.java:93-99).
 template <>
 struct Unit<F_Q4_1> {
+    static constexpr int FMT = F_Q4_1;
     static constexpr int UV = 32, NS = 1, SG = 8;
     struct Raw { u32x4 q; uint32_t dm; };
     static constexpr int NOFF = 1;
@@ -407,6 +412,7 @@ struct Unit<F_Q4_1> {
 // comes back out through the block sum of x.
 template <>
 struct Unit<F_Q8_0> {
+    static constexpr int FMT = F_Q8_0;
     static constexpr int UV = 32, NS = 1, SG = 8;
     struct Raw { u32x4 q0, q1; uint32_t d; };
     static constexpr int NOFF = 1;
@@ -448,6 +454,167 @@ struct Unit<F_Q8_0> {
     }
 };
 
+// ------------------------------------------------------------------------------------- pairs of 32-value blocks
+// For rows whose block count is even, the 32-value formats are decoded two blocks per lane: a pair of blocks
+// starts on a 4-byte boundary (36, 40 and 68 bytes), so the lane fetches it with aligned 128-bit loads and
+// realigns the half-word-shifted quants of the first block with v_alignbit instead of issuing loads that
+// straddle dwords.  The unit is 64 values like the k-quants': one wave step per 4096 values.
+template <int FMT>
+struct UnitPair;
+
+// two block_q4_0: bytes 0-1 d0, 2-17 qs0, 18-19 d1, 20-35 qs1
+template <>
+struct UnitPair<F_Q4_0> {
+    static constexpr int FMT = F_Q4_0;
+    static constexpr int UV = 64, NS = 2, SG = 8, NOFF = 1;
+    struct Raw { u32x4 a, b; uint32_t c; };
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) { o[0] = (uint32_t)u * 36u; }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.a = ld128<4>(row + o[0]);
+        r.b = ld128<4>(row + o[0] + 16);
+        r.c = ld32<4>(row + o[0] + 32);
+    }
+    __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 4; g = f & 15; }
+
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
+        (void)u;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t q0[4] = {__builtin_amdgcn_alignbit(w[r].a.y, w[r].a.x, 16), __builtin_amdgcn_alignbit(w[r].a.z, w[r].a.y, 16),
+                                    __builtin_amdgcn_alignbit(w[r].a.w, w[r].a.z, 16), __builtin_amdgcn_alignbit(w[r].b.x, w[r].a.w, 16)};
+            const uint32_t q1[4] = {w[r].b.y, w[r].b.z, w[r].b.w, w[r].c};
+            float s0[B], s1[B];
+#pragma unroll
+            for (int b = 0; b < B; ++b) s0[b] = s1[b] = 0.f;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                float l0, l1, l2, l3, h0, h1, h2, h3;
+                cvt4<CV>(q0[p] & 0x0f0f0f0fu, l0, l1, l2, l3);
+                cvt4<CV>((q0[p] >> 4) & 0x0f0f0f0fu, h0, h1, h2, h3);
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    s0[b] = dot4(l0, l1, l2, l3, xs.q(b, p), s0[b]);
+                    s0[b] = dot4(h0, h1, h2, h3, xs.q(b, p + 4), s0[b]);
+                }
+                cvt4<CV>(q1[p] & 0x0f0f0f0fu, l0, l1, l2, l3);
+                cvt4<CV>((q1[p] >> 4) & 0x0f0f0f0fu, h0, h1, h2, h3);
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    s1[b] = dot4(l0, l1, l2, l3, xs.q(b, 8 + p), s1[b]);
+                    s1[b] = dot4(h0, h1, h2, h3, xs.q(b, 12 + p), s1[b]);
+                }
+            }
+            const float d0 = h2f(w[r].a.x), d1 = h2f(w[r].b.x >> 16);
+#pragma unroll
+            for (int b = 0; b < B; ++b) {
+                float t = d0 * __builtin_fmaf(nib, s0[b], -8.f * xs.s(b, 0));
+                acc[r][b] += __builtin_fmaf(d1, __builtin_fmaf(nib, s1[b], -8.f * xs.s(b, 1)), t);
+            }
+        }
+    }
+};
+
+// two block_q4_1: bytes 0-3 d0 m0, 4-19 qs0, 20-23 d1 m1, 24-39 qs1
+template <>
+struct UnitPair<F_Q4_1> {
+    static constexpr int FMT = F_Q4_1;
+    static constexpr int UV = 64, NS = 2, SG = 8, NOFF = 1;
+    struct Raw { u32x4 a, b; u32x2 c; };
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) { o[0] = (uint32_t)u * 40u; }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.a = ld128<4>(row + o[0]);
+        r.b = ld128<4>(row + o[0] + 16);
+        r.c = *reinterpret_cast<const u32x2 *>(row + o[0] + 32);  // 40u + 32 is a multiple of 8
+    }
+    __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 4; g = f & 15; }
+
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
+        (void)u;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t q0[4] = {w[r].a.y, w[r].a.z, w[r].a.w, w[r].b.x};
+            const uint32_t q1[4] = {w[r].b.z, w[r].b.w, w[r].c.x, w[r].c.y};
+            float s0[B], s1[B];
+#pragma unroll
+            for (int b = 0; b < B; ++b) s0[b] = s1[b] = 0.f;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                float l0, l1, l2, l3, h0, h1, h2, h3;
+                cvt4<CV>(q0[p] & 0x0f0f0f0fu, l0, l1, l2, l3);
+                cvt4<CV>((q0[p] >> 4) & 0x0f0f0f0fu, h0, h1, h2, h3);
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    s0[b] = dot4(l0, l1, l2, l3, xs.q(b, p), s0[b]);
+                    s0[b] = dot4(h0, h1, h2, h3, xs.q(b, p + 4), s0[b]);
+                }
+                cvt4<CV>(q1[p] & 0x0f0f0f0fu, l0, l1, l2, l3);
+                cvt4<CV>((q1[p] >> 4) & 0x0f0f0f0fu, h0, h1, h2, h3);
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    s1[b] = dot4(l0, l1, l2, l3, xs.q(b, 8 + p), s1[b]);
+                    s1[b] = dot4(h0, h1, h2, h3, xs.q(b, 12 + p), s1[b]);
+                }
+            }
+            const float d0 = h2f(w[r].a.x) * nib, m0 = h2f(w[r].a.x >> 16), d1 = h2f(w[r].b.y) * nib, m1 = h2f(w[r].b.y >> 16);
+#pragma unroll
+            for (int b = 0; b < B; ++b) {
+                float t = __builtin_fmaf(d0, s0[b], m0 * xs.s(b, 0));
+                t = __builtin_fmaf(d1, s1[b], t);
+                acc[r][b] += __builtin_fmaf(m1, xs.s(b, 1), t);
+            }
+        }
+    }
+};
+
+// two block_q8_0: bytes 0-1 d0, 2-33 qs0, 34-35 d1, 36-67 qs1
+template <>
+struct UnitPair<F_Q8_0> {
+    static constexpr int FMT = F_Q8_0;
+    static constexpr int UV = 64, NS = 2, SG = 8, NOFF = 1;
+    struct Raw { u32x4 a, b, c, d; uint32_t e; };
+    __device__ static __forceinline__ void offsets(int u, uint32_t (&o)[NOFF]) { o[0] = (uint32_t)u * 68u; }
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *row, const uint32_t (&o)[NOFF]) {
+        r.a = ld128<4>(row + o[0]);
+        r.b = ld128<4>(row + o[0] + 16);
+        r.c = ld128<4>(row + o[0] + 32);
+        r.d = ld128<4>(row + o[0] + 48);
+        r.e = ld32<4>(row + o[0] + 64);
+    }
+    __device__ static __forceinline__ void slot(int f, int &u, int &g) { u = f >> 4; g = f & 15; }
+
+    template <int B, int R, int CV, class X>
+    __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
+        (void)u;
+        (void)nib;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t v[17] = {w[r].a.x, w[r].a.y, w[r].a.z, w[r].a.w, w[r].b.x, w[r].b.y, w[r].b.z, w[r].b.w, w[r].c.x,
+                                    w[r].c.y, w[r].c.z, w[r].c.w, w[r].d.x, w[r].d.y, w[r].d.z, w[r].d.w, w[r].e};
+            float s0[B], s1[B];
+#pragma unroll
+            for (int b = 0; b < B; ++b) s0[b] = s1[b] = 0.f;
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const uint32_t a = __builtin_amdgcn_alignbit(v[p + 1], v[p], 16) ^ 0x80808080u;
+                const uint32_t c = v[9 + p] ^ 0x80808080u;
+#pragma unroll
+                for (int b = 0; b < B; ++b) {
+                    s0[b] = dot4(ub0(a), ub1(a), ub2(a), ub3(a), xs.q(b, p), s0[b]);
+                    s1[b] = dot4(ub0(c), ub1(c), ub2(c), ub3(c), xs.q(b, 8 + p), s1[b]);
+                }
+            }
+            const float d0 = h2f(v[0]), d1 = h2f(v[8] >> 16);
+#pragma unroll
+            for (int b = 0; b < B; ++b) {
+                float t = d0 * __builtin_fmaf(-128.f, xs.s(b, 0), s0[b]);
+                acc[r][b] += __builtin_fmaf(d1, __builtin_fmaf(-128.f, xs.s(b, 1), s1[b]), t);
+            }
+        }
+    }
+};
+
 // Batch-1 GEMV for rows of at most 4096 values: the activations live in registers.
 //
 // The vector is staged through LDS once per workgroup (coalesced global read, unit-order write), each lane
@@ -460,12 +627,11 @@ struct Unit<F_Q8_0> {
 // The first rows' loads are issued before the staging barrier, so HBM latency overlaps the staging too.
 constexpr int XREG_THREADS = 256;  // workgroup size of gemv_xreg_kernel (compile-time: the staging is fully unrolled)
 
-template <int FMT, int STEPS, int CV, int PF, bool BIAS>
+template <class U, int CV, int PF, bool BIAS>
 __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
                                                          const float *__restrict__ bias, float *__restrict__ y, int n, int k, float nib) {
-    using U = Unit<FMT>;
+    constexpr int FMT = U::FMT, STEPS = 64 / U::UV;  // a lane keeps 64 activations: one 64-value unit or two of 32
     constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG, NB = PF + 1;
-    static_assert(STEPS * U::UV == 64, "a lane keeps 64 activations");
     __shared__ float4 xl[STEPS * 64 * (UQ + 1)];
     __shared__ float sums[STEPS * 64 * NS];
     constexpr int nwaves = XREG_THREADS / 64;
@@ -565,18 +731,17 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *
 //   launch: blockDim.x = 64 * slices, dynamic LDS = gemv_ksplit_lds_bytes<FMT>(slices).
 constexpr int KS_FLUSH = 32;
 
-template <int FMT>
+template <class U>
 __host__ __device__ constexpr size_t gemv_ksplit_lds_bytes(int slices) {
-    constexpr int STEPS = 64 / Unit<FMT>::UV;
-    return (size_t)slices * STEPS * 64 * ((Unit<FMT>::UV / 4 + 1) * 16 + Unit<FMT>::NS * 4);
+    constexpr int STEPS = 64 / U::UV;
+    return (size_t)slices * STEPS * 64 * ((U::UV / 4 + 1) * 16 + U::NS * 4);
 }
 
-template <int FMT, int STEPS, int CV, int PF>
+template <class U, int CV, int PF>
 __global__ void __launch_bounds__(512) gemv_ksplit_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
                                                             const float *__restrict__ bias, float *__restrict__ y, int n, int k, float nib) {
-    using U = Unit<FMT>;
+    constexpr int FMT = U::FMT, STEPS = 64 / U::UV;
     constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG, NB = PF + 1;
-    static_assert(STEPS * U::UV == 64, "a lane keeps 64 activations");
     extern __shared__ float4 smem[];
     __shared__ float part[KS_FLUSH][8];  // at most 8 slices: rows of up to 32768 values
     const int tid = threadIdx.x, lane = tid & 63;

@@ -53,7 +53,7 @@ struct State {
     size_t max_lds = 0;      // LDS one workgroup may ask for
     size_t lds_per_cu = 0;   // LDS of a compute unit
     int xreg_blocks_per_cu = 0;  // JITNN_HIP_XREG_BLOCKS: override of the workgroups per CU (0 = built-in choice)
-    int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1..3 (0 = built-in choice)
+    int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1 or 2 (0 = built-in choice)
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
 };
 State g;
@@ -112,24 +112,23 @@ int unit_values(int fmt) { return block_values(fmt) == 256 ? 64 : 32; }
 
 typedef void (*gemv1_fn)(const uint8_t *, const float *, const float *, float *, int, int, float);
 
+// The 32-value formats decode pairs of blocks when the row holds an even number of them (aligned loads),
+// single blocks otherwise.
 template <int PF, bool BIAS>
-gemv1_fn pick_xreg_pf(int fmt) {
+gemv1_fn pick_xreg_pf(int fmt, bool pairs) {
     switch (fmt) {
-    case F_Q4_0: return gemv_xreg_kernel<F_Q4_0, 2, 1, PF, BIAS>;
-    case F_Q4_1: return gemv_xreg_kernel<F_Q4_1, 2, 1, PF, BIAS>;
-    case F_Q8_0: return gemv_xreg_kernel<F_Q8_0, 2, 0, PF, BIAS>;
-    case F_Q4_K: return gemv_xreg_kernel<F_Q4_K, 1, 1, PF, BIAS>;
-    case F_Q5_K: return gemv_xreg_kernel<F_Q5_K, 1, 0, PF, BIAS>;
-    default: return gemv_xreg_kernel<F_Q6_K, 1, 0, PF, BIAS>;
+    case F_Q4_0: return pairs ? gemv_xreg_kernel<UnitPair<F_Q4_0>, 1, PF, BIAS> : gemv_xreg_kernel<Unit<F_Q4_0>, 1, PF, BIAS>;
+    case F_Q4_1: return pairs ? gemv_xreg_kernel<UnitPair<F_Q4_1>, 1, PF, BIAS> : gemv_xreg_kernel<Unit<F_Q4_1>, 1, PF, BIAS>;
+    case F_Q8_0: return pairs ? gemv_xreg_kernel<UnitPair<F_Q8_0>, 0, PF, BIAS> : gemv_xreg_kernel<Unit<F_Q8_0>, 0, PF, BIAS>;
+    case F_Q4_K: return gemv_xreg_kernel<Unit<F_Q4_K>, 1, PF, BIAS>;
+    case F_Q5_K: return gemv_xreg_kernel<Unit<F_Q5_K>, 0, PF, BIAS>;
+    default: return gemv_xreg_kernel<Unit<F_Q6_K>, 0, PF, BIAS>;
     }
 }
 
-gemv1_fn pick_xreg(int fmt, bool bias, int pf) {
-    switch (pf) {
-    case 1: return bias ? pick_xreg_pf<1, true>(fmt) : pick_xreg_pf<1, false>(fmt);
-    case 3: return bias ? pick_xreg_pf<3, true>(fmt) : pick_xreg_pf<3, false>(fmt);
-    default: return bias ? pick_xreg_pf<2, true>(fmt) : pick_xreg_pf<2, false>(fmt);
-    }
+gemv1_fn pick_xreg(int fmt, bool pairs, bool bias, int pf) {
+    if (pf == 1) return bias ? pick_xreg_pf<1, true>(fmt, pairs) : pick_xreg_pf<1, false>(fmt, pairs);
+    return bias ? pick_xreg_pf<2, true>(fmt, pairs) : pick_xreg_pf<2, false>(fmt, pairs);
 }
 
 // Batch 1, rows of at most 4096 values: activations in registers, one row per wave iteration.
@@ -143,32 +142,26 @@ int launch_gemv_xreg(const jitnn_hip_weight *w, const float *x, const float *bia
     if (blocks > cap) blocks = cap;
     const int rows_per_wave = (w->n + blocks * waves - 1) / (blocks * waves);
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
-    hipLaunchKernelGGL(pick_xreg(w->fmt, bias != nullptr, pf), dim3(blocks), dim3(threads), 0, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
+    hipLaunchKernelGGL(pick_xreg(w->fmt, w->k % 64 == 0, bias != nullptr, pf), dim3(blocks), dim3(threads), 0, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
 
 template <int PF>
-gemv1_fn pick_ksplit_pf(int fmt) {
+gemv1_fn pick_ksplit_pf(int fmt, bool pairs) {
     switch (fmt) {
-    case F_Q4_0: return gemv_ksplit_kernel<F_Q4_0, 2, 1, PF>;
-    case F_Q4_1: return gemv_ksplit_kernel<F_Q4_1, 2, 1, PF>;
-    case F_Q8_0: return gemv_ksplit_kernel<F_Q8_0, 2, 0, PF>;
-    case F_Q4_K: return gemv_ksplit_kernel<F_Q4_K, 1, 1, PF>;
-    case F_Q5_K: return gemv_ksplit_kernel<F_Q5_K, 1, 0, PF>;
-    default: return gemv_ksplit_kernel<F_Q6_K, 1, 0, PF>;
+    case F_Q4_0: return pairs ? gemv_ksplit_kernel<UnitPair<F_Q4_0>, 1, PF> : gemv_ksplit_kernel<Unit<F_Q4_0>, 1, PF>;
+    case F_Q4_1: return pairs ? gemv_ksplit_kernel<UnitPair<F_Q4_1>, 1, PF> : gemv_ksplit_kernel<Unit<F_Q4_1>, 1, PF>;
+    case F_Q8_0: return pairs ? gemv_ksplit_kernel<UnitPair<F_Q8_0>, 0, PF> : gemv_ksplit_kernel<Unit<F_Q8_0>, 0, PF>;
+    case F_Q4_K: return gemv_ksplit_kernel<Unit<F_Q4_K>, 1, PF>;
+    case F_Q5_K: return gemv_ksplit_kernel<Unit<F_Q5_K>, 0, PF>;
+    default: return gemv_ksplit_kernel<Unit<F_Q6_K>, 0, PF>;
     }
 }
 
-size_t ksplit_lds(int fmt, int slices) {
-    switch (fmt) {
-    case F_Q4_0: return gemv_ksplit_lds_bytes<F_Q4_0>(slices);
-    case F_Q4_1: return gemv_ksplit_lds_bytes<F_Q4_1>(slices);
-    case F_Q8_0: return gemv_ksplit_lds_bytes<F_Q8_0>(slices);
-    case F_Q4_K: return gemv_ksplit_lds_bytes<F_Q4_K>(slices);
-    case F_Q5_K: return gemv_ksplit_lds_bytes<F_Q5_K>(slices);
-    default: return gemv_ksplit_lds_bytes<F_Q6_K>(slices);
-    }
+size_t ksplit_lds(int fmt, int slices) {  // the single-block units need the most: 2 x 64 x (9 quads + 1 sum)
+    if (block_values(fmt) == 32) return gemv_ksplit_lds_bytes<Unit<F_Q4_0>>(slices);
+    return fmt == F_Q6_K ? gemv_ksplit_lds_bytes<Unit<F_Q6_K>>(slices) : gemv_ksplit_lds_bytes<Unit<F_Q4_K>>(slices);
 }
 
 // Batch 1, rows of 4097..32768 values: one wave per 4096-value slice of the row, partial sums joined in LDS.
@@ -183,7 +176,7 @@ int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *b
     int blocks = w->n < g.cus * per_cu ? w->n : g.cus * per_cu;
     const int rows_per_block = (w->n + blocks - 1) / blocks;
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_block >= 16 ? 1 : 2);
-    gemv1_fn fn = pf == 1 ? pick_ksplit_pf<1>(w->fmt) : pf == 3 ? pick_ksplit_pf<3>(w->fmt) : pick_ksplit_pf<2>(w->fmt);
+    gemv1_fn fn = pf == 1 ? pick_ksplit_pf<1>(w->fmt, w->k % 64 == 0) : pick_ksplit_pf<2>(w->fmt, w->k % 64 == 0);
     if (lds > 65536) HIP_TRY(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(64 * slices), lds, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
     HIP_TRY(hipGetLastError());
@@ -296,7 +289,7 @@ int jitnn_hip_init(int device_ordinal) {
     }
     if (const char *e = getenv("JITNN_HIP_XREG_PF")) {
         int v = atoi(e);
-        if (v >= 1 && v <= 3) g.xreg_pf = v;
+        if (v >= 1 && v <= 2) g.xreg_pf = v;
     }
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     g.device = device_ordinal;
