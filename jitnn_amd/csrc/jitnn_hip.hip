@@ -14,6 +14,7 @@
 
 #include "dequant.h"
 #include "gemv.h"
+#include "prefill.h"
 
 using namespace jitnn;
 
@@ -54,6 +55,10 @@ struct State {
     size_t lds_per_cu = 0;   // LDS of a compute unit
     int xreg_blocks_per_cu = 0;  // JITNN_HIP_XREG_BLOCKS: override of the workgroups per CU (0 = built-in choice)
     int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1 or 2 (0 = built-in choice)
+    // JITNN_HIP_GEMV_MAX_ROWS: up to this many rows run the FP32 GEMV kernels (in batches of 8), more rows the FP16
+    // MFMA kernel - the counterpart of jitnn.gguf.tiledRows (core/JitnnConfig.java:423-424).  64 keeps every row
+    // count the reference's own tests use (1, 5, 40) on the FP32 path, whose error meets their 2e-4 / 1e-3 bars.
+    int gemv_max_rows = 64;
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
 };
 State g;
@@ -208,6 +213,70 @@ int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float
     return JITNN_HIP_OK;
 }
 
+// Per-thread device scratch for the many-row path (FP16 activations and their row scales).  It only grows; a call
+// on another stream than the last one first waits for the previous user, so concurrent streams of one thread
+// cannot overwrite each other's activations.
+struct Workspace {
+    void *ptr = nullptr;
+    size_t cap = 0;
+    hipStream_t last = nullptr;
+    hipEvent_t ev = nullptr;
+    bool used = false;
+};
+thread_local Workspace g_ws;
+
+int workspace(size_t bytes, hipStream_t stream, void **out) {
+    Workspace &w = g_ws;
+    if (!w.ev) HIP_TRY(hipEventCreateWithFlags(&w.ev, hipEventDisableTiming));
+    if (bytes > w.cap) {
+        if (w.ptr) HIP_TRY(hipFree(w.ptr));  // waits for the device: nobody is still reading the old block
+        w.ptr = nullptr;
+        w.cap = 0;
+        const size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+        hipError_t e = hipMalloc(&w.ptr, want);
+        if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc of %zu bytes of scratch: %s", want, hipGetErrorString(e));
+        w.cap = want;
+        w.used = false;
+    }
+    if (w.used && w.last != stream) HIP_TRY(hipStreamWaitEvent(stream, w.ev, 0));
+    *out = w.ptr;
+    return JITNN_HIP_OK;
+}
+
+int workspace_done(hipStream_t stream) {
+    Workspace &w = g_ws;
+    HIP_TRY(hipEventRecord(w.ev, stream));
+    w.last = stream;
+    w.used = true;
+    return JITNN_HIP_OK;
+}
+
+template <int FMT>
+void launch_prefill_fmt(const jitnn_hip_weight *w, const _Float16 *xh, const float *inv, int rows, const float *bias, float *y, hipStream_t s) {
+    dim3 grid((w->n + PF_BN - 1) / PF_BN, (rows + PF_BM - 1) / PF_BM);
+    hipLaunchKernelGGL(prefill_mfma_kernel<FMT>, grid, dim3(256), 0, s, w->dev, xh, inv, bias, y, rows, w->n, w->k);
+}
+
+// rows > 8: FP16 activations + dequantise-to-LDS MFMA kernel
+int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    const size_t xh_bytes = ((size_t)rows * w->k * 2 + 255) & ~(size_t)255;
+    void *ws = nullptr;
+    if (int rc = workspace(xh_bytes + (size_t)rows * 4, stream, &ws)) return rc;
+    _Float16 *xh = (_Float16 *)ws;
+    float *inv = (float *)((uint8_t *)ws + xh_bytes);
+    hipLaunchKernelGGL(x_to_f16_kernel, dim3(rows), dim3(256), 0, stream, x, xh, inv, w->k);
+    switch (w->fmt) {
+    case F_Q4_0: launch_prefill_fmt<F_Q4_0>(w, xh, inv, rows, bias, y, stream); break;
+    case F_Q4_1: launch_prefill_fmt<F_Q4_1>(w, xh, inv, rows, bias, y, stream); break;
+    case F_Q8_0: launch_prefill_fmt<F_Q8_0>(w, xh, inv, rows, bias, y, stream); break;
+    case F_Q4_K: launch_prefill_fmt<F_Q4_K>(w, xh, inv, rows, bias, y, stream); break;
+    case F_Q5_K: launch_prefill_fmt<F_Q5_K>(w, xh, inv, rows, bias, y, stream); break;
+    default: launch_prefill_fmt<F_Q6_K>(w, xh, inv, rows, bias, y, stream); break;
+    }
+    HIP_TRY(hipGetLastError());
+    return workspace_done(stream);
+}
+
 template <int FMT>
 void launch_dequant(const jitnn_hip_weight *w, float *y, hipStream_t stream) {
     const size_t quads = (size_t)w->n * w->k / 4;
@@ -290,6 +359,10 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_XREG_PF")) {
         int v = atoi(e);
         if (v >= 1 && v <= 2) g.xreg_pf = v;
+    }
+    if (const char *e = getenv("JITNN_HIP_GEMV_MAX_ROWS")) {
+        int v = atoi(e);
+        if (v >= 1) g.gemv_max_rows = v;
     }
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     g.device = device_ordinal;
@@ -400,6 +473,7 @@ int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows
     if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
     if (int rc = check_ready()) return rc;
     hipStream_t s = (hipStream_t)stream;
+    if (rows > g.gemv_max_rows) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s);
     for (int r0 = 0; r0 < rows; r0 += 8) {
         const int nb = rows - r0 < 8 ? rows - r0 : 8;
         if (int rc = launch_gemv(w, x_dev + (size_t)r0 * w->k, nb, bias_dev, y_dev + (size_t)r0 * w->n, s)) return rc;

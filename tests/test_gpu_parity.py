@@ -11,7 +11,12 @@ from helpers import (GGML_ID, GGML_NAMES, GOLDEN_CODE_TO_GGML, HOT_FORMATS, Java
 
 pytestmark = pytest.mark.gpu
 
-GEMV_BAR = 1e-4
+GEMV_BAR = 1e-4    # up to 64 rows: FP32 GEMV kernels (this covers every row count the reference's own tests use)
+MFMA_BAR = 2e-3    # more rows (prefill): FP16 MFMA kernel
+
+
+def bar(rows):
+    return GEMV_BAR if rows <= 64 else MFMA_BAR
 
 
 @pytest.fixture(scope="module")
@@ -72,7 +77,7 @@ def test_linear_goldens(jn, goldens, code, rows):
     y = jn.Gguf.linear(jn.Tensor.of(x), weight(jn, fmt, raw, n, 512), jn.Tensor.of(bias)).numpy()
     assert y.shape == out.shape
     assert checks_close(y, out, 1e-4, 1e-3)
-    assert norm_err(y, out) <= GEMV_BAR
+    assert norm_err(y, out) <= bar(rows)
 
 
 @pytest.mark.parametrize("fmt", HOT_FORMATS)
@@ -88,8 +93,8 @@ def test_linear_ggufchecks_recipe(jn, gguf_fixture, fmt):
         x = np.array([rnd.next_float() * np.float32(2) - np.float32(1) for _ in range(rows * 512)], dtype=np.float32).reshape(rows, 512)
         ref = (bias.astype(np.float64)[None, :] + x.astype(np.float64) @ expect.T).astype(np.float32)
         y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias)).numpy()
-        assert norm_err(y, ref) <= 2e-4
-        assert norm_err(y, oracle.gguf_linear(GGML_ID[fmt], x, raw, bias, 3, 512)) <= GEMV_BAR
+        assert norm_err(y, ref) <= 2e-4, (fmt, rows, norm_err(y, ref))
+        assert norm_err(y, oracle.gguf_linear(GGML_ID[fmt], x, raw, bias, 3, 512)) <= bar(rows)
 
 
 # ------------------------------------------------------------------------------------------ linear, seeded inputs vs oracle
@@ -117,18 +122,57 @@ def test_gemv_vs_oracle(jn, fmt, n, k):
 
 @pytest.mark.parametrize("fmt", HOT_FORMATS)
 def test_small_k_32_blocks_and_many_rows(jn, fmt):
-    """K of a single block for the 32-value formats; rows beyond one batch of 8 (9, 17, 40)."""
+    """K of a single block for the 32-value formats; rows beyond one batch of 8 (9, 17, 40, 64)."""
     from oracle import oracle
     rng = np.random.default_rng(77)
     k = 32 * 3 if fmt in ("Q8_0", "Q4_0", "Q4_1") else 256
     n = 19
     raw = random_valid_blocks(rng, fmt, n, k)
     w = weight(jn, fmt, raw, n, k)
-    for rows in (9, 17, 40):
+    for rows in (9, 17, 40, 64):
         x = rng.standard_normal((rows, k)).astype(np.float32)
         ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, None, n, k)
         y = jn.Gguf.linear(jn.Tensor.of(x), w, None).numpy()
-        assert norm_err(y, ref) <= GEMV_BAR, (fmt, rows)
+        assert norm_err(y, ref) <= bar(rows), (fmt, rows, norm_err(y, ref))
+
+
+PREFILL_SHAPES = [  # (n, k, rows): ragged tiles in every dimension, K past one step, a 32-value K tail
+    (256, 1024, 65), (131, 4096, 200), (64, 14336, 97), (130, 512, 129), (1, 256, 70),
+]
+
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
+@pytest.mark.parametrize("n,k,rows", PREFILL_SHAPES)
+def test_prefill_mfma_vs_oracle(jn, fmt, n, k, rows):
+    """More than 64 rows run the dequantise-to-LDS MFMA kernel (FP16 operands, FP32 accumulation): bar 2e-3."""
+    from oracle import oracle
+    rng = np.random.default_rng(n * 7 + k + rows + GGML_ID[fmt])
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[0] *= 1e4      # rows of very different magnitude: the per-row FP16 scale must cope
+    x[1] *= 1e-6
+    bias = rng.standard_normal(n).astype(np.float32)
+    ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, bias, n, k)
+    y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias)).numpy()
+    assert y.shape == (rows, n)
+    # row by row (a tiny row must not hide behind a huge one), against the larger of the row's biggest output and the
+    # typical output magnitude |x_r| * rms row norm of W (one output alone can be small by cancellation)
+    wnorm = float(np.sqrt((ggml_numpy.dequant(fmt, raw).astype(np.float64) ** 2).sum() / n))
+    for r in range(rows):
+        scale = max(float(np.abs(ref[r] - bias).max()), float(np.linalg.norm(x[r].astype(np.float64))) * wnorm, 1e-30)
+        assert np.abs(y[r] - ref[r]).max() <= MFMA_BAR * scale + 1e-6 * np.abs(bias).max(), (fmt, r)
+
+
+@pytest.mark.parametrize("fmt", ["Q4_0", "Q8_0", "Q4_1"])
+def test_prefill_k_tail_of_32(jn, fmt):
+    from oracle import oracle
+    rng = np.random.default_rng(3)
+    n, k, rows = 40, 32 * 7, 70
+    raw = random_valid_blocks(rng, fmt, n, k)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    y = jn.Gguf.linear(jn.Tensor.of(x), weight(jn, fmt, raw, n, k), None).numpy()
+    assert norm_err(y, oracle.gguf_linear(GGML_ID[fmt], x, raw, None, n, k)) <= MFMA_BAR
 
 
 @pytest.mark.parametrize("fmt", HOT_FORMATS)
