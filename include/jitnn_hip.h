@@ -120,6 +120,52 @@ JITNN_HIP_API int jitnn_hip_free(void *dev);
 JITNN_HIP_API int jitnn_hip_memcpy_h2d(void *dev, const void *host, long long nbytes);
 JITNN_HIP_API int jitnn_hip_memcpy_d2h(void *host, const void *dev, long long nbytes);
 
+/* ---- Llama-style decode step on quantised weights (BASELINE config 5) ----------------------------- */
+
+/* The reference has no quantised Llama and no KV-cache operator; the step is the composition of its operators as
+ * Llama.Block.forward defines it (jitnn-nn/src/main/java/ai/beestream/jitnn/nn/models/Llama.java:167-174,209-222)
+ * with every Linear replaced by the quantised linear above and attention of the one new token over an FP32
+ * cache: RMSNorm (core/ops/RowNorm.java:286-306), rotary embedding in the rotate-half form
+ * (core/ops/Rope.java:86-150), grouped-query attention (core/F.java:588-624, core/ops/FlashAttention.java:538-626),
+ * SwiGLU (core/F.java:1159-1161), residual adds.  Activations stay in HBM for the whole step. */
+typedef struct jitnn_hip_llama jitnn_hip_llama;
+
+#define JITNN_HIP_W_ATTN_Q 0
+#define JITNN_HIP_W_ATTN_K 1
+#define JITNN_HIP_W_ATTN_V 2
+#define JITNN_HIP_W_ATTN_O 3
+#define JITNN_HIP_W_FFN_GATE 4
+#define JITNN_HIP_W_FFN_UP 5
+#define JITNN_HIP_W_FFN_DOWN 6
+#define JITNN_HIP_W_OUTPUT 7 /* layer argument ignored */
+
+#define JITNN_HIP_NORM_ATTN 0
+#define JITNN_HIP_NORM_FFN 1
+#define JITNN_HIP_NORM_OUTPUT 2 /* layer argument ignored */
+
+/* head_dim must be 64, 128, 192 or 256; heads a multiple of kv_heads.  Allocates the KV cache
+ * (2 * layers * max_ctx * kv_heads * head_dim floats) and the activation buffers. */
+JITNN_HIP_API int jitnn_hip_llama_create(int layers, int d_model, int heads, int kv_heads, int head_dim, int ffn, int vocab, int max_ctx,
+                                         float rms_eps, float rope_theta, jitnn_hip_llama **out);
+JITNN_HIP_API int jitnn_hip_llama_free(jitnn_hip_llama *m);
+
+/* Attaches a weight (not owned; shapes are checked: q/o [heads*head_dim, d_model] resp. [d_model, heads*head_dim],
+ * k/v [kv_heads*head_dim, d_model], gate/up [ffn, d_model], down [d_model, ffn], output [vocab, d_model]). */
+JITNN_HIP_API int jitnn_hip_llama_set_weight(jitnn_hip_llama *m, int layer, int which, const jitnn_hip_weight *w);
+/* Copies an RMSNorm weight vector [d_model] from host memory. */
+JITNN_HIP_API int jitnn_hip_llama_set_norm(jitnn_hip_llama *m, int layer, int which, const float *w_host);
+
+/* Writes / reads `count` cache positions from pos0 of one layer: k and v are [count, kv_heads, head_dim] in host
+ * memory (keys as stored, i.e. already rotated). */
+JITNN_HIP_API int jitnn_hip_llama_kv_write(jitnn_hip_llama *m, int layer, int pos0, int count, const float *k_host, const float *v_host);
+JITNN_HIP_API int jitnn_hip_llama_kv_read(const jitnn_hip_llama *m, int layer, int pos0, int count, float *k_host, float *v_host);
+
+/* One token: x [d_model] is the token's embedding, pos its position (the cache must hold positions 0..pos-1);
+ * appends the token's keys and values at pos and writes logits [vocab].  _dev only enqueues on the stream and
+ * allocates nothing, so it can be captured into a HIP graph. */
+JITNN_HIP_API int jitnn_hip_llama_decode(jitnn_hip_llama *m, const float *x_host, int pos, float *logits_host);
+JITNN_HIP_API int jitnn_hip_llama_decode_dev(jitnn_hip_llama *m, const float *x_dev, int pos, float *logits_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,3 +8,4 @@ from ._lib import JitnnError, device_info, init  # noqa: F401
 from .dtype import DType  # noqa: F401
 from .ops import F, Gguf, Quant  # noqa: F401
 from .tensor import Tensor  # noqa: F401
+from .llama import LlamaDecoder  # noqa: F401

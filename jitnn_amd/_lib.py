@@ -45,6 +45,14 @@ def _bind() -> C.CDLL:
         "jitnn_hip_free": (i, [vp]),
         "jitnn_hip_memcpy_h2d": (i, [vp, vp, ll]),
         "jitnn_hip_memcpy_d2h": (i, [vp, vp, ll]),
+        "jitnn_hip_llama_create": (i, [i, i, i, i, i, i, i, i, C.c_float, C.c_float, C.POINTER(vp)]),
+        "jitnn_hip_llama_free": (i, [vp]),
+        "jitnn_hip_llama_set_weight": (i, [vp, i, i, vp]),
+        "jitnn_hip_llama_set_norm": (i, [vp, i, i, vp]),
+        "jitnn_hip_llama_kv_write": (i, [vp, i, i, i, vp, vp]),
+        "jitnn_hip_llama_kv_read": (i, [vp, i, i, i, vp, vp]),
+        "jitnn_hip_llama_decode": (i, [vp, vp, i, vp]),
+        "jitnn_hip_llama_decode_dev": (i, [vp, vp, i, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol

@@ -8,12 +8,16 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <utility>
+#include <vector>
 
 #include "dequant.h"
 #include "gemv.h"
+#include "glue.h"
 #include "prefill.h"
 
 using namespace jitnn;
@@ -64,6 +68,7 @@ struct State {
 State g;
 std::mutex g_mu;
 
+
 __global__ void fp8_probe_kernel(float *out) {
     f32x2 p = __builtin_amdgcn_cvt_pk_f32_fp8(0x00000f01, false);
     out[0] = p.x;
@@ -71,6 +76,21 @@ __global__ void fp8_probe_kernel(float *out) {
 }
 
 bool known(int fmt) { return block_values(fmt) != 0; }
+
+// Kernels that want more than 64 KiB of dynamic LDS must be told so once; remembered per kernel so that steady-state
+// launches (and launches under graph capture) make no attribute calls.
+int allow_lds(const void *fn, size_t lds) {
+    if (lds <= 65536) return JITNN_HIP_OK;
+    static std::mutex mu;
+    static std::vector<std::pair<const void *, size_t>> seen;
+    std::lock_guard<std::mutex> lock(mu);
+    for (auto &e : seen)
+        if (e.first == fn && e.second >= lds) return JITNN_HIP_OK;
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return fail(JITNN_HIP_EDEVICE, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds, hipGetErrorString(e));
+    seen.emplace_back(fn, lds);
+    return JITNN_HIP_OK;
+}
 
 int check_ready() {
     if (!g.ready) return fail(JITNN_HIP_ENODEVICE, "jitnn_hip_init has not succeeded in this process");
@@ -182,7 +202,7 @@ int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *b
     const int rows_per_block = (w->n + blocks - 1) / blocks;
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_block >= 16 ? 1 : 2);
     gemv1_fn fn = pf == 1 ? pick_ksplit_pf<1>(w->fmt, w->k % 64 == 0) : pick_ksplit_pf<2>(w->fmt, w->k % 64 == 0);
-    if (lds > 65536) HIP_TRY(hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (int rc = allow_lds((const void *)fn, lds)) return rc;
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(64 * slices), lds, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
@@ -202,7 +222,7 @@ int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float
     if (itc > steps) itc = steps;
     const size_t lds = v.lds_per_step * itc;
     if (lds > g.max_lds) return fail(JITNN_HIP_EINVAL, "GEMV needs %zu bytes of LDS, the device offers %zu", lds, g.max_lds);
-    if (lds > 65536) HIP_TRY(hipFuncSetAttribute((const void *)v.fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    if (int rc = allow_lds((const void *)v.fn, lds)) return rc;
     const int threads = 256, waves = threads / 64;
     const int groups = (w->n + v.R - 1) / v.R;
     int blocks = (groups + waves - 1) / waves;
@@ -564,6 +584,211 @@ int jitnn_hip_memcpy_d2h(void *host, const void *dev, long long nbytes) {
     if (!dev || !host || nbytes < 0) return fail(JITNN_HIP_EINVAL, "bad arguments");
     if (int rc = check_ready()) return rc;
     HIP_TRY(hipMemcpy(host, dev, (size_t)nbytes, hipMemcpyDeviceToHost));
+    return JITNN_HIP_OK;
+}
+
+}  // extern "C"
+
+// ================================================================================================ decode step
+
+struct jitnn_hip_llama {
+    int layers, d, heads, kv, hd, ffn, vocab, max_ctx;
+    float eps, theta;
+    const jitnn_hip_weight **w;  // [layers][7] then output
+    const jitnn_hip_weight *w_out;
+    float *norms;                // [layers][2][d] then output norm [d]
+    float *kc, *vc;              // [layers][max_ctx][kv][hd]
+    float *cosv, *sinv;          // [max_ctx][hd/2]
+    float *xin, *xa, *xb, *xn, *q, *k, *v, *att, *gate, *up, *h, *part, *logits;
+    int chunks_max;
+};
+
+namespace {
+
+template <int D>
+void launch_attention(const jitnn_hip_llama *m, int layer, int s, hipStream_t st) {
+    const int chunks = (s + ATT_CH - 1) / ATT_CH;
+    const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
+    hipLaunchKernelGGL(attn_partial_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->kc + lo, m->vc + lo, m->part, m->heads, m->kv, s,
+                       1.0f / sqrtf((float)D));
+    hipLaunchKernelGGL(attn_combine_kernel<D>, dim3(m->heads), dim3(64), 0, st, m->part, m->att, chunks);
+}
+
+int check_model(const jitnn_hip_llama *m) {
+    if (!m) return fail(JITNN_HIP_EINVAL, "model is NULL");
+    for (int l = 0; l < m->layers; ++l)
+        for (int i = 0; i < 7; ++i)
+            if (!m->w[l * 7 + i]) return fail(JITNN_HIP_EINVAL, "layer %d has no weight %d", l, i);
+    if (!m->w_out) return fail(JITNN_HIP_EINVAL, "no output weight");
+    return JITNN_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int jitnn_hip_llama_create(int layers, int d_model, int heads, int kv_heads, int head_dim, int ffn, int vocab, int max_ctx, float rms_eps,
+                           float rope_theta, jitnn_hip_llama **out) {
+    if (!out) return fail(JITNN_HIP_EINVAL, "out is NULL");
+    *out = nullptr;
+    if (layers < 1 || d_model < 1 || heads < 1 || kv_heads < 1 || ffn < 1 || vocab < 1 || max_ctx < 1)
+        return fail(JITNN_HIP_EINVAL, "non-positive model dimension");
+    if (heads % kv_heads != 0) return fail(JITNN_HIP_EINVAL, "grouped-query attention: %d query heads over %d key/value heads", heads, kv_heads);
+    if (head_dim != 64 && head_dim != 128 && head_dim != 192 && head_dim != 256)
+        return fail(JITNN_HIP_EINVAL, "head_dim %d (64, 128, 192 and 256 are built)", head_dim);
+    if (int rc = check_ready()) return rc;
+    jitnn_hip_llama *m = new (std::nothrow) jitnn_hip_llama();
+    if (!m) return fail(JITNN_HIP_ENOMEM, "out of host memory");
+    *m = jitnn_hip_llama{};
+    m->layers = layers; m->d = d_model; m->heads = heads; m->kv = kv_heads; m->hd = head_dim; m->ffn = ffn; m->vocab = vocab;
+    m->max_ctx = max_ctx; m->eps = rms_eps; m->theta = rope_theta;
+    m->w = new (std::nothrow) const jitnn_hip_weight *[(size_t)layers * 7]();
+    m->chunks_max = (max_ctx + ATT_CH - 1) / ATT_CH;
+    const size_t cache = (size_t)layers * max_ctx * kv_heads * head_dim;
+    const int qd = heads * head_dim, kd = kv_heads * head_dim, half = head_dim / 2;
+    struct { float **p; size_t n; } bufs[] = {
+        {&m->norms, ((size_t)layers * 2 + 1) * d_model}, {&m->kc, cache}, {&m->vc, cache}, {&m->cosv, (size_t)max_ctx * half},
+        {&m->sinv, (size_t)max_ctx * half}, {&m->xin, (size_t)d_model}, {&m->xa, (size_t)d_model}, {&m->xb, (size_t)d_model}, {&m->xn, (size_t)d_model},
+        {&m->q, (size_t)qd}, {&m->k, (size_t)kd}, {&m->v, (size_t)kd}, {&m->att, (size_t)qd}, {&m->gate, (size_t)ffn}, {&m->up, (size_t)ffn},
+        {&m->h, (size_t)ffn}, {&m->part, (size_t)heads * m->chunks_max * (head_dim + 2)}, {&m->logits, (size_t)vocab}};
+    bool ok = m->w != nullptr;
+    for (auto &b : bufs) {
+        if (!ok) break;
+        ok = hipMalloc(b.p, b.n * sizeof(float)) == hipSuccess;
+    }
+    if (ok) {
+        // cos/sin of t * base^(-2i/D) in double, stored FP32: Rope.tables (core/ops/Rope.java:86-102)
+        float *c = new (std::nothrow) float[(size_t)max_ctx * half], *s = new (std::nothrow) float[(size_t)max_ctx * half];
+        ok = c && s;
+        if (ok) {
+            for (int t = 0; t < max_ctx; ++t)
+                for (int i = 0; i < half; ++i) {
+                    const double frequency = pow((double)rope_theta, -2.0 * i / head_dim);
+                    const double angle = t * frequency;
+                    c[(size_t)t * half + i] = (float)cos(angle);
+                    s[(size_t)t * half + i] = (float)sin(angle);
+                }
+            ok = hipMemcpy(m->cosv, c, (size_t)max_ctx * half * 4, hipMemcpyHostToDevice) == hipSuccess &&
+                 hipMemcpy(m->sinv, s, (size_t)max_ctx * half * 4, hipMemcpyHostToDevice) == hipSuccess;
+        }
+        delete[] c;
+        delete[] s;
+    }
+    if (!ok) {
+        jitnn_hip_llama_free(m);
+        return fail(JITNN_HIP_ENOMEM, "allocating the model buffers (%zu bytes of KV cache) failed", 2 * cache * sizeof(float));
+    }
+    *out = m;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_free(jitnn_hip_llama *m) {
+    if (!m) return JITNN_HIP_OK;
+    float *bufs[] = {m->norms, m->kc, m->vc, m->cosv, m->sinv, m->xin, m->xa, m->xb, m->xn, m->q, m->k, m->v, m->att, m->gate, m->up, m->h, m->part, m->logits};
+    for (float *b : bufs)
+        if (b) (void)hipFree(b);
+    delete[] m->w;
+    delete m;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_set_weight(jitnn_hip_llama *m, int layer, int which, const jitnn_hip_weight *w) {
+    if (!m || !w) return fail(JITNN_HIP_EINVAL, "model or weight is NULL");
+    if (which < 0 || which > JITNN_HIP_W_OUTPUT) return fail(JITNN_HIP_EINVAL, "weight slot %d", which);
+    const int qd = m->heads * m->hd, kd = m->kv * m->hd;
+    const int en[] = {qd, kd, kd, m->d, m->ffn, m->ffn, m->d, m->vocab};
+    const int ek[] = {m->d, m->d, m->d, qd, m->d, m->d, m->ffn, m->d};
+    if (w->n != en[which] || w->k != ek[which])
+        return fail(JITNN_HIP_EINVAL, "weight slot %d needs shape [%d, %d], got [%d, %d]", which, en[which], ek[which], w->n, w->k);
+    if (which == JITNN_HIP_W_OUTPUT) {
+        m->w_out = w;
+        return JITNN_HIP_OK;
+    }
+    if (layer < 0 || layer >= m->layers) return fail(JITNN_HIP_EINVAL, "layer %d of %d", layer, m->layers);
+    m->w[layer * 7 + which] = w;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_set_norm(jitnn_hip_llama *m, int layer, int which, const float *w_host) {
+    if (!m || !w_host) return fail(JITNN_HIP_EINVAL, "model or weights are NULL");
+    size_t off;
+    if (which == JITNN_HIP_NORM_OUTPUT) {
+        off = (size_t)m->layers * 2 * m->d;
+    } else if (which == JITNN_HIP_NORM_ATTN || which == JITNN_HIP_NORM_FFN) {
+        if (layer < 0 || layer >= m->layers) return fail(JITNN_HIP_EINVAL, "layer %d of %d", layer, m->layers);
+        off = ((size_t)layer * 2 + which) * m->d;
+    } else {
+        return fail(JITNN_HIP_EINVAL, "norm slot %d", which);
+    }
+    HIP_TRY(hipMemcpy(m->norms + off, w_host, (size_t)m->d * 4, hipMemcpyHostToDevice));
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_kv_write(jitnn_hip_llama *m, int layer, int pos0, int count, const float *k_host, const float *v_host) {
+    if (!m || !k_host || !v_host) return fail(JITNN_HIP_EINVAL, "NULL argument");
+    if (layer < 0 || layer >= m->layers || pos0 < 0 || count < 0 || pos0 + count > m->max_ctx)
+        return fail(JITNN_HIP_EINVAL, "layer %d positions [%d, %d) of a cache of %d", layer, pos0, pos0 + count, m->max_ctx);
+    const size_t row = (size_t)m->kv * m->hd, off = ((size_t)layer * m->max_ctx + pos0) * row;
+    HIP_TRY(hipMemcpy(m->kc + off, k_host, count * row * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(m->vc + off, v_host, count * row * 4, hipMemcpyHostToDevice));
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_kv_read(const jitnn_hip_llama *m, int layer, int pos0, int count, float *k_host, float *v_host) {
+    if (!m || !k_host || !v_host) return fail(JITNN_HIP_EINVAL, "NULL argument");
+    if (layer < 0 || layer >= m->layers || pos0 < 0 || count < 0 || pos0 + count > m->max_ctx)
+        return fail(JITNN_HIP_EINVAL, "layer %d positions [%d, %d) of a cache of %d", layer, pos0, pos0 + count, m->max_ctx);
+    const size_t row = (size_t)m->kv * m->hd, off = ((size_t)layer * m->max_ctx + pos0) * row;
+    HIP_TRY(hipMemcpy(k_host, m->kc + off, count * row * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(v_host, m->vc + off, count * row * 4, hipMemcpyDeviceToHost));
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_decode_dev(jitnn_hip_llama *m, const float *x_dev, int pos, float *logits_dev, void *stream) {
+    if (int rc = check_model(m)) return rc;
+    if (!x_dev || !logits_dev) return fail(JITNN_HIP_EINVAL, "input or output is NULL");
+    if (pos < 0 || pos >= m->max_ctx) return fail(JITNN_HIP_EINVAL, "position %d of a cache of %d", pos, m->max_ctx);
+    hipStream_t st = (hipStream_t)stream;
+    const int d = m->d;
+    // residual stream: layer input x (the caller's buffer for layer 0, xb afterwards) -> xa after attention -> xb after the FFN
+    const float *x = x_dev;
+    for (int l = 0; l < m->layers; ++l) {
+        const jitnn_hip_weight *const *w = m->w + (size_t)l * 7;
+        const float *nw = m->norms + (size_t)l * 2 * d;
+        hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, x, nw, m->xn, d, m->eps);
+        if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_Q], m->xn, 1, nullptr, m->q, st)) return rc;
+        if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_K], m->xn, 1, nullptr, m->k, st)) return rc;
+        if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_V], m->xn, 1, nullptr, m->v, st)) return rc;
+        const size_t lo = (size_t)l * m->max_ctx * m->kv * m->hd;
+        hipLaunchKernelGGL(rope_append_kernel, dim3(8), dim3(256), 0, st, m->q, m->k, m->v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads,
+                           m->kv, m->hd, pos);
+        switch (m->hd) {
+        case 64: launch_attention<64>(m, l, pos + 1, st); break;
+        case 128: launch_attention<128>(m, l, pos + 1, st); break;
+        case 192: launch_attention<192>(m, l, pos + 1, st); break;
+        default: launch_attention<256>(m, l, pos + 1, st); break;
+        }
+        // xa = x + Wo att, xb = xa + W2 h: the residual rides in the linear's bias slot
+        if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_O], m->att, 1, x, m->xa, st)) return rc;
+        hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, m->xa, nw + d, m->xn, d, m->eps);
+        if (int rc = launch_gemv(w[JITNN_HIP_W_FFN_GATE], m->xn, 1, nullptr, m->gate, st)) return rc;
+        if (int rc = launch_gemv(w[JITNN_HIP_W_FFN_UP], m->xn, 1, nullptr, m->up, st)) return rc;
+        hipLaunchKernelGGL(swiglu_kernel, dim3((m->ffn + 1023) / 1024), dim3(256), 0, st, m->gate, m->up, m->h, m->ffn);
+        if (int rc = launch_gemv(w[JITNN_HIP_W_FFN_DOWN], m->h, 1, m->xa, m->xb, st)) return rc;
+        x = m->xb;
+    }
+    hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, x, m->norms + (size_t)m->layers * 2 * d, m->xn, d, m->eps);
+    if (int rc = launch_gemv(m->w_out, m->xn, 1, nullptr, logits_dev, st)) return rc;
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_decode(jitnn_hip_llama *m, const float *x_host, int pos, float *logits_host) {
+    if (int rc = check_model(m)) return rc;
+    if (!x_host || !logits_host) return fail(JITNN_HIP_EINVAL, "input or output is NULL");
+    HIP_TRY(hipMemcpy(m->xin, x_host, (size_t)m->d * 4, hipMemcpyHostToDevice));
+    if (int rc = jitnn_hip_llama_decode_dev(m, m->xin, pos, m->logits, nullptr)) return rc;
+    HIP_TRY(hipMemcpy(logits_host, m->logits, (size_t)m->vocab * 4, hipMemcpyDeviceToHost));
     return JITNN_HIP_OK;
 }
 

@@ -1,0 +1,84 @@
+"""Host mirror of the decode-step entry points (jitnn_hip_llama_*): a Llama-style stack whose linears are
+quantised weights, one token per step over an FP32 KV cache.  The arithmetic is the reference's Llama.Block.forward
+(jitnn-nn/src/main/java/ai/beestream/jitnn/nn/models/Llama.java:167-174,209-222) with Gguf.linear in place of Linear."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from .tensor import Tensor
+
+W_ATTN_Q, W_ATTN_K, W_ATTN_V, W_ATTN_O, W_FFN_GATE, W_FFN_UP, W_FFN_DOWN, W_OUTPUT = range(8)
+NORM_ATTN, NORM_FFN, NORM_OUTPUT = range(3)
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+class LlamaDecoder:
+    def __init__(self, layers, d_model, heads, kv_heads, head_dim, ffn, vocab, max_ctx, rms_eps=1e-5, rope_theta=5e5):
+        _lib.init()
+        self.cfg = dict(layers=layers, d_model=d_model, heads=heads, kv_heads=kv_heads, head_dim=head_dim, ffn=ffn, vocab=vocab,
+                        max_ctx=max_ctx, rms_eps=rms_eps, rope_theta=rope_theta)
+        self._h = C.c_void_p()
+        _lib.check(_lib.lib.jitnn_hip_llama_create(layers, d_model, heads, kv_heads, head_dim, ffn, vocab, max_ctx, rms_eps, rope_theta,
+                                                   C.byref(self._h)), "jitnn_hip_llama_create")
+        self._keep = []  # weights are not owned by the native model: keep their tensors alive
+
+    def close(self):
+        if self._h:
+            _lib.lib.jitnn_hip_llama_free(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def handle(self):
+        return self._h
+
+    def set_weight(self, layer: int, which: int, w: Tensor) -> None:
+        _lib.check(_lib.lib.jitnn_hip_llama_set_weight(self._h, layer, which, w.handle), "jitnn_hip_llama_set_weight")
+        self._keep.append(w)
+
+    def set_weight_handle(self, layer: int, which: int, handle) -> None:
+        _lib.check(_lib.lib.jitnn_hip_llama_set_weight(self._h, layer, which, handle), "jitnn_hip_llama_set_weight")
+
+    def set_norm(self, layer: int, which: int, w) -> None:
+        a = np.ascontiguousarray(w, dtype=np.float32)
+        if a.size != self.cfg["d_model"]:
+            raise ValueError(f"norm weight of {a.size} values for d_model {self.cfg['d_model']}")
+        _lib.check(_lib.lib.jitnn_hip_llama_set_norm(self._h, layer, which, _p(a)), "jitnn_hip_llama_set_norm")
+
+    def kv_write(self, layer: int, pos0: int, k, v) -> None:
+        k = np.ascontiguousarray(k, dtype=np.float32)
+        v = np.ascontiguousarray(v, dtype=np.float32)
+        row = self.cfg["kv_heads"] * self.cfg["head_dim"]
+        if k.shape != v.shape or k.size % row != 0:
+            raise ValueError(f"cache rows of shape {k.shape} / {v.shape}")
+        _lib.check(_lib.lib.jitnn_hip_llama_kv_write(self._h, layer, pos0, k.size // row, _p(k), _p(v)), "jitnn_hip_llama_kv_write")
+
+    def kv_read(self, layer: int, pos0: int, count: int):
+        shape = (count, self.cfg["kv_heads"], self.cfg["head_dim"])
+        k, v = np.empty(shape, dtype=np.float32), np.empty(shape, dtype=np.float32)
+        _lib.check(_lib.lib.jitnn_hip_llama_kv_read(self._h, layer, pos0, count, _p(k), _p(v)), "jitnn_hip_llama_kv_read")
+        return k, v
+
+    def decode(self, x, pos: int) -> np.ndarray:
+        """Logits [vocab] of the token whose embedding is x [d_model] at position pos."""
+        a = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+        if a.size != self.cfg["d_model"]:
+            raise ValueError(f"embedding of {a.size} values for d_model {self.cfg['d_model']}")
+        y = np.empty(self.cfg["vocab"], dtype=np.float32)
+        _lib.check(_lib.lib.jitnn_hip_llama_decode(self._h, _p(a), pos, _p(y)), "jitnn_hip_llama_decode")
+        return y
+
+    def decode_dev(self, x_ptr: int, pos: int, logits_ptr: int, stream_ptr: int = 0) -> None:
+        _lib.check(_lib.lib.jitnn_hip_llama_decode_dev(self._h, C.c_void_p(x_ptr), pos, C.c_void_p(logits_ptr), C.c_void_p(stream_ptr)),
+                   "jitnn_hip_llama_decode_dev")

@@ -1,0 +1,108 @@
+"""The on-device decode step (jitnn_hip_llama_*) against the CPU oracle's composition of the reference operators."""
+import numpy as np
+import pytest
+import torch
+
+import quantizers
+from decode_oracle import SLOTS, decode_ref
+from helpers import GGML_ID, norm_err
+
+pytestmark = pytest.mark.gpu
+
+MIX = {"attn_q": "Q4_K", "attn_k": "Q4_K", "attn_v": "Q6_K", "attn_o": "Q4_K", "ffn_gate": "Q4_K", "ffn_up": "Q4_K", "ffn_down": "Q6_K"}
+
+
+def build(jn, cfg, seed, mix=MIX, out_fmt="Q6_K"):
+    g = torch.Generator().manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    d, qd, kd, ffn = cfg["d_model"], cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"], cfg["ffn"]
+    shapes = {"attn_q": (qd, d), "attn_k": (kd, d), "attn_v": (kd, d), "attn_o": (d, qd), "ffn_gate": (ffn, d), "ffn_up": (ffn, d),
+              "ffn_down": (d, ffn)}
+    dec = jn.LlamaDecoder(**cfg)
+    layers = []
+    for li in range(cfg["layers"]):
+        L = {}
+        for si, slot in enumerate(SLOTS):
+            n, k = shapes[slot]
+            fmt = mix[slot]
+            raw = quantizers.quantize(fmt, torch.randn(n, k, generator=g) * 0.02).numpy()
+            L[slot] = (GGML_ID[fmt], raw, n, k)
+            dec.set_weight(li, si, jn.Tensor.quantized(jn.DType[fmt], raw, n, k))
+        for ni, name in enumerate(("attn_norm", "ffn_norm")):
+            L[name] = (1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+            dec.set_norm(li, ni, L[name])
+        layers.append(L)
+    out_norm = (1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    dec.set_norm(0, 2, out_norm)
+    raw = quantizers.quantize(out_fmt, torch.randn(cfg["vocab"], d, generator=g) * 0.02).numpy()
+    out_w = (GGML_ID[out_fmt], raw, cfg["vocab"], d)
+    dec.set_weight(0, 7, jn.Tensor.quantized(jn.DType[out_fmt], raw, cfg["vocab"], d))
+    return dec, layers, out_norm, out_w
+
+
+@pytest.fixture(scope="module")
+def jn():
+    import jitnn_amd
+    jitnn_amd.init()
+    return jitnn_amd
+
+
+@pytest.mark.parametrize("mix_name", ["q4_k_m", "q8_0", "q4_0_q5_k"])
+def test_decode_small_model(jn, mix_name):
+    """Two layers, grouped heads 8/2 of size 64, three tokens decoded in a row on a pre-filled cache."""
+    cfg = dict(layers=2, d_model=512, heads=8, kv_heads=2, head_dim=64, ffn=1024, vocab=1000, max_ctx=48, rms_eps=1e-5, rope_theta=5e5)
+    mix = {"q4_k_m": MIX, "q8_0": {s: "Q8_0" for s in SLOTS},
+           "q4_0_q5_k": {**{s: "Q4_0" for s in SLOTS}, "attn_v": "Q5_K", "ffn_down": "Q5_K", "attn_o": "Q4_1"}}[mix_name]
+    dec, layers, out_norm, out_w = build(jn, cfg, 5, mix, "Q8_0" if mix_name == "q8_0" else "Q6_K")
+    rng = np.random.default_rng(1)
+    ctx0 = 37
+    kc = np.zeros((cfg["layers"], cfg["max_ctx"], cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :ctx0] = rng.standard_normal(kc[:, :ctx0].shape)
+    vc[:, :ctx0] = rng.standard_normal(vc[:, :ctx0].shape)
+    for li in range(cfg["layers"]):
+        dec.kv_write(li, 0, kc[li, :ctx0], vc[li, :ctx0])
+    for step in range(3):
+        pos = ctx0 + step
+        x = rng.standard_normal(cfg["d_model"]).astype(np.float32)
+        ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x, pos)
+        y = dec.decode(x, pos)
+        assert norm_err(y, ref) <= 1e-4, (mix_name, step, norm_err(y, ref))
+        for li in range(cfg["layers"]):  # the appended (rotated) keys and the values
+            k, v = dec.kv_read(li, pos, 1)
+            assert np.allclose(k[0], kc[li, pos], rtol=1e-5, atol=1e-6)
+            assert np.allclose(v[0], vc[li, pos], rtol=1e-5, atol=1e-6)
+    dec.close()
+
+
+def test_decode_8b_shaped_layer(jn):
+    """One layer at the 8B shape of BASELINE config 5 (d_model 4096, 32/8 heads of 128, FFN 14336, context 512) with a
+    cut-down vocabulary, Q4_K_M mix."""
+    cfg = dict(layers=1, d_model=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, vocab=2048, max_ctx=513, rms_eps=1e-5, rope_theta=5e5)
+    dec, layers, out_norm, out_w = build(jn, cfg, 9)
+    rng = np.random.default_rng(2)
+    kc = np.zeros((1, 513, 8, 128), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :512] = rng.standard_normal((1, 512, 8, 128))
+    vc[:, :512] = rng.standard_normal((1, 512, 8, 128))
+    dec.kv_write(0, 0, kc[0, :512], vc[0, :512])
+    x = rng.standard_normal(4096).astype(np.float32)
+    ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x, 512)
+    y = dec.decode(x, 512)
+    assert norm_err(y, ref) <= 1e-4, norm_err(y, ref)
+    dec.close()
+
+
+def test_decode_argument_checks(jn):
+    cfg = dict(layers=1, d_model=256, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=64, max_ctx=8, rms_eps=1e-5, rope_theta=1e4)
+    dec = jn.LlamaDecoder(**cfg)
+    with pytest.raises(ValueError, match="has no weight"):
+        dec.decode(np.zeros(256, dtype=np.float32), 0)
+    w = jn.Tensor.quantized(jn.DType.Q4_K, np.zeros(144 * 3, dtype=np.uint8), 3, 256)
+    with pytest.raises(ValueError, match="needs shape"):
+        dec.set_weight(0, 0, w)
+    with pytest.raises(ValueError):
+        jn.LlamaDecoder(**{**cfg, "heads": 3})
+    with pytest.raises(ValueError):
+        jn.LlamaDecoder(**{**cfg, "head_dim": 80})
+    dec.close()
