@@ -30,6 +30,9 @@ sys.path.insert(0, str(ROOT))
 sys.path.insert(0, str(ROOT / "tests"))
 
 PEAK_HBM_GBPS = 8000.0
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc (profiles/gemv_q4_k_14336x4096_b1_pmc_traffic.txt):
+# FETCH_SIZE 16234.9 KiB x 2.0 (a 256 MiB copy kernel reads 131087 on this counter) + WRITE_SIZE 112.0 KiB x 1.0
+HEADLINE_TRAFFIC_BYTES = int((16234.9 * 2.0 + 112.0) * 1024)
 BLOCK = {"Q8_0": (8, 32, 34), "Q4_0": (2, 32, 18), "Q4_1": (3, 32, 20), "Q4_K": (12, 256, 144), "Q5_K": (13, 256, 176),
          "Q6_K": (14, 256, 210)}
 
@@ -96,6 +99,22 @@ class Workload:
         t1 = time.perf_counter()
         return t1 - t0, e0.elapsed_time(e1) * 1e-3
 
+    def read_probe(self, steps: int):
+        """Microseconds per launch of a pure 128-bit streaming read over the same weight bytes, rotating like time()."""
+        torch = self.torch
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        ptrs = [(C.c_void_p(t.data_ptr()), t.numel()) for t in self.weights]
+        for i in range(10):
+            self.lib.lib.jitnn_hip_probe_read_dev(ptrs[i % len(ptrs)][0], ptrs[i % len(ptrs)][1], stream)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(steps):
+            self.lib.lib.jitnn_hip_probe_read_dev(ptrs[i % len(ptrs)][0], ptrs[i % len(ptrs)][1], stream)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
     def parity(self, rows: int = 192):
         """Normalised max error of the device result against the CPU oracle on a spread of output rows."""
         import numpy as np
@@ -123,7 +142,9 @@ def measure(torch, lib, fmt, n, k, b, copies, steps, warmup, seed, parity=True):
     wl = Workload(torch, lib, fmt, n, k, b, copies, seed)
     err = wl.parity() if parity else None
     wall, ev = wl.time(steps, warmup)
+    probe_us = wl.read_probe(min(steps, 400))
     out = {"workload": f"{fmt} GEMV {n}x{k} batch {b}", "copies": copies, "steps": steps, "bytes_per_step": wl.bytes,
+           "pure_read_us_per_launch": probe_us, "pure_read_GBps": wl.weights[0].numel() / probe_us / 1e3,
            "us_per_step_wall": wall / steps * 1e6, "us_per_step_events": ev / steps * 1e6, "GBps": wl.bytes * steps / wall / 1e9,
            "GBps_events": wl.bytes * steps / ev / 1e9, "pct_of_peak": wl.bytes * steps / ev / 1e9 / PEAK_HBM_GBPS * 100,
            "parity_norm_err": err}
@@ -152,6 +173,139 @@ def cpu_baseline(wl: Workload, budget_s: float = 12.0):
                       "reference's scalar FP64 host loop (Gguf.MatVec.reference), same weight bytes and activations as the GPU"}
 
 
+def quantized_device_weight(torch, lib, fmt, n, k, seed):
+    """N(0, 0.02) weight [n, k] quantised to fmt on the device; returns the uint8 tensor."""
+    import quantizers
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    parts = []
+    for r0 in range(0, n, 8192):
+        w = torch.randn(min(8192, n - r0), k, generator=g, device="cuda") * 0.02
+        parts.append(quantizers.quantize(fmt, w))
+        del w
+    return torch.cat(parts)
+
+
+def wrap(lib, fmt, t, n, k):
+    h = C.c_void_p()
+    lib.check(lib.lib.jitnn_hip_weight_wrap_dev(BLOCK[fmt][0], C.c_void_p(t.data_ptr()), t.numel(), n, k, C.byref(h)), "wrap")
+    return h
+
+
+def bench_decode(torch, lib, steps, warmup):
+    """BASELINE config 5: 32 layers, d_model 4096, 32/8 heads of 128, FFN 14336, vocab 128256, Q4_K_M mix (Q4_K; Q6_K for
+    attn_v, ffn_down, output), FP32 KV cache pre-filled with N(0,1) at context 512, one token per step.  Every layer
+    has its own copy of the weights in HBM (the values of layer 0 repeated: the step streams 4.9 GB)."""
+    import jitnn_amd
+    cfg = dict(layers=32, d_model=4096, heads=32, kv_heads=8, head_dim=128, ffn=14336, vocab=128256, max_ctx=520, rms_eps=1e-5, rope_theta=5e5)
+    shapes = [("Q4_K", 4096, 4096), ("Q4_K", 1024, 4096), ("Q6_K", 1024, 4096), ("Q4_K", 4096, 4096), ("Q4_K", 14336, 4096),
+              ("Q4_K", 14336, 4096), ("Q6_K", 4096, 14336)]
+    base = [quantized_device_weight(torch, lib, f, n, k, 1050 + i) for i, (f, n, k) in enumerate(shapes)]
+    dec = jitnn_amd.LlamaDecoder(**cfg)
+    keep, handles = [], []
+    weight_bytes = 0
+    for l in range(cfg["layers"]):
+        for i, (f, n, k) in enumerate(shapes):
+            t = base[i] if l == 0 else base[i].clone()
+            keep.append(t)
+            h = wrap(lib, f, t, n, k)
+            handles.append(h)
+            dec.set_weight_handle(l, i, h)
+            weight_bytes += t.numel()
+        dec.set_norm(l, 0, torch.ones(4096).numpy())
+        dec.set_norm(l, 1, torch.ones(4096).numpy())
+    dec.set_norm(0, 2, torch.ones(4096).numpy())
+    head = quantized_device_weight(torch, lib, "Q6_K", cfg["vocab"], 4096, 1049)
+    hh = wrap(lib, "Q6_K", head, cfg["vocab"], 4096)
+    dec.set_weight_handle(0, 7, hh)
+    weight_bytes += head.numel()
+    g = torch.Generator().manual_seed(11)
+    for l in range(cfg["layers"]):
+        dec.kv_write(l, 0, torch.randn(512, 8, 128, generator=g).numpy(), torch.randn(512, 8, 128, generator=g).numpy())
+    x = torch.randn(4096, device="cuda")
+    logits = torch.empty(cfg["vocab"], device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run(n):
+        for _ in range(n):
+            dec.decode_dev(x.data_ptr(), 512, logits.data_ptr(), st)
+
+    run(warmup)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    run(steps)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ok = bool(torch.isfinite(logits).all().item())
+    kv_bytes = 32 * 2 * 513 * 8 * 128 * 4
+    out = {"workload": "Llama-8B-shaped decode step, Q4_K_M mix, context 512, batch 1", "steps": steps, "ms_per_token": wall / steps * 1e3,
+           "ms_per_token_events": e0.elapsed_time(e1) / steps, "tokens_per_s": steps / wall, "bytes_per_token": weight_bytes + kv_bytes,
+           "GBps": (weight_bytes + kv_bytes) * steps / wall / 1e9, "pct_of_peak": (weight_bytes + kv_bytes) * steps / wall / 1e9 / PEAK_HBM_GBPS * 100,
+           "launch": "direct", "logits_finite": ok}
+    # the same step replayed as a HIP graph (no host launch cost per kernel)
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            dec.decode_dev(x.data_ptr(), 512, logits.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        ref = logits.clone()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        gw = time.perf_counter() - t0
+        out["graph_ms_per_token"] = gw / steps * 1e3
+        out["graph_tokens_per_s"] = steps / gw
+        out["graph_matches_direct"] = bool(torch.equal(ref, logits))
+    except Exception as e:  # report, never hide
+        out["graph_error"] = f"{type(e).__name__}: {e}"
+    for h in handles + [hh]:
+        lib.lib.jitnn_hip_weight_free(h)
+    dec.close()
+    return out
+
+
+def bench_prefill(torch, lib, steps=20):
+    """512-token linears through the MFMA path at the layer shapes of config 5: achieved TFLOP/s (2*M*N*K per call)."""
+    res = {}
+    for name, fmt, n, k in (("q4_k_14336x4096", "Q4_K", 14336, 4096), ("q6_k_4096x14336", "Q6_K", 4096, 14336), ("q4_k_4096x4096", "Q4_K", 4096, 4096)):
+        t = quantized_device_weight(torch, lib, fmt, n, k, 1060)
+        h = wrap(lib, fmt, t, n, k)
+        x = torch.randn(512, k, device="cuda")
+        y = torch.empty(512, n, device="cuda")
+        st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        call = lambda: lib.check(lib.lib.jitnn_hip_linear_dev(h, C.c_void_p(x.data_ptr()), 512, None, C.c_void_p(y.data_ptr()), st), "linear")
+        for _ in range(3):
+            call()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        flops = 2.0 * 512 * n * k
+        # parity on a sample of outputs against FP64 on the dequantised weights of a few rows
+        import numpy as np
+        from oracle import oracle
+        sel = np.unique(np.linspace(0, n - 1, 24).astype(np.int64))
+        rb = k // BLOCK[fmt][1] * BLOCK[fmt][2]
+        raw = t.view(n, rb)[torch.as_tensor(sel, device="cuda")].cpu().numpy().reshape(-1)
+        wd = oracle.dequantize(BLOCK[fmt][0], raw, len(sel) * k).reshape(len(sel), k).astype(np.float64)
+        ref = x.cpu().numpy().astype(np.float64) @ wd.T
+        err = float(np.abs(y.cpu().numpy()[:, sel] - ref).max() / np.abs(ref).max())
+        res[name] = {"workload": f"{fmt} linear {n}x{k}, 512 rows (MFMA path)", "ms": ms, "TFLOPs": flops / ms / 1e9,
+                     "pct_of_fp16_peak": flops / ms / 1e9 / 2500.0 * 100, "parity_norm_err": err}
+        lib.lib.jitnn_hip_weight_free(h)
+        del t, x, y
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -160,6 +314,9 @@ def main() -> int:
     ap.add_argument("--quick", action="store_true", help="headline workload only (no other configs, short CPU baseline)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma list of extra configs to run (default all)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device-to-device copy kernel (known traffic: 256 MiB read, 256 MiB written) so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command can scale its counters")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this build measures one GPU (the path has no cross-GPU work); --gpus {a.gpus} is not supported", file=sys.stderr)
@@ -174,6 +331,14 @@ def main() -> int:
     jitnn_amd.init(0)
     info = jitnn_amd.device_info()
 
+    if a.calibrate_copy:
+        src = torch.empty(64 << 20, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- headline: Q4_K 14336x4096 batch 1, rotating over 16 copies
     wl, head = measure(torch, lib, "Q4_K", 14336, 4096, 1, 16, a.steps, a.warmup, seed=1030)
     hot_wall, hot_ev = wl.time(min(a.steps, 2000), 50, rotate=False)
@@ -182,6 +347,7 @@ def main() -> int:
     wl.close()
 
     configs = {}
+    only = set(filter(None, a.only.split(",")))
     if not a.quick:
         extra = [
             ("q8_0_4096x4096_b1", "Q8_0", 4096, 4096, 1, 24, 1010),
@@ -191,7 +357,6 @@ def main() -> int:
             ("q4_k_14336x4096_b8", "Q4_K", 14336, 4096, 8, 16, 1030),
             ("q6_k_128256x4096_b1", "Q6_K", 128256, 4096, 1, 2, 1040),
         ]
-        only = set(filter(None, a.only.split(",")))
         for name, fmt, n, k, b, copies, seed in extra:
             if only and name not in only:
                 continue
@@ -199,6 +364,13 @@ def main() -> int:
             w2, out = measure(torch, lib, fmt, n, k, b, copies, steps, 20, seed)
             w2.close()
             configs[name] = out
+
+    decode = prefill = None
+    if not a.quick:
+        if not only or "decode" in only:
+            decode = bench_decode(torch, lib, steps=30, warmup=3)
+        if not only or "prefill" in only:
+            prefill = bench_prefill(torch, lib)
 
     ms = head["us_per_step_wall"] / 1e3
     line = {
@@ -218,12 +390,15 @@ def main() -> int:
         "config": {"workload": "Q4_K GEMV 14336x4096 batch 1 (BASELINE configs[2]), weights N(0,0.02) quantised to Q4_K, x N(0,1); "
                                "16 weight copies rotated per step (528 MB > 256 MB Infinity Cache)",
                    "bytes_per_step": head_bytes, "device": info["name"], "compute_units": info["compute_units"],
-                   "cache_resident_GBps": head_bytes * min(a.steps, 2000) / hot_ev / 1e9, "parity_norm_err": head["parity_norm_err"]},
+                   "cache_resident_GBps": head_bytes * min(a.steps, 2000) / hot_ev / 1e9, "parity_norm_err": head["parity_norm_err"],
+                   "pure_read_GBps": head["pure_read_GBps"], "pure_read_us_per_launch": head["pure_read_us_per_launch"]},
         "roofline": {"bound": "hbm", "achieved": head["GBps_events"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                     "frac": head["GBps_events"] / PEAK_HBM_GBPS, "traffic": None,
+                     "frac": head["GBps_events"] / PEAK_HBM_GBPS, "traffic": HEADLINE_TRAFFIC_BYTES,
                      "kernel": "gemv Q4_K batch 1", "us_per_launch": head["us_per_step_events"]},
         "cpu_baseline": cpu,
         "configs": configs,
+        "decode": decode,
+        "prefill": prefill,
     }
     print(json.dumps(line))
     return 0

@@ -113,6 +113,13 @@ JITNN_HIP_API int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x
 JITNN_HIP_API int jitnn_hip_quantize_q8_0(const float *x_host, long long numel, void *blocks_host);
 JITNN_HIP_API int jitnn_hip_quantize_q8_0_dev(const float *x_dev, long long numel, void *blocks_dev, void *stream);
 
+/* ---- measurement aid ---------------------------------------------------------------------------- */
+
+/* Streams nbytes of device memory through 128-bit loads and nothing else (the result is discarded): what the
+ * device gives a pure read of the same bytes, launch included.  The benchmark prints it beside the GEMV figures;
+ * it has no counterpart in the reference. */
+JITNN_HIP_API int jitnn_hip_probe_read_dev(const void *dev, long long nbytes, void *stream);
+
 /* ---- device memory for callers that have no HIP binding of their own (the Java side) ------------- */
 
 JITNN_HIP_API int jitnn_hip_malloc(long long nbytes, void **dev);

@@ -75,6 +75,20 @@ __global__ void fp8_probe_kernel(float *out) {
     out[1] = p.y;
 }
 
+// Pure streaming read: every thread xors the 16-byte words it loads; the store can never happen for real data
+// but keeps the loads alive.
+__global__ void __launch_bounds__(256) probe_read_kernel(const u32x4 *__restrict__ p, size_t n16, uint32_t *sink) {
+    const size_t stride = (size_t)gridDim.x * 256;
+    u32x4 acc = {0, 0, 0, 0};
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    for (; i + 3 * stride < n16; i += 4 * stride) {
+        const u32x4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], d = p[i + 3 * stride];
+        acc ^= a ^ b ^ c ^ d;
+    }
+    for (; i < n16; i += stride) acc ^= p[i];
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) *sink = acc.x;
+}
+
 bool known(int fmt) { return block_values(fmt) != 0; }
 
 // Kernels that want more than 64 KiB of dynamic LDS must be told so once; remembered per kernel so that steady-state
@@ -556,6 +570,14 @@ int jitnn_hip_quantize_q8_0(const float *x_host, long long numel, void *blocks_h
     }
     (void)hipFree(buf);
     return rc;
+}
+
+int jitnn_hip_probe_read_dev(const void *dev, long long nbytes, void *stream) {
+    if (!dev || nbytes < 16 || ((uintptr_t)dev & 15) != 0) return fail(JITNN_HIP_EINVAL, "need a 16-byte aligned buffer of at least 16 bytes");
+    if (int rc = check_ready()) return rc;
+    hipLaunchKernelGGL(probe_read_kernel, dim3(g.cus * 2), dim3(256), 0, (hipStream_t)stream, (const u32x4 *)dev, (size_t)nbytes / 16, (uint32_t *)nullptr);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
 }
 
 int jitnn_hip_malloc(long long nbytes, void **dev) {
