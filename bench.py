@@ -314,6 +314,7 @@ def main() -> int:
     ap.add_argument("--quick", action="store_true", help="headline workload only (no other configs, short CPU baseline)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="comma list of extra configs to run (default all)")
+    ap.add_argument("--decode", action="store_true", help="with --quick: still run the decode-step leg")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device-to-device copy kernel (known traffic: 256 MiB read, 256 MiB written) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command can scale its counters")
@@ -366,10 +367,10 @@ def main() -> int:
             configs[name] = out
 
     decode = prefill = None
-    if not a.quick:
+    if not a.quick or a.decode:
         if not only or "decode" in only:
             decode = bench_decode(torch, lib, steps=30, warmup=3)
-        if not only or "prefill" in only:
+        if (not only or "prefill" in only) and not a.quick:
             prefill = bench_prefill(torch, lib)
 
     ms = head["us_per_step_wall"] / 1e3

@@ -627,16 +627,38 @@ struct UnitPair<F_Q8_0> {
 // The first rows' loads are issued before the staging barrier, so HBM latency overlaps the staging too.
 constexpr int XREG_THREADS = 256;  // workgroup size of gemv_xreg_kernel (compile-time: the staging is fully unrolled)
 
-template <class U, int CV, int PF, bool BIAS>
-__global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
-                                                         const float *__restrict__ bias, float *__restrict__ y, int n, int k, float nib) {
+// Arguments of gemv_xreg_kernel.  Up to three matrices of the same format and row length share one launch and
+// one activation vector (the q and k projections of a decode step): their rows are numbered one after the other.
+struct XregArgs {
+    const uint8_t *w[3];   // row segments: n[i] rows each, all [*, k] in the kernel's format
+    float *y[3];           // outputs of the segments
+    const float *bias[3];  // BIAS: added to the segment's rows (a residual rides here), else ignored
+    int n[3];
+    const uint8_t *w2;     // DUAL: second matrix of the shape of w[0]; the kernel writes silu(w[0] x) * (w2 x) to y[0]
+    const float *x;        // [k]
+    const float *nw;       // NORM: RMSNorm weight [k]; the kernel multiplies x by nw / sqrt(mean(x^2) + eps) while staging it
+    float eps;
+    int k;
+    float nib;
+};
+
+// Extra template switches:
+//   NORM  fuses the RMSNorm that precedes the linear (ops/RowNorm.java:286-306) into the staging of x;
+//   DUAL  computes the SwiGLU gate of a Llama FFN (F.swiglu, F.java:1159-1161) from two matrices in one pass: the
+//         ring alternates rows of w[0] (gate) and w2 (up), so NB = PF + 1 must be even.
+template <class U, int CV, int PF, bool BIAS, bool NORM, bool DUAL>
+__global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const XregArgs a) {
     constexpr int FMT = U::FMT, STEPS = 64 / U::UV;  // a lane keeps 64 activations: one 64-value unit or two of 32
     constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG, NB = PF + 1;
+    static_assert(!DUAL || NB % 2 == 0, "gate and up rows alternate in the ring");
+    constexpr int RSTEP = DUAL ? NB / 2 : NB;  // rows a full turn of the ring advances
     __shared__ float4 xl[STEPS * 64 * (UQ + 1)];
     __shared__ float sums[STEPS * 64 * NS];
+    __shared__ float red[XREG_THREADS / 64];
     constexpr int nwaves = XREG_THREADS / 64;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: row numbers, row pointers and the loop run on the SALU
+    const int k = a.k, n = a.n[0] + a.n[1] + a.n[2];
     const int units = k / U::UV;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
     const int stride = gridDim.x * nwaves;
@@ -648,11 +670,19 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *
         uc[s] = min(s * 64 + lane, units - 1);  // lanes past the row end: last unit, zeroed x
         U::offsets(uc[s], off[s]);
     }
-    // loads of buffer b for row r; a row past the end is "loaded" from the first bytes of the matrix by every lane
-    // (one cache line, no traffic) so that the number of loads in flight never depends on the data
-    auto fill = [&](typename U::Raw(&dst)[STEPS], float &bdst, int r) {
+    // segment and local row of global row r (scalar)
+    auto locate = [&](int r, int &seg, int &local) {
+        seg = (r >= a.n[0]) + (r >= a.n[0] + a.n[1]);
+        local = r - (seg > 0 ? a.n[0] : 0) - (seg > 1 ? a.n[1] : 0);
+    };
+    // loads of a buffer for row r of matrix `second ? w2 : w[seg]`; a row past the end is "loaded" from the first bytes
+    // of the matrix by every lane (one cache line, no traffic) so that the number of loads in flight never depends on
+    // the data
+    auto fill = [&](typename U::Raw(&dst)[STEPS], float &bdst, int r, bool second) {
         const bool live = r < n;
-        const uint8_t *rp = W + (live ? (size_t)r * rowbytes : 0);
+        int seg = 0, local = 0;
+        if (live) locate(r, seg, local);
+        const uint8_t *rp = (DUAL && second ? a.w2 : a.w[seg]) + (size_t)local * rowbytes;
 #pragma unroll
         for (int s = 0; s < STEPS; ++s) {
             uint32_t o[U::NOFF];
@@ -660,20 +690,21 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *
             for (int i = 0; i < U::NOFF; ++i) o[i] = live ? off[s][i] : 0u;
             U::load(dst[s], rp, o);
         }
-        if (BIAS) bdst = bias[live ? r : 0];
+        if (BIAS) bdst = a.bias[seg][local];
     };
 
     // ---- activations first: their loads (L2 hits) are issued ahead of the weight loads because the hardware counts
     // returning loads in order - waiting for x must not mean waiting for the first weight rows from HBM
     constexpr int QUADS = STEPS * 64 * UQ, PER = QUADS / XREG_THREADS;
     static_assert(QUADS % XREG_THREADS == 0, "whole passes");
-    float4 xv[PER];
+    float4 xv[PER], nv[PER];
     {
         const int kq = k >> 2;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             const int f = tid + i * XREG_THREADS;
-            xv[i] = f < kq ? reinterpret_cast<const float4 *>(x)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+            xv[i] = f < kq ? reinterpret_cast<const float4 *>(a.x)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (NORM) nv[i] = f < kq ? reinterpret_cast<const float4 *>(a.nw)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
     typename U::Raw buf[NB][STEPS];
@@ -681,7 +712,19 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         bv[b] = 0.f;
-        fill(buf[b], bv[b], row0 + b * stride);
+        fill(buf[b], bv[b], row0 + (DUAL ? b / 2 : b) * stride, DUAL && (b & 1));
+    }
+    if (NORM) {  // x <- x * nw / sqrt(mean(x^2) + eps): every workgroup normalises the whole vector for itself
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        const float is = 1.f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)k + a.eps);
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            xv[i] = make_float4(xv[i].x * is * nv[i].x, xv[i].y * is * nv[i].y, xv[i].z * is * nv[i].z, xv[i].w * is * nv[i].w);
     }
     // ---- stage x (and the partial sums) in unit order
 #pragma unroll
@@ -703,21 +746,29 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const uint8_t *
         for (int i = 0; i < NS; ++i) xs[s].sm[i] = sums[(s * 64 + lane) * NS + i];
     }
 
-    for (int base = row0; base < n; base += NB * stride) {
+    float gate = 0.f;  // DUAL: the gate row's result, held until the up row of the same index is done
+    for (int base = row0; base < n; base += RSTEP * stride) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-            const int row = base + b * stride;
+            const int row = base + (DUAL ? b / 2 : b) * stride;
             if (row < n) {  // wave-uniform
                 float acc[1][1] = {{0.f}};
 #pragma unroll
                 for (int s = 0; s < STEPS; ++s) {
                     const typename U::Raw(&w1)[1] = reinterpret_cast<const typename U::Raw(&)[1]>(buf[b][s]);
-                    U::template dot<1, 1, CV>(w1, uc[s], xs[s], acc, nib);
+                    U::template dot<1, 1, CV>(w1, uc[s], xs[s], acc, a.nib);
                 }
-                float t = wave_sum(acc[0][0]);
-                if (lane == 0) y[row] = BIAS ? t + bv[b] : t;
+                const float t = wave_sum(acc[0][0]);
+                if (DUAL) {
+                    if ((b & 1) == 0) gate = t;
+                    else if (lane == 0) a.y[0][row] = (gate / (1.f + __expf(-gate))) * t;
+                } else {
+                    int seg, local;
+                    locate(row, seg, local);
+                    if (lane == 0) a.y[seg][local] = BIAS ? t + bv[b] : t;
+                }
             }
-            fill(buf[b], bv[b], row + NB * stride);
+            fill(buf[b], bv[b], row + RSTEP * stride, DUAL && (b & 1));
         }
     }
 }

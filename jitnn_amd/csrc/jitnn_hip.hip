@@ -150,40 +150,85 @@ GemvVariant pick(int fmt, int rows) {
 int unit_values(int fmt) { return block_values(fmt) == 256 ? 64 : 32; }
 
 typedef void (*gemv1_fn)(const uint8_t *, const float *, const float *, float *, int, int, float);
+typedef void (*xreg_fn)(const XregArgs);
 
 // The 32-value formats decode pairs of blocks when the row holds an even number of them (aligned loads),
 // single blocks otherwise.
-template <int PF, bool BIAS>
-gemv1_fn pick_xreg_pf(int fmt, bool pairs) {
+template <int PF, bool BIAS, bool NORM, bool DUAL>
+xreg_fn pick_xreg_fmt(int fmt, bool pairs) {
     switch (fmt) {
-    case F_Q4_0: return pairs ? gemv_xreg_kernel<UnitPair<F_Q4_0>, 1, PF, BIAS> : gemv_xreg_kernel<Unit<F_Q4_0>, 1, PF, BIAS>;
-    case F_Q4_1: return pairs ? gemv_xreg_kernel<UnitPair<F_Q4_1>, 1, PF, BIAS> : gemv_xreg_kernel<Unit<F_Q4_1>, 1, PF, BIAS>;
-    case F_Q8_0: return pairs ? gemv_xreg_kernel<UnitPair<F_Q8_0>, 0, PF, BIAS> : gemv_xreg_kernel<Unit<F_Q8_0>, 0, PF, BIAS>;
-    case F_Q4_K: return gemv_xreg_kernel<Unit<F_Q4_K>, 1, PF, BIAS>;
-    case F_Q5_K: return gemv_xreg_kernel<Unit<F_Q5_K>, 0, PF, BIAS>;
-    default: return gemv_xreg_kernel<Unit<F_Q6_K>, 0, PF, BIAS>;
+    case F_Q4_0:
+        return pairs ? gemv_xreg_kernel<UnitPair<F_Q4_0>, 1, PF, BIAS, NORM, DUAL> : gemv_xreg_kernel<Unit<F_Q4_0>, 1, PF, BIAS, NORM, DUAL>;
+    case F_Q4_1:
+        return pairs ? gemv_xreg_kernel<UnitPair<F_Q4_1>, 1, PF, BIAS, NORM, DUAL> : gemv_xreg_kernel<Unit<F_Q4_1>, 1, PF, BIAS, NORM, DUAL>;
+    case F_Q8_0:
+        return pairs ? gemv_xreg_kernel<UnitPair<F_Q8_0>, 0, PF, BIAS, NORM, DUAL> : gemv_xreg_kernel<Unit<F_Q8_0>, 0, PF, BIAS, NORM, DUAL>;
+    case F_Q4_K: return gemv_xreg_kernel<Unit<F_Q4_K>, 1, PF, BIAS, NORM, DUAL>;
+    case F_Q5_K: return gemv_xreg_kernel<Unit<F_Q5_K>, 0, PF, BIAS, NORM, DUAL>;
+    default: return gemv_xreg_kernel<Unit<F_Q6_K>, 0, PF, BIAS, NORM, DUAL>;
     }
 }
 
-gemv1_fn pick_xreg(int fmt, bool pairs, bool bias, int pf) {
-    if (pf == 1) return bias ? pick_xreg_pf<1, true>(fmt, pairs) : pick_xreg_pf<1, false>(fmt, pairs);
-    return bias ? pick_xreg_pf<2, true>(fmt, pairs) : pick_xreg_pf<2, false>(fmt, pairs);
+// mode 0: plain; 1: with bias; 2: with fused RMSNorm; 3: fused RMSNorm + SwiGLU pair (PF 1 or 3)
+xreg_fn pick_xreg(int fmt, bool pairs, int mode, int pf) {
+    switch (mode) {
+    case 1: return pf == 1 ? pick_xreg_fmt<1, true, false, false>(fmt, pairs) : pick_xreg_fmt<2, true, false, false>(fmt, pairs);
+    case 2: return pf == 1 ? pick_xreg_fmt<1, false, true, false>(fmt, pairs) : pick_xreg_fmt<2, false, true, false>(fmt, pairs);
+    case 3: return pf == 1 ? pick_xreg_fmt<1, false, true, true>(fmt, pairs) : pick_xreg_fmt<3, false, true, true>(fmt, pairs);
+    default: return pf == 1 ? pick_xreg_fmt<1, false, false, false>(fmt, pairs) : pick_xreg_fmt<2, false, false, false>(fmt, pairs);
+    }
 }
 
-// Batch 1, rows of at most 4096 values: activations in registers, one row per wave iteration.
-int launch_gemv_xreg(const jitnn_hip_weight *w, const float *x, const float *bias, float *y, hipStream_t stream) {
+// One launch of the register-resident batch-1 kernel (rows of at most 4096 values) over up to three matrices of one
+// format and row length.  norm_w != NULL fuses the RMSNorm of x; w2 != NULL computes silu(w x) * (w2 x).
+struct XregCall {
+    const jitnn_hip_weight *w[3] = {nullptr, nullptr, nullptr};
+    float *y[3] = {nullptr, nullptr, nullptr};
+    const float *bias = nullptr;  // for w[0] only
+    const jitnn_hip_weight *w2 = nullptr;
+    const float *x = nullptr, *norm_w = nullptr;
+    float eps = 0.f;
+};
+
+int launch_xreg(const XregCall &c, hipStream_t stream) {
+    XregArgs a{};
+    int n = 0;
+    for (int i = 0; i < 3; ++i) {
+        a.w[i] = c.w[i] ? c.w[i]->dev : c.w[0]->dev;
+        a.y[i] = c.y[i] ? c.y[i] : c.y[0];
+        a.bias[i] = c.bias;
+        a.n[i] = c.w[i] ? c.w[i]->n : 0;
+        n += a.n[i];
+    }
+    a.w2 = c.w2 ? c.w2->dev : nullptr;
+    a.x = c.x;
+    a.nw = c.norm_w;
+    a.eps = c.eps;
+    a.k = c.w[0]->k;
+    a.nib = g.nib;
     const int threads = XREG_THREADS, waves = threads / 64;
-    int blocks = (w->n + waves - 1) / waves;
+    int blocks = (n + waves - 1) / waves;
     // Two workgroups (eight waves) per CU measured best for streaming: fewer, longer row streams keep HBM pages
     // open.  A wave that sees many rows needs one row of prefetch; when it sees only a handful (a 14336-row
     // matrix gives a wave seven rows) a second row in flight covers the start-up latency.
     const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : 2);
     if (blocks > cap) blocks = cap;
-    const int rows_per_wave = (w->n + blocks * waves - 1) / (blocks * waves);
+    const int rows_per_wave = (n + blocks * waves - 1) / (blocks * waves);
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
-    hipLaunchKernelGGL(pick_xreg(w->fmt, w->k % 64 == 0, bias != nullptr, pf), dim3(blocks), dim3(threads), 0, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
+    const int mode = c.w2 ? 3 : c.norm_w ? 2 : c.bias ? 1 : 0;
+    hipLaunchKernelGGL(pick_xreg(c.w[0]->fmt, a.k % 64 == 0, mode, pf), dim3(blocks), dim3(threads), 0, stream, a);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
+}
+
+// Batch 1, rows of at most 4096 values: activations in registers, one row per wave iteration.
+int launch_gemv_xreg(const jitnn_hip_weight *w, const float *x, const float *bias, float *y, hipStream_t stream) {
+    XregCall c;
+    c.w[0] = w;
+    c.y[0] = y;
+    c.bias = bias;
+    c.x = x;
+    return launch_xreg(c, stream);
 }
 
 template <int PF>
@@ -628,12 +673,46 @@ struct jitnn_hip_llama {
 namespace {
 
 template <int D>
-void launch_attention(const jitnn_hip_llama *m, int layer, int s, hipStream_t st) {
-    const int chunks = (s + ATT_CH - 1) / ATT_CH;
+void launch_attention(const jitnn_hip_llama *m, int layer, int pos, hipStream_t st) {
+    const int chunks = (pos + 1 + AttCfg<D>::CH - 1) / AttCfg<D>::CH;
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
-    hipLaunchKernelGGL(attn_partial_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->kc + lo, m->vc + lo, m->part, m->heads, m->kv, s,
-                       1.0f / sqrtf((float)D));
-    hipLaunchKernelGGL(attn_combine_kernel<D>, dim3(m->heads), dim3(64), 0, st, m->part, m->att, chunks);
+    hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->k, m->v, m->kc + lo, m->vc + lo, m->cosv, m->sinv,
+                       m->part, m->heads, m->kv, pos, 1.0f / sqrtf((float)D));
+    hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(m->heads), dim3(D), 0, st, m->part, m->att, chunks);
+}
+
+bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !g.force_lds; }
+
+// y_i = W_i RMSNorm(x; nw) for `count` (at most 3) weights over the same x.  Weights the register-resident kernel
+// takes get the norm fused into their launch, neighbours of one format share the launch; anything else goes through
+// a separate RMSNorm and the general GEMV.
+int normed_linears(const jitnn_hip_llama *m, const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, const float *nw,
+                   hipStream_t st) {
+    bool normed = false;
+    for (int i = 0; i < count;) {
+        if (xreg_ok(ws[i])) {
+            XregCall c;
+            int j = 0;
+            while (i + j < count && j < 3 && xreg_ok(ws[i + j]) && ws[i + j]->fmt == ws[i]->fmt && ws[i + j]->k == ws[i]->k) {
+                c.w[j] = ws[i + j];
+                c.y[j] = ys[i + j];
+                ++j;
+            }
+            c.x = x;
+            c.norm_w = nw;
+            c.eps = m->eps;
+            if (int rc = launch_xreg(c, st)) return rc;
+            i += j;
+        } else {
+            if (!normed) {
+                hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, x, nw, m->xn, m->d, m->eps);
+                normed = true;
+            }
+            if (int rc = launch_gemv(ws[i], m->xn, 1, nullptr, ys[i], st)) return rc;
+            ++i;
+        }
+    }
+    return JITNN_HIP_OK;
 }
 
 int check_model(const jitnn_hip_llama *m) {
@@ -656,6 +735,7 @@ int jitnn_hip_llama_create(int layers, int d_model, int heads, int kv_heads, int
     if (layers < 1 || d_model < 1 || heads < 1 || kv_heads < 1 || ffn < 1 || vocab < 1 || max_ctx < 1)
         return fail(JITNN_HIP_EINVAL, "non-positive model dimension");
     if (heads % kv_heads != 0) return fail(JITNN_HIP_EINVAL, "grouped-query attention: %d query heads over %d key/value heads", heads, kv_heads);
+    if (heads / kv_heads > ATT_GMAX) return fail(JITNN_HIP_EINVAL, "%d query heads per key/value head (at most %d are built)", heads / kv_heads, ATT_GMAX);
     if (head_dim != 64 && head_dim != 128 && head_dim != 192 && head_dim != 256)
         return fail(JITNN_HIP_EINVAL, "head_dim %d (64, 128, 192 and 256 are built)", head_dim);
     if (int rc = check_ready()) return rc;
@@ -665,7 +745,7 @@ int jitnn_hip_llama_create(int layers, int d_model, int heads, int kv_heads, int
     m->layers = layers; m->d = d_model; m->heads = heads; m->kv = kv_heads; m->hd = head_dim; m->ffn = ffn; m->vocab = vocab;
     m->max_ctx = max_ctx; m->eps = rms_eps; m->theta = rope_theta;
     m->w = new (std::nothrow) const jitnn_hip_weight *[(size_t)layers * 7]();
-    m->chunks_max = (max_ctx + ATT_CH - 1) / ATT_CH;
+    m->chunks_max = (max_ctx + 15) / 16;  // the smallest key chunk any head size uses
     const size_t cache = (size_t)layers * max_ctx * kv_heads * head_dim;
     const int qd = heads * head_dim, kd = kv_heads * head_dim, half = head_dim / 2;
     struct { float **p; size_t n; } bufs[] = {
@@ -777,30 +857,45 @@ int jitnn_hip_llama_decode_dev(jitnn_hip_llama *m, const float *x_dev, int pos, 
     for (int l = 0; l < m->layers; ++l) {
         const jitnn_hip_weight *const *w = m->w + (size_t)l * 7;
         const float *nw = m->norms + (size_t)l * 2 * d;
-        hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, x, nw, m->xn, d, m->eps);
-        if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_Q], m->xn, 1, nullptr, m->q, st)) return rc;
-        if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_K], m->xn, 1, nullptr, m->k, st)) return rc;
-        if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_V], m->xn, 1, nullptr, m->v, st)) return rc;
-        const size_t lo = (size_t)l * m->max_ctx * m->kv * m->hd;
-        hipLaunchKernelGGL(rope_append_kernel, dim3(8), dim3(256), 0, st, m->q, m->k, m->v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads,
-                           m->kv, m->hd, pos);
-        switch (m->hd) {
-        case 64: launch_attention<64>(m, l, pos + 1, st); break;
-        case 128: launch_attention<128>(m, l, pos + 1, st); break;
-        case 192: launch_attention<192>(m, l, pos + 1, st); break;
-        default: launch_attention<256>(m, l, pos + 1, st); break;
+        // q, k, v = W (RMSNorm x): the norm is fused into the linears; projections of one format share a launch
+        {
+            const jitnn_hip_weight *ws[3] = {w[JITNN_HIP_W_ATTN_Q], w[JITNN_HIP_W_ATTN_K], w[JITNN_HIP_W_ATTN_V]};
+            float *ys[3] = {m->q, m->k, m->v};
+            if (int rc = normed_linears(m, ws, ys, 3, x, nw, st)) return rc;
+        }
+        switch (m->hd) {  // RoPE, cache append and attention per key chunk, then the merge of the chunks
+        case 64: launch_attention<64>(m, l, pos, st); break;
+        case 128: launch_attention<128>(m, l, pos, st); break;
+        case 192: launch_attention<192>(m, l, pos, st); break;
+        default: launch_attention<256>(m, l, pos, st); break;
         }
         // xa = x + Wo att, xb = xa + W2 h: the residual rides in the linear's bias slot
         if (int rc = launch_gemv(w[JITNN_HIP_W_ATTN_O], m->att, 1, x, m->xa, st)) return rc;
-        hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, m->xa, nw + d, m->xn, d, m->eps);
-        if (int rc = launch_gemv(w[JITNN_HIP_W_FFN_GATE], m->xn, 1, nullptr, m->gate, st)) return rc;
-        if (int rc = launch_gemv(w[JITNN_HIP_W_FFN_UP], m->xn, 1, nullptr, m->up, st)) return rc;
-        hipLaunchKernelGGL(swiglu_kernel, dim3((m->ffn + 1023) / 1024), dim3(256), 0, st, m->gate, m->up, m->h, m->ffn);
+        // h = silu(W1 n) * (W3 n), n = RMSNorm(xa): one launch when gate and up share a format
+        const jitnn_hip_weight *wg = w[JITNN_HIP_W_FFN_GATE], *wu = w[JITNN_HIP_W_FFN_UP];
+        if (xreg_ok(wg) && wg->fmt == wu->fmt) {
+            XregCall c;
+            c.w[0] = wg;
+            c.w2 = wu;
+            c.y[0] = m->h;
+            c.x = m->xa;
+            c.norm_w = nw + d;
+            c.eps = m->eps;
+            if (int rc = launch_xreg(c, st)) return rc;
+        } else {
+            const jitnn_hip_weight *ws[2] = {wg, wu};
+            float *ys[2] = {m->gate, m->up};
+            if (int rc = normed_linears(m, ws, ys, 2, m->xa, nw + d, st)) return rc;
+            hipLaunchKernelGGL(swiglu_kernel, dim3((m->ffn + 1023) / 1024), dim3(256), 0, st, m->gate, m->up, m->h, m->ffn);
+        }
         if (int rc = launch_gemv(w[JITNN_HIP_W_FFN_DOWN], m->h, 1, m->xa, m->xb, st)) return rc;
         x = m->xb;
     }
-    hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, x, m->norms + (size_t)m->layers * 2 * d, m->xn, d, m->eps);
-    if (int rc = launch_gemv(m->w_out, m->xn, 1, nullptr, logits_dev, st)) return rc;
+    {
+        const jitnn_hip_weight *ws[1] = {m->w_out};
+        float *ys[1] = {logits_dev};
+        if (int rc = normed_linears(m, ws, ys, 1, x, m->norms + (size_t)m->layers * 2 * d, st)) return rc;
+    }
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
