@@ -102,22 +102,22 @@ struct Unit<F_Q4_K> {
             for (int b = 0; b < B; ++b) sl[r][b] = sh[r][b] = 0.f;
 #pragma unroll
         for (int d = 0; d < 8; ++d) {
-            float4 xa[B], xb[B];
-#pragma unroll
-            for (int b = 0; b < B; ++b) {
-                xa[b] = xs.q(b, d);
-                xb[b] = xs.q(b, d + 8);
-            }
+            // decode the step's nibbles of every row first, then walk the batch rows: one pair of activation quads
+            // is live at a time, whatever the batch size
+            float lo[R][4], hi[R][4];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                uint32_t v = d < 4 ? w[r].q0[d & 3] : w[r].q1[d & 3];
-                float l0, l1, l2, l3, h0, h1, h2, h3;
-                cvt4<CV>(v & 0x0f0f0f0fu, l0, l1, l2, l3);
-                cvt4<CV>((v >> 4) & 0x0f0f0f0fu, h0, h1, h2, h3);
+                const uint32_t v = d < 4 ? w[r].q0[d & 3] : w[r].q1[d & 3];
+                cvt4<CV>(v & 0x0f0f0f0fu, lo[r][0], lo[r][1], lo[r][2], lo[r][3]);
+                cvt4<CV>((v >> 4) & 0x0f0f0f0fu, hi[r][0], hi[r][1], hi[r][2], hi[r][3]);
+            }
 #pragma unroll
-                for (int b = 0; b < B; ++b) {
-                    sl[r][b] = dot4(l0, l1, l2, l3, xa[b], sl[r][b]);
-                    sh[r][b] = dot4(h0, h1, h2, h3, xb[b], sh[r][b]);
+            for (int b = 0; b < B; ++b) {
+                const float4 xa = xs.q(b, d), xb = xs.q(b, d + 8);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    sl[r][b] = dot4(lo[r][0], lo[r][1], lo[r][2], lo[r][3], xa, sl[r][b]);
+                    sh[r][b] = dot4(hi[r][0], hi[r][1], hi[r][2], hi[r][3], xb, sh[r][b]);
                 }
             }
         }
@@ -171,22 +171,21 @@ struct Unit<F_Q5_K> {
             for (int b = 0; b < B; ++b) sl[r][b] = sh[r][b] = 0.f;
 #pragma unroll
         for (int d = 0; d < 8; ++d) {
-            float4 xa[B], xb[B];
-#pragma unroll
-            for (int b = 0; b < B; ++b) {
-                xa[b] = xs.q(b, d);
-                xb[b] = xs.q(b, d + 8);
-            }
+            uint32_t lo[R], hi[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                uint32_t v = d < 4 ? w[r].q0[d & 3] : w[r].q1[d & 3];
-                uint32_t t = (d < 4 ? w[r].qh0[d & 3] : w[r].qh1[d & 3]) >> j2;
-                uint32_t lo = (v & 0x0f0f0f0fu) | ((t << 4) & 0x10101010u);
-                uint32_t hi = ((v >> 4) & 0x0f0f0f0fu) | ((t << 3) & 0x10101010u);
+                const uint32_t v = d < 4 ? w[r].q0[d & 3] : w[r].q1[d & 3];
+                const uint32_t t = (d < 4 ? w[r].qh0[d & 3] : w[r].qh1[d & 3]) >> j2;
+                lo[r] = (v & 0x0f0f0f0fu) | ((t << 4) & 0x10101010u);
+                hi[r] = ((v >> 4) & 0x0f0f0f0fu) | ((t << 3) & 0x10101010u);
+            }
 #pragma unroll
-                for (int b = 0; b < B; ++b) {
-                    sl[r][b] = dot4(ub0(lo), ub1(lo), ub2(lo), ub3(lo), xa[b], sl[r][b]);
-                    sh[r][b] = dot4(ub0(hi), ub1(hi), ub2(hi), ub3(hi), xb[b], sh[r][b]);
+            for (int b = 0; b < B; ++b) {
+                const float4 xa = xs.q(b, d), xb = xs.q(b, d + 8);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    sl[r][b] = dot4(ub0(lo[r]), ub1(lo[r]), ub2(lo[r]), ub3(lo[r]), xa, sl[r][b]);
+                    sh[r][b] = dot4(ub0(hi[r]), ub1(hi[r]), ub2(hi[r]), ub3(hi[r]), xb, sh[r][b]);
                 }
             }
         }
@@ -253,27 +252,24 @@ struct Unit<F_Q6_K> {
                 for (int k = 0; k < 4; ++k) s[r][b][k] = 0.f;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            float4 x0[B], x1[B], x2[B], x3[B];
-#pragma unroll
-            for (int b = 0; b < B; ++b) {
-                x0[b] = xs.q(b, p);
-                x1[b] = xs.q(b, 4 + p);
-                x2[b] = xs.q(b, 8 + p);
-                x3[b] = xs.q(b, 12 + p);
-            }
+            uint32_t q0[R], q1[R], q2[R], q3[R];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                uint32_t a = w[r].ql0[p], c = w[r].ql1[p], h = w[r].qh[p];
-                uint32_t q0 = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
-                uint32_t q1 = (c & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
-                uint32_t q2 = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
-                uint32_t q3 = ((c >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
+                const uint32_t a = w[r].ql0[p], c = w[r].ql1[p], h = w[r].qh[p];
+                q0[r] = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
+                q1[r] = (c & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
+                q2[r] = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
+                q3[r] = ((c >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
+            }
 #pragma unroll
-                for (int b = 0; b < B; ++b) {
-                    s[r][b][0] = dot4(ub0(q0), ub1(q0), ub2(q0), ub3(q0), x0[b], s[r][b][0]);
-                    s[r][b][1] = dot4(ub0(q1), ub1(q1), ub2(q1), ub3(q1), x1[b], s[r][b][1]);
-                    s[r][b][2] = dot4(ub0(q2), ub1(q2), ub2(q2), ub3(q2), x2[b], s[r][b][2]);
-                    s[r][b][3] = dot4(ub0(q3), ub1(q3), ub2(q3), ub3(q3), x3[b], s[r][b][3]);
+            for (int b = 0; b < B; ++b) {
+                const float4 x0 = xs.q(b, p), x1 = xs.q(b, 4 + p), x2 = xs.q(b, 8 + p), x3 = xs.q(b, 12 + p);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    s[r][b][0] = dot4(ub0(q0[r]), ub1(q0[r]), ub2(q0[r]), ub3(q0[r]), x0, s[r][b][0]);
+                    s[r][b][1] = dot4(ub0(q1[r]), ub1(q1[r]), ub2(q1[r]), ub3(q1[r]), x1, s[r][b][1]);
+                    s[r][b][2] = dot4(ub0(q2[r]), ub1(q2[r]), ub2(q2[r]), ub3(q2[r]), x2, s[r][b][2]);
+                    s[r][b][3] = dot4(ub0(q3[r]), ub1(q3[r]), ub2(q3[r]), ub3(q3[r]), x3, s[r][b][3]);
                 }
             }
         }
@@ -504,7 +500,7 @@ struct UnitPair<F_Q4_0> {
                     s1[b] = dot4(l0, l1, l2, l3, xs.q(b, 8 + p), s1[b]);
                     s1[b] = dot4(h0, h1, h2, h3, xs.q(b, 12 + p), s1[b]);
                 }
-            }
+                }
             const float d0 = h2f(w[r].a.x), d1 = h2f(w[r].b.x >> 16);
 #pragma unroll
             for (int b = 0; b < B; ++b) {
@@ -556,7 +552,7 @@ struct UnitPair<F_Q4_1> {
                     s1[b] = dot4(l0, l1, l2, l3, xs.q(b, 8 + p), s1[b]);
                     s1[b] = dot4(h0, h1, h2, h3, xs.q(b, 12 + p), s1[b]);
                 }
-            }
+                }
             const float d0 = h2f(w[r].a.x) * nib, m0 = h2f(w[r].a.x >> 16), d1 = h2f(w[r].b.y) * nib, m1 = h2f(w[r].b.y >> 16);
 #pragma unroll
             for (int b = 0; b < B; ++b) {
@@ -604,7 +600,7 @@ struct UnitPair<F_Q8_0> {
                     s0[b] = dot4(ub0(a), ub1(a), ub2(a), ub3(a), xs.q(b, p), s0[b]);
                     s1[b] = dot4(ub0(c), ub1(c), ub2(c), ub3(c), xs.q(b, 8 + p), s1[b]);
                 }
-            }
+                }
             const float d0 = h2f(v[0]), d1 = h2f(v[8] >> 16);
 #pragma unroll
             for (int b = 0; b < B; ++b) {
@@ -898,23 +894,29 @@ __global__ void __launch_bounds__(512) gemv_ksplit_kernel(const uint8_t *__restr
 }
 
 // LDS bytes one staged K-chunk of `itc` wave steps takes for batch B.
-template <int FMT>
+template <class U>
 __host__ __device__ constexpr size_t gemv_lds_bytes(int B, int itc) {
-    return (size_t)B * itc * 64 * ((Unit<FMT>::UV / 4 + 1) * 16 + Unit<FMT>::NS * 4);
+    return (size_t)B * itc * 64 * ((U::UV / 4 + 1) * 16 + U::NS * 4);
 }
 
+// Batch 2..8 GEMV (and any batch-1 shape the register-resident kernels do not take):
 // y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) for b < rows <= B.
+//   The activations of all batch rows are staged in LDS in unit order; a wave decodes the units of R weight rows
+//   once per step and uses them for every batch row, reading the activations from LDS.  Work items (row group,
+//   step) run through a ring of NBUF register buffers: with two, the next item's weights are in flight while one is
+//   decoded; the big-batch variants keep one buffer (their accumulators need the registers) and rely on the other
+//   resident waves to cover the latency.
 //   grid: any number of workgroups of a multiple of 64 threads; waves take row groups of R rows round-robin.
 //   itc : wave steps (64 units each) staged in LDS at a time; K beyond that is processed in further chunks,
 //         each wave adding its partial sums to y (same wave, same order: deterministic).
-template <int FMT, int B, int R, int CV>
+template <class U, int B, int R, int CV, int NBUF>
 __global__ void __launch_bounds__(512) gemv_lds_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
                                                         const float *__restrict__ bias, float *__restrict__ y, int n, int k, int rows,
                                                         int itc, float nib) {
-    using U = Unit<FMT>;
-    constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG;
+    constexpr int FMT = U::FMT, UQ = U::UV / 4, NS = U::NS, SG = U::SG;
     extern __shared__ float4 smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x, nwaves = nthreads >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int units = k / U::UV;
     const int steps = (units + 63) >> 6;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
@@ -924,58 +926,91 @@ __global__ void __launch_bounds__(512) gemv_lds_kernel(const uint8_t *__restrict
     float4 *xl = smem;
     float *sums = reinterpret_cast<float *>(xl + (size_t)B * bs);
     const int kq = k >> 2;  // quads per activation row
+    const int first = blockIdx.x * nwaves + wave, gstride = gridDim.x * nwaves;
 
     for (int c0 = 0; c0 < steps; c0 += itc) {
         const int nit = min(itc, steps - c0);
         if (c0 > 0) __syncthreads();
-        // ---- stage x[:, chunk] in unit order, with the partial sums of each group of SG quads
-        const int f0 = c0 * 64 * UQ, f1 = (c0 + nit) * 64 * UQ;  // quad range of the chunk (may run past kq: zero fill)
-        for (int b = 0; b < B; ++b) {
-            for (int f = f0 + tid; f < f1; f += blockDim.x) {  // f1 - f0 is a multiple of 64: whole waves
-                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (f < kq && b < rows) v = reinterpret_cast<const float4 *>(x + (size_t)b * k)[f];
-                int u, g;
-                U::slot(f, u, g);
-                u -= c0 * 64;
-                xl[(size_t)b * bs + (size_t)u * (UQ + 1) + g] = v;
-                const float s = group_sum<SG>((v.x + v.y) + (v.z + v.w));
-                if ((f & (SG - 1)) == 0) sums[(size_t)b * ss + u * NS + g / SG] = s;
+        // ---- stage x[:, chunk] in unit order with the partial sums of each group of SG quads; eight loads per thread
+        // are issued before the first LDS write so that their latencies overlap
+        const int f0 = c0 * 64 * UQ, nq = nit * 64 * UQ;  // quads of the chunk per batch row (may run past kq: zero fill)
+        for (int base = 0; base < B * nq; base += nthreads * 8) {
+            float4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int idx = base + j * nthreads + tid;
+                const int b = idx / nq, f = f0 + idx - b * nq;
+                v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < B * nq && f < kq && b < rows) v[j] = reinterpret_cast<const float4 *>(x + (size_t)b * k)[f];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int idx = base + j * nthreads + tid;
+                if (idx < B * nq) {  // whole waves: nq and nthreads are multiples of 64
+                    const int b = idx / nq, f = f0 + idx - b * nq;
+                    int u, g;
+                    U::slot(f, u, g);
+                    u -= c0 * 64;
+                    xl[(size_t)b * bs + (size_t)u * (UQ + 1) + g] = v[j];
+                    const float sm = group_sum<SG>((v[j].x + v[j].y) + (v[j].z + v[j].w));
+                    if ((f & (SG - 1)) == 0) sums[(size_t)b * ss + u * NS + g / SG] = sm;
+                }
             }
         }
         __syncthreads();
-        // ---- row groups
-        for (int rg = blockIdx.x * nwaves + wave; rg < ngroups; rg += gridDim.x * nwaves) {
-            float acc[R][B];
+        // ---- work items (row group, step) through the ring
+        typename U::Raw buf[NBUF][R];
+        auto fill = [&](typename U::Raw(&dst)[R], int rg, int it) {
+            const bool live = rg < ngroups;  // a dead item is "loaded" from the first bytes of the matrix: one cache line
+            uint32_t off[U::NOFF];
+            U::offsets(min((c0 + it) * 64 + lane, units - 1), off);
 #pragma unroll
-            for (int r = 0; r < R; ++r)
+            for (int i = 0; i < U::NOFF; ++i) off[i] = live ? off[i] : 0u;
 #pragma unroll
-                for (int b = 0; b < B; ++b) acc[r][b] = 0.f;
-            for (int it = 0; it < nit; ++it) {
-                const int u = (c0 + it) * 64 + lane;
-                const int uc = min(u, units - 1);  // lanes past the row end re-read the last unit against zeroed x
-                typename U::Raw w[R];
-                uint32_t off[U::NOFF];
-                U::offsets(uc, off);
+            for (int r = 0; r < R; ++r) U::load(dst[r], W + (live ? (size_t)min(rg * R + r, n - 1) * rowbytes : 0), off);
+        };
+        int rg_l = first, it_l = 0;  // next item to load
+        int rg_c = first, it_c = 0;  // next item to decode
 #pragma unroll
-                for (int r = 0; r < R; ++r) U::load(w[r], W + (size_t)min(rg * R + r, n - 1) * rowbytes, off);
-                const XLds xs{xl + (size_t)(it * 64 + lane) * (UQ + 1), sums + (it * 64 + lane) * NS, bs, ss};
-                U::template dot<B, R, CV>(w, uc, xs, acc, nib);
-            }
+        for (int sl = 0; sl < NBUF; ++sl) {
+            fill(buf[sl], rg_l, it_l);
+            if (++it_l == nit) { it_l = 0; rg_l += gstride; }
+        }
+        float acc[R][B];
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
+        for (int r = 0; r < R; ++r)
 #pragma unroll
-                for (int b = 0; b < B; ++b) {
-                    float t = wave_sum(acc[r][b]);
-                    const int row = rg * R + r;
-                    if (lane == 0 && row < n && b < rows) {
-                        float *o = y + (size_t)b * n + row;
-                        if (c0 == 0) {
-                            *o = bias ? t + bias[row] : t;
-                        } else {
-                            *o += t;
+            for (int b = 0; b < B; ++b) acc[r][b] = 0.f;
+        while (rg_c < ngroups) {
+#pragma unroll
+            for (int sl = 0; sl < NBUF; ++sl) {
+                if (rg_c < ngroups) {  // wave-uniform
+                    const int uc = min((c0 + it_c) * 64 + lane, units - 1);  // lanes past the row end: last unit, zeroed x
+                    const XLds xs{xl + (size_t)(it_c * 64 + lane) * (UQ + 1), sums + (it_c * 64 + lane) * NS, bs, ss};
+                    U::template dot<B, R, CV>(buf[sl], uc, xs, acc, nib);
+                    if (it_c == nit - 1) {
+#pragma unroll
+                        for (int r = 0; r < R; ++r) {
+#pragma unroll
+                            for (int b = 0; b < B; ++b) {
+                                const float t = wave_sum(acc[r][b]);
+                                acc[r][b] = 0.f;
+                                const int row = rg_c * R + r;
+                                if (lane == 0 && row < n && b < rows) {
+                                    float *o = y + (size_t)b * n + row;
+                                    if (c0 == 0) {
+                                        *o = bias ? t + bias[row] : t;
+                                    } else {
+                                        *o += t;
+                                    }
+                                }
+                            }
                         }
                     }
                 }
+                if (++it_c == nit) { it_c = 0; rg_c += gstride; }
+                fill(buf[sl], rg_l, it_l);
+                if (++it_l == nit) { it_l = 0; rg_l += gstride; }
             }
         }
     }

@@ -119,35 +119,40 @@ struct GemvVariant {
     gemv_fn fn;
     int B, R;
     size_t lds_per_step;  // LDS bytes per staged wave step
+    int unit_values;      // values one lane decodes per step
 };
 
-template <int FMT, int B, int R>
+template <class U, int B, int R, int NBUF>
 GemvVariant variant() {
     // the fp8 nibble conversion only applies to the 4-bit formats; the others ignore CV
-    constexpr int CV = (FMT == F_Q4_K || FMT == F_Q4_0 || FMT == F_Q4_1) ? 1 : 0;
-    return GemvVariant{gemv_lds_kernel<FMT, B, R, CV>, B, R, gemv_lds_bytes<FMT>(B, 1)};
+    constexpr int CV = (U::FMT == F_Q4_K || U::FMT == F_Q4_0 || U::FMT == F_Q4_1) ? 1 : 0;
+    return GemvVariant{gemv_lds_kernel<U, B, R, CV, NBUF>, B, R, gemv_lds_bytes<U>(B, 1), U::UV};
 }
 
-template <int FMT>
-GemvVariant pick_fmt(int rows) {
-    if (rows <= 1) return variant<FMT, 1, 4>();
-    if (rows <= 2) return variant<FMT, 2, 4>();
-    if (rows <= 4) return variant<FMT, 4, 2>();
-    return variant<FMT, 8, 2>();
-}
-
-GemvVariant pick(int fmt, int rows) {
-    switch (fmt) {
-    case F_Q4_0: return pick_fmt<F_Q4_0>(rows);
-    case F_Q4_1: return pick_fmt<F_Q4_1>(rows);
-    case F_Q8_0: return pick_fmt<F_Q8_0>(rows);
-    case F_Q4_K: return pick_fmt<F_Q4_K>(rows);
-    case F_Q5_K: return pick_fmt<F_Q5_K>(rows);
-    default: return pick_fmt<F_Q6_K>(rows);
+// batch rows -> (rows decoded together, ring depth): chosen so that no variant spills registers
+template <class U>
+GemvVariant pick_unit(int rows) {
+    if (rows <= 1) return variant<U, 1, 2, 2>();
+    if (rows <= 2) return variant<U, 2, 2, 2>();
+    if constexpr (U::FMT == F_Q8_0) {  // 17 dwords per block pair: one row at a time
+        if (rows <= 4) return variant<U, 4, 1, 1>();
+        return variant<U, 8, 1, 1>();
+    } else {
+        if (rows <= 4) return variant<U, 4, 2, 1>();
+        return variant<U, 8, 2, 1>();
     }
 }
 
-int unit_values(int fmt) { return block_values(fmt) == 256 ? 64 : 32; }
+GemvVariant pick(int fmt, int rows, bool pairs) {
+    switch (fmt) {
+    case F_Q4_0: return pairs ? pick_unit<UnitPair<F_Q4_0>>(rows) : pick_unit<Unit<F_Q4_0>>(rows);
+    case F_Q4_1: return pairs ? pick_unit<UnitPair<F_Q4_1>>(rows) : pick_unit<Unit<F_Q4_1>>(rows);
+    case F_Q8_0: return pairs ? pick_unit<UnitPair<F_Q8_0>>(rows) : pick_unit<Unit<F_Q8_0>>(rows);
+    case F_Q4_K: return pick_unit<Unit<F_Q4_K>>(rows);
+    case F_Q5_K: return pick_unit<Unit<F_Q5_K>>(rows);
+    default: return pick_unit<Unit<F_Q6_K>>(rows);
+    }
+}
 
 typedef void (*gemv1_fn)(const uint8_t *, const float *, const float *, float *, int, int, float);
 typedef void (*xreg_fn)(const XregArgs);
@@ -272,8 +277,8 @@ int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float
         if (w->k <= 4096) return launch_gemv_xreg(w, x, bias, y, stream);
         if (w->k <= 32768 && ksplit_lds(w->fmt, (w->k + 4095) / 4096) <= g.max_lds) return launch_gemv_ksplit(w, x, bias, y, stream);
     }
-    GemvVariant v = pick(w->fmt, rows);
-    const int units = w->k / unit_values(w->fmt);
+    GemvVariant v = pick(w->fmt, rows, w->k % 64 == 0);
+    const int units = w->k / v.unit_values;
     const int steps = (units + 63) / 64;
     // stage as many steps as fit in 64 KiB (keeps several workgroups per CU); one step may need more
     int itc = (int)(65536 / v.lds_per_step);
@@ -282,10 +287,14 @@ int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float
     const size_t lds = v.lds_per_step * itc;
     if (lds > g.max_lds) return fail(JITNN_HIP_EINVAL, "GEMV needs %zu bytes of LDS, the device offers %zu", lds, g.max_lds);
     if (int rc = allow_lds((const void *)v.fn, lds)) return rc;
-    const int threads = 256, waves = threads / 64;
+    // at least eight waves per CU: big LDS footprints leave room for one or two workgroups only, so those get 8 waves each
+    int per_cu = (int)((g.lds_per_cu - 2048) / lds);
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 4) per_cu = 4;
+    const int threads = per_cu >= 2 ? 256 : 512, waves = threads / 64;
     const int groups = (w->n + v.R - 1) / v.R;
     int blocks = (groups + waves - 1) / waves;
-    const int cap = g.cus * 8;
+    const int cap = g.cus * per_cu;
     if (blocks > cap) blocks = cap;
     hipLaunchKernelGGL(v.fn, dim3(blocks), dim3(threads), lds, stream, w->dev, x, bias, y, w->n, w->k, rows, itc, g.nib);
     HIP_TRY(hipGetLastError());
