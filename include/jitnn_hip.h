@@ -34,6 +34,8 @@ extern "C" {
 #define JITNN_HIP_EDEVICE (-2)  /* a HIP runtime call failed */
 #define JITNN_HIP_ENODEVICE (-3) /* no gfx950 device / library not initialised */
 #define JITNN_HIP_ENOMEM (-4)
+#define JITNN_HIP_EIO (-5)       /* a file cannot be read or is not a valid GGUF file (Java: IOException) */
+#define JITNN_HIP_EUNSUPPORTED (-6) /* a ggml type this path has no tensor type for (Java: UnsupportedOperationException) */
 
 #define JITNN_HIP_Q4_0 2
 #define JITNN_HIP_Q4_1 3
@@ -126,6 +128,39 @@ JITNN_HIP_API int jitnn_hip_malloc(long long nbytes, void **dev);
 JITNN_HIP_API int jitnn_hip_free(void *dev);
 JITNN_HIP_API int jitnn_hip_memcpy_h2d(void *dev, const void *host, long long nbytes);
 JITNN_HIP_API int jitnn_hip_memcpy_d2h(void *host, const void *dev, long long nbytes);
+
+/* ---- GGUF files ------------------------------------------------------------------------------------ */
+
+/* Reader of llama.cpp's model format, versions 2 and 3, with the acceptance rules of GgufFile.open
+ * (gguf/GgufFile.java:100-175, parsing :428-572): magic and version, counts that must fit the file, every metadata
+ * value type (arrays nested at most 64 deep), general.alignment a power of two (default 32), tensor shapes reversed
+ * to outermost-first, every tensor aligned and inside the file; truncated or crafted files give JITNN_HIP_EIO.
+ * Needs no device except for jitnn_hip_gguf_tensor_upload. */
+typedef struct jitnn_hip_gguf jitnn_hip_gguf;
+
+JITNN_HIP_API int jitnn_hip_gguf_open(const char *path, jitnn_hip_gguf **out);
+JITNN_HIP_API int jitnn_hip_gguf_close(jitnn_hip_gguf *f);
+/* version(), alignment(), dataOffset() and the sizes of tensorInfos() / metadata() (gguf/GgufFile.java:177-200). */
+JITNN_HIP_API int jitnn_hip_gguf_header(const jitnn_hip_gguf *f, int *version, int *alignment, long long *data_offset, long long *tensor_count,
+                                        long long *kv_count);
+/* All metadata, in file order, as one JSON object in UTF-8 (metadata(), gguf/GgufFile.java:203-206): integers of any
+ * width as integers (a uint64 above 2^63-1 reads as negative, as in the reference), float32/float64 as numbers with a
+ * fraction or exponent, bool, string, arrays (nested arrays as nested lists).  Copies at most cap bytes including the
+ * terminating NUL and returns the full length without it. */
+JITNN_HIP_API long long jitnn_hip_gguf_metadata_json(const jitnn_hip_gguf *f, char *buf, long long cap);
+/* Name of tensor `index` in file order (NUL-terminated, truncated to cap). */
+JITNN_HIP_API int jitnn_hip_gguf_tensor_name(const jitnn_hip_gguf *f, long long index, char *name, int cap);
+/* info(name) (gguf/GgufFile.java:319-326, gguf/GgufTensorInfo.java:29-39): ggml type id, shape (outermost first, up to
+ * 8 axes), byte offset in the file, byte count (-1 for a type id this reader does not know).  Any out pointer may be
+ * NULL.  Unknown name: JITNN_HIP_EINVAL. */
+JITNN_HIP_API int jitnn_hip_gguf_tensor_info(const jitnn_hip_gguf *f, const char *name, int *ggml_type, int *ndims, long long *dims,
+                                             long long *file_offset, long long *nbytes);
+/* raw(name): the tensor's bytes as stored (gguf/GgufFile.java:358-366).  nbytes must be the tensor's byte count. */
+JITNN_HIP_API int jitnn_hip_gguf_tensor_read(const jitnn_hip_gguf *f, const char *name, void *dst_host, long long nbytes);
+/* tensor(name) for the block-quantised types of this path (gguf/GgufFile.java:329-346): the blocks go from the
+ * mapped file to HBM unchanged; an n-d tensor becomes [numel / last axis, last axis].  Other types:
+ * JITNN_HIP_EUNSUPPORTED. */
+JITNN_HIP_API int jitnn_hip_gguf_tensor_upload(const jitnn_hip_gguf *f, const char *name, jitnn_hip_weight **out);
 
 /* ---- Llama-style decode step on quantised weights (BASELINE config 5) ----------------------------- */
 

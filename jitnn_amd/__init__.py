@@ -9,3 +9,5 @@ from .dtype import DType  # noqa: F401
 from .ops import F, Gguf, Quant  # noqa: F401
 from .tensor import Tensor  # noqa: F401
 from .llama import LlamaDecoder  # noqa: F401
+from .gguf_file import GgufFile, GgufTensorInfo  # noqa: F401
+from ._lib import UnsupportedTypeError  # noqa: F401

@@ -11,7 +11,11 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libjitnn_hip.so"
 
-OK, EINVAL, EDEVICE, ENODEVICE, ENOMEM = 0, -1, -2, -3, -4
+OK, EINVAL, EDEVICE, ENODEVICE, ENOMEM, EIO, EUNSUPPORTED = 0, -1, -2, -3, -4, -5, -6
+
+
+class UnsupportedTypeError(TypeError):
+    """A ggml type this path has no tensor type for (the reference's UnsupportedOperationException)."""
 
 
 class JitnnError(RuntimeError):
@@ -46,6 +50,14 @@ def _bind() -> C.CDLL:
         "jitnn_hip_free": (i, [vp]),
         "jitnn_hip_memcpy_h2d": (i, [vp, vp, ll]),
         "jitnn_hip_memcpy_d2h": (i, [vp, vp, ll]),
+        "jitnn_hip_gguf_open": (i, [C.c_char_p, C.POINTER(vp)]),
+        "jitnn_hip_gguf_close": (i, [vp]),
+        "jitnn_hip_gguf_header": (i, [vp, C.POINTER(i), C.POINTER(i), C.POINTER(ll), C.POINTER(ll), C.POINTER(ll)]),
+        "jitnn_hip_gguf_metadata_json": (ll, [vp, C.c_char_p, ll]),
+        "jitnn_hip_gguf_tensor_name": (i, [vp, ll, C.c_char_p, i]),
+        "jitnn_hip_gguf_tensor_info": (i, [vp, C.c_char_p, C.POINTER(i), C.POINTER(i), C.POINTER(ll), C.POINTER(ll), C.POINTER(ll)]),
+        "jitnn_hip_gguf_tensor_read": (i, [vp, C.c_char_p, vp, ll]),
+        "jitnn_hip_gguf_tensor_upload": (i, [vp, C.c_char_p, C.POINTER(vp)]),
         "jitnn_hip_llama_create": (i, [i, i, i, i, i, i, i, i, C.c_float, C.c_float, C.POINTER(vp)]),
         "jitnn_hip_llama_free": (i, [vp]),
         "jitnn_hip_llama_set_weight": (i, [vp, i, i, vp]),
@@ -78,6 +90,10 @@ def check(rc: int, what: str) -> None:
     msg = f"calling {what} failed: {last_error()}"
     if rc == EINVAL:
         raise ValueError(msg)
+    if rc == EIO:
+        raise OSError(msg)  # the reference's IOException
+    if rc == EUNSUPPORTED:
+        raise UnsupportedTypeError(msg)
     raise JitnnError(msg)
 
 

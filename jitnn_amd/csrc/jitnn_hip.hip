@@ -17,6 +17,7 @@
 
 #include "dequant.h"
 #include "gemv.h"
+#include "gguf_file.h"
 #include "glue.h"
 #include "prefill.h"
 
@@ -661,6 +662,110 @@ int jitnn_hip_memcpy_d2h(void *host, const void *dev, long long nbytes) {
     if (int rc = check_ready()) return rc;
     HIP_TRY(hipMemcpy(host, dev, (size_t)nbytes, hipMemcpyDeviceToHost));
     return JITNN_HIP_OK;
+}
+
+}  // extern "C"
+
+// ================================================================================================ GGUF files
+
+struct jitnn_hip_gguf {
+    GgufFile *f;
+};
+
+extern "C" {
+
+int jitnn_hip_gguf_open(const char *path, jitnn_hip_gguf **out) {
+    if (!out) return fail(JITNN_HIP_EINVAL, "out is NULL");
+    *out = nullptr;
+    if (!path) return fail(JITNN_HIP_EINVAL, "path is NULL");
+    std::string err;
+    GgufFile *f = gguf_open(path, err);
+    if (!f) return fail(JITNN_HIP_EIO, "%s", err.c_str());
+    jitnn_hip_gguf *h = new (std::nothrow) jitnn_hip_gguf{f};
+    if (!h) {
+        delete f;
+        return fail(JITNN_HIP_ENOMEM, "out of host memory");
+    }
+    *out = h;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_gguf_close(jitnn_hip_gguf *h) {
+    if (!h) return JITNN_HIP_OK;
+    delete h->f;
+    delete h;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_gguf_header(const jitnn_hip_gguf *h, int *version, int *alignment, long long *data_offset, long long *tensor_count,
+                          long long *kv_count) {
+    if (!h) return fail(JITNN_HIP_EINVAL, "file is NULL");
+    if (version) *version = h->f->version;
+    if (alignment) *alignment = h->f->alignment;
+    if (data_offset) *data_offset = h->f->data_offset;
+    if (tensor_count) *tensor_count = (long long)h->f->tensors.size();
+    if (kv_count) *kv_count = h->f->kv_count;
+    return JITNN_HIP_OK;
+}
+
+long long jitnn_hip_gguf_metadata_json(const jitnn_hip_gguf *h, char *buf, long long cap) {
+    if (!h) return fail(JITNN_HIP_EINVAL, "file is NULL");
+    const std::string &j = h->f->metadata_json;
+    if (buf && cap > 0) {
+        const size_t n = j.size() < (size_t)cap - 1 ? j.size() : (size_t)cap - 1;
+        memcpy(buf, j.data(), n);
+        buf[n] = 0;
+    }
+    return (long long)j.size();
+}
+
+int jitnn_hip_gguf_tensor_name(const jitnn_hip_gguf *h, long long index, char *name, int cap) {
+    if (!h || !name || cap < 1) return fail(JITNN_HIP_EINVAL, "bad arguments");
+    if (index < 0 || index >= (long long)h->f->tensors.size()) return fail(JITNN_HIP_EINVAL, "tensor %lld of %zu", index, h->f->tensors.size());
+    strncpy(name, h->f->tensors[(size_t)index].name.c_str(), (size_t)cap - 1);
+    name[cap - 1] = 0;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_gguf_tensor_info(const jitnn_hip_gguf *h, const char *name, int *type, int *ndims, long long *dims, long long *file_offset,
+                               long long *nbytes) {
+    if (!h || !name) return fail(JITNN_HIP_EINVAL, "file or name is NULL");
+    const GgufTensor *t = h->f->find(name);
+    if (!t) return fail(JITNN_HIP_EINVAL, "%s: no tensor %s", h->f->path.c_str(), name);
+    if (type) *type = t->type_id;
+    if (ndims) *ndims = (int)t->shape.size();
+    if (dims)
+        for (size_t i = 0; i < t->shape.size(); ++i) dims[i] = t->shape[i];
+    if (file_offset) *file_offset = t->offset;
+    if (nbytes) *nbytes = t->bytes;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_gguf_tensor_read(const jitnn_hip_gguf *h, const char *name, void *dst_host, long long nbytes) {
+    if (!h || !name || !dst_host) return fail(JITNN_HIP_EINVAL, "NULL argument");
+    const GgufTensor *t = h->f->find(name);
+    if (!t) return fail(JITNN_HIP_EINVAL, "%s: no tensor %s", h->f->path.c_str(), name);
+    if (t->bytes < 0) return fail(JITNN_HIP_EUNSUPPORTED, "%s: ggml type %d is unknown, so its size is too", name, t->type_id);
+    if (nbytes != t->bytes) return fail(JITNN_HIP_EINVAL, "%s holds %lld bytes, asked for %lld", name, t->bytes, nbytes);
+    memcpy(dst_host, h->f->map + t->offset, (size_t)nbytes);
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_gguf_tensor_upload(const jitnn_hip_gguf *h, const char *name, jitnn_hip_weight **out) {
+    if (!out) return fail(JITNN_HIP_EINVAL, "out is NULL");
+    *out = nullptr;
+    if (!h || !name) return fail(JITNN_HIP_EINVAL, "file or name is NULL");
+    const GgufTensor *t = h->f->find(name);
+    if (!t) return fail(JITNN_HIP_EINVAL, "%s: no tensor %s", h->f->path.c_str(), name);
+    if (!known(t->type_id)) {
+        const GgmlTypeInfo *ti = ggml_type(t->type_id);
+        return fail(JITNN_HIP_EUNSUPPORTED, "%s: ggml type %s%d has no block-quantised tensor type on this path", name, ti ? ti->name : "id ",
+                    ti ? 0 : t->type_id);
+    }
+    if (t->shape.empty() || t->numel > 0x7fffffffLL)
+        return fail(JITNN_HIP_EUNSUPPORTED, "%s: %lld values; tensors hold at most 2^31-1", name, t->numel);
+    const long long k = t->shape.back(), n = k > 0 ? t->numel / k : 0;
+    return jitnn_hip_weight_upload(t->type_id, h->f->map + t->offset, t->bytes, (int)n, (int)k, out);
 }
 
 }  // extern "C"

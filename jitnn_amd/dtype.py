@@ -8,6 +8,7 @@ from enum import Enum
 class DType(Enum):
     #        ggml id, values per block, bytes per block
     F32 = (0, 0, 0)
+    I32 = (26, 0, 0)
     Q4_0 = (2, 32, 18)
     Q4_1 = (3, 32, 20)
     Q8_0 = (8, 32, 34)

@@ -87,11 +87,19 @@ class Tensor:
             raise ValueError("numpy() is for FP32 tensors; use to_float_array() to dequantise")
         return self._host
 
+    def to_int_array(self) -> np.ndarray:
+        """Row-major values of an I32 tensor (Tensor.toIntArray)."""
+        if self._dtype != DType.I32:
+            raise ValueError(f"to_int_array() on a {self._dtype.name} tensor")
+        return self._host.reshape(-1).copy()
+
     def to_float_array(self) -> np.ndarray:
         """Row-major values as FP32; block tensors are dequantised on the device, bit-identical to the reference's
         per-value decode (Tensor.toFloatArray, core/Tensor.java:539-555)."""
         if self._dtype == DType.F32:
             return self._host.reshape(-1).copy()
+        if self._dtype == DType.I32:
+            return self._host.reshape(-1).astype(np.float32)
         y = np.empty(self.numel(), dtype=np.float32)
         _lib.check(_lib.lib.jitnn_hip_dequantize(self._handle, y.ctypes.data_as(C.c_void_p)), "jitnn_hip_dequantize")
         return y
