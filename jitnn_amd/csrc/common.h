@@ -21,6 +21,10 @@ __host__ __device__ constexpr int block_bytes(int fmt) {
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 // 128/64/32/16-bit global loads from addresses that are only A-byte aligned.  Q8_0, Q4_0 and Q6_K blocks
 // are 34, 18 and 210 bytes long, so their fields sit on 2-byte boundaries; gfx950 global memory

@@ -17,6 +17,7 @@
 
 #include "dequant.h"
 #include "gemv.h"
+#include "gemv_mfma.h"
 #include "gguf_file.h"
 #include "glue.h"
 #include "prefill.h"
@@ -65,6 +66,7 @@ struct State {
     // count the reference's own tests use (1, 5, 40) on the FP32 path, whose error meets their 2e-4 / 1e-3 bars.
     int gemv_max_rows = 64;
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
+    bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
 };
 State g;
 std::mutex g_mu;
@@ -273,7 +275,39 @@ int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *b
     return JITNN_HIP_OK;
 }
 
+typedef void (*mfma_fn)(const uint8_t *, const float *, const float *, float *, int, int, int);
+
+struct MfmaVariant {
+    mfma_fn fn;
+    size_t lds;
+};
+
+MfmaVariant pick_mfma(int fmt) {
+    switch (fmt) {
+    case F_Q4_0: return {gemv_mfma_kernel<F_Q4_0>, gemv_mfma_lds_bytes<F_Q4_0>()};
+    case F_Q4_1: return {gemv_mfma_kernel<F_Q4_1>, gemv_mfma_lds_bytes<F_Q4_1>()};
+    case F_Q8_0: return {gemv_mfma_kernel<F_Q8_0>, gemv_mfma_lds_bytes<F_Q8_0>()};
+    case F_Q4_K: return {gemv_mfma_kernel<F_Q4_K>, gemv_mfma_lds_bytes<F_Q4_K>()};
+    case F_Q5_K: return {gemv_mfma_kernel<F_Q5_K>, gemv_mfma_lds_bytes<F_Q5_K>()};
+    default: return {nullptr, 0};
+    }
+}
+
+// Batch 2..8, rows a multiple of 256 values long: block sums on the matrix cores, one workgroup of 16 waves per CU.
+int launch_gemv_mfma(const MfmaVariant &v, const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    if (int rc = allow_lds((const void *)v.fn, v.lds)) return rc;
+    const int groups = (w->n + 15) / 16;
+    const int blocks = groups < g.cus ? groups : g.cus;
+    hipLaunchKernelGGL(v.fn, dim3(blocks), dim3(MF_THREADS), v.lds, stream, w->dev, x, bias, y, w->n, w->k, rows);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    if (rows >= 2 && rows <= 8 && w->k % 256 == 0 && w->n >= 16 && g.batch_mfma) {
+        const MfmaVariant v = pick_mfma(w->fmt);
+        if (v.fn && v.lds <= g.max_lds) return launch_gemv_mfma(v, w, x, rows, bias, y, stream);
+    }
     if (rows == 1 && !g.force_lds) {
         if (w->k <= 4096) return launch_gemv_xreg(w, x, bias, y, stream);
         if (w->k <= 32768 && ksplit_lds(w->fmt, (w->k + 4095) / 4096) <= g.max_lds) return launch_gemv_ksplit(w, x, bias, y, stream);
@@ -454,6 +488,7 @@ int jitnn_hip_init(int device_ordinal) {
         if (v >= 1) g.gemv_max_rows = v;
     }
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     g.device = device_ordinal;
     g.ready = true;
     return JITNN_HIP_OK;

@@ -16,9 +16,6 @@
 
 namespace jitnn {
 
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int PF_BN = 128, PF_BM = 128, PF_BK = 64, PF_LD = PF_BK + 8;  // LDS row pitch in halves: 144 bytes, conflict-free 16-byte reads
