@@ -9,16 +9,21 @@
 //     exact in the FP32 accumulator, so the block sums are as good as FP32 arithmetic;
 //   * the block scales (and the Q4_K / Q5_K / Q4_1 offsets) are applied in FP32 to the 4 x 16 block sums a wave
 //     holds, never to individual weights.
-// A workgroup of 16 waves owns groups of 16 weight rows and walks K in passes of 4096 values; wave w owns column w
-// of a pass (256 values: one K-quant super-block, eight 32-value blocks).
-//   * Weights: the 16 x 4096 values of a row group are 16 contiguous byte runs; the whole workgroup copies them
-//     with full 128-bit coalesced loads through registers into LDS (two stages in LDS, two more groups in flight
-//     in registers), and each wave then picks the bytes of its column from LDS in operand order.
-//   * Activations: a wave builds the A operands of its column once per pass - one coalesced read of the 8 x 256
+// A workgroup of 8 waves (two per SIMD, 256 VGPRs each) owns groups of 16 weight rows and walks K in passes of
+// 4096 values; wave w owns columns w and w + 8 of a pass (a column = 256 values: one K-quant super-block, eight
+// 32-value blocks), so a tile is 16 weight rows x one column.
+//   * Weights: the bytes of a tile are 16 contiguous runs (144 bytes each for Q4_K).  The wave copies them with
+//     full 128-bit loads - consecutive lanes on consecutive 16-byte chunks of a run - through a two-deep ring of
+//     registers into its own LDS region, and each lane then picks the bytes of its row in operand order from there.
+//     No workgroup barrier is involved: the region belongs to the wave.
+//   * Activations: a wave builds the A operands of its columns once per pass - one coalesced read of the 8 x 256
 //     values, scale 2^e from the column's largest magnitude per row, FP16 split, transposition into operand order
-//     through a private LDS region - and keeps them in 36 VGPRs for all row groups.
-//   * The partial sums of the 16 waves meet in LDS (double buffered), added in wave order: a fixed summation order,
-//     no atomics.  Passes after the first add to y.
+//     through the same LDS region - and keeps them in 72 VGPRs for all row groups.  The loads of x go out before the
+//     first weight loads (loads return in order) and the build runs while HBM works on the weights.
+//   * A wave keeps the partial sums of up to four row groups; then the sums of the eight waves meet in LDS and are
+//     added in wave order: a fixed summation order, no atomics.  Passes after the first add to y.
+// The kernel is bound by the VALU work of turning quants into FP16 (about 170 instructions per tile) and of the
+// operand build, not by HBM: it runs near 2.3 TB/s at every batch size from 2 to 8.
 //
 // Lane roles inside a wave: n = lane & 15 is the weight row of the group (B column, C column) and the A row it
 // supplies; kq = lane >> 4 selects the eight K positions of a 32-value block the lane supplies to both operands.
@@ -262,12 +267,12 @@ struct MTile<F_Q8_0> {
     }
 };
 
-// Pitch of a tile row in a wave's LDS region: at least BYTES, a multiple of 16, and an odd multiple of 32 so that
-// the 16 rows of an operand read start in different banks.
+// Pitch of a tile row in a wave's LDS region: at least BYTES and an odd multiple of 16, so that the 16 rows of an
+// operand read (two dwords per lane, 64 banks) start four banks apart and never collide.
 template <int FMT>
 __host__ __device__ constexpr int mf_row_pitch() {
-    int p = (MTile<FMT>::BYTES + 31) / 32 * 32;
-    return (p / 32) % 2 ? p : p + 32;
+    int p = MTile<FMT>::BYTES;  // a multiple of 16
+    return (p / 16) % 2 ? p : p + 16;
 }
 constexpr int MF_GROUPS = 4;            // row groups whose partial sums a wave keeps before the workgroup adds them
 constexpr int MF_XBUILD = 4096 + 256;   // a region while a wave builds A operands in it: four 1 KiB operands + the block sums'
@@ -404,10 +409,6 @@ __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__
                 loff[c][i] = live[c] && crow[i] < 16 ? (uint32_t)(crow[i] * rowbytes + (size_t)(t0 + wave + c * MF_WAVES) * T::BYTES + (size_t)cidx[i] * 16) : 0u;
         }
         auto fetch = [&](u32x4(&dst)[NC][NL], int grp) {
-#ifdef MF_PROBE_DEAD
-            for (int c = 0; c < NC; ++c) for (int i = 0; i < NL; ++i) dst[c][i] = ld128<16>(W);
-            return;
-#endif
             if (grp >= ngroups) return;  // workgroup-uniform
             // the last group of a ragged matrix is the last 16 rows: in bounds, its first rows computed twice, stored once
             const uint8_t *gb = W + (size_t)min(grp * 16, n - 16) * rowbytes;
@@ -444,16 +445,8 @@ __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__
 
         f16x8 xa[NC][8], xs[NC];
         float inv[NC][4];
-#ifdef MF_PROBE_NOPRO
-        for (int c = 0; c < NC; ++c) {
-            for (int j = 0; j < 8; ++j) xa[c][j] = f16x8{1, 1, 1, 1, 1, 1, 1, 1};
-            xs[c] = xa[c][0];
-            for (int i = 0; i < 4; ++i) inv[c][i] = 1.f + v[c][i].x;
-        }
-#else
 #pragma unroll
         for (int c = 0; c < NC; ++c) mf_build_operands<T>(v[c], have[c], reg + c * REGION, lane, xa[c], xs[c], inv[c]);
-#endif
 
         // ---- row groups, MF_GROUPS at a time: registers -> the wave's LDS regions -> operands -> partial sums
         for (int base = blockIdx.x; base < ngroups; base += MF_GROUPS * stride) {
@@ -469,11 +462,7 @@ __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__
 #pragma unroll
                     for (int c = 0; c < NC; ++c) {
                         if (!live[c]) continue;  // wave-uniform: nothing was staged for a column past the end of the row
-#ifdef MF_PROBE_NOMMA
-                        const f32x4 a = f32x4{(float)reg[c * REGION + nq * PITCH + kq], (float)xa[c][0][0], 0.f, 0.f};
-#else
                         const f32x4 a = T::mma(reg + c * REGION + nq * PITCH, kq, xa[c], xs[c]);
-#endif
 #pragma unroll
                         for (int i = 0; i < 4; ++i) acc[gi][i] = __builtin_fmaf(a[i], inv[c][i], acc[gi][i]);
                     }

@@ -121,6 +121,35 @@ def test_gemv_vs_oracle(jn, fmt, n, k):
 
 
 @pytest.mark.parametrize("fmt", HOT_FORMATS)
+@pytest.mark.parametrize("rows", [2, 5, 7, 8])
+def test_batch_rows_of_very_different_magnitude(jn, fmt, rows):
+    """Batches 2..8 with K a multiple of 256 run on the matrix cores with the activations split into two FP16 parts
+    under a power-of-two scale per (row, 256-value column): huge, tiny, zero and outlier-dominated rows must each
+    meet the GEMV bar against their own largest output."""
+    from oracle import oracle
+    rng = np.random.default_rng(rows * 31 + GGML_ID[fmt])
+    n, k = 83, 2048 + 256
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    x = rng.standard_normal((rows, k)).astype(np.float32)
+    x[0] *= np.float32(1e6)
+    x[1] *= np.float32(1e-6)
+    if rows > 2:
+        x[2] = 0
+    if rows > 3:
+        x[3, 700] = np.float32(1e4)     # one outlier in a column of ordinary values
+    if rows > 4:
+        x[4, :256] *= np.float32(1e-30)  # a column near the bottom of the FP32 range
+    ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, None, n, k)
+    y = jn.Gguf.linear(jn.Tensor.of(x), w, None).numpy()
+    for r in range(rows):
+        scale = max(float(np.abs(ref[r]).max()), 1e-30)
+        assert float(np.abs(y[r].astype(np.float64) - ref[r]).max()) / scale <= GEMV_BAR, (fmt, rows, r)
+    if rows > 2:
+        assert not y[2].any()
+
+
+@pytest.mark.parametrize("fmt", HOT_FORMATS)
 def test_small_k_32_blocks_and_many_rows(jn, fmt):
     """K of a single block for the 32-value formats; rows beyond one batch of 8 (9, 17, 40, 64)."""
     from oracle import oracle
