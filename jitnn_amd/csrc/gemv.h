@@ -642,8 +642,10 @@ struct XregArgs {
 //   NORM  fuses the RMSNorm that precedes the linear (ops/RowNorm.java:286-306) into the staging of x;
 //   DUAL  computes the SwiGLU gate of a Llama FFN (F.swiglu, F.java:1159-1161) from two matrices in one pass: the
 //         ring alternates rows of w[0] (gate) and w2 (up), so NB = PF + 1 must be even.
+// The body takes its workgroup number and the number of workgroups as arguments so that two of them, for two
+// formats, can share one launch (gemv_xreg2_kernel).
 template <class U, int CV, int PF, bool BIAS, bool NORM, bool DUAL>
-__global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const XregArgs a) {
+__device__ __forceinline__ void gemv_xreg_body(const XregArgs &a, const int bid, const int nblocks) {
     constexpr int FMT = U::FMT, STEPS = 64 / U::UV;  // a lane keeps 64 activations: one 64-value unit or two of 32
     constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG, NB = PF + 1;
     static_assert(!DUAL || NB % 2 == 0, "gate and up rows alternate in the ring");
@@ -657,8 +659,8 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const XregArgs 
     const int k = a.k, n = a.n[0] + a.n[1] + a.n[2];
     const int units = k / U::UV;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
-    const int stride = gridDim.x * nwaves;
-    const int row0 = blockIdx.x * nwaves + wave;
+    const int stride = nblocks * nwaves;
+    const int row0 = bid * nwaves + wave;
     int uc[STEPS];
     uint32_t off[STEPS][U::NOFF];  // byte offsets of this lane's fields within a row: the same for every row
 #pragma unroll
@@ -767,6 +769,20 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const XregArgs 
             fill(buf[b], bv[b], row + RSTEP * stride, DUAL && (b & 1));
         }
     }
+}
+
+template <class U, int CV, int PF, bool BIAS, bool NORM, bool DUAL>
+__global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_kernel(const XregArgs a) {
+    gemv_xreg_body<U, CV, PF, BIAS, NORM, DUAL>(a, blockIdx.x, gridDim.x);
+}
+
+// Two sets of matrices in two formats over the same activations in one launch (the q / k and the v projections of a
+// Q4_K_M layer): workgroups below `split` run the first set, the others the second, each exactly as its own launch
+// would.  Always with the RMSNorm fused, never with bias or SwiGLU: that is the one place a decode step needs it.
+template <class UA, int CVA, class UB, int CVB, int PF>
+__global__ void __launch_bounds__(XREG_THREADS) gemv_xreg2_kernel(const XregArgs a, const XregArgs b, const int split) {
+    if ((int)blockIdx.x < split) gemv_xreg_body<UA, CVA, PF, false, true, false>(a, blockIdx.x, split);
+    else gemv_xreg_body<UB, CVB, PF, false, true, false>(b, blockIdx.x - split, gridDim.x - split);
 }
 
 // Batch-1 GEMV for rows longer than 4096 values: the row is cut into slices of 4096 values, one per wave of

@@ -133,27 +133,31 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
     }
 }
 
-// Merge of the key chunks of attn_decode_kernel: chunks in order with a running maximum (a fixed summation order);
-// one workgroup per query head, one thread per value; loads in batches of eight so that their latencies overlap.
+// Merge of the key chunks of attn_decode_kernel: one workgroup per query head, two threads per value - one takes the
+// even chunks, one the odd ones, each with a running maximum over its chunks in order, then the two meet in LDS (a
+// fixed summation order).  A thread issues the loads of 16 chunks before it uses the first, so a context of up to
+// 1024 keys costs one round trip to memory.
 // A separate launch on purpose: publishing the partial results to another workgroup inside one kernel needs
 // device-scope fences, which cost several times this kernel on a part with one L2 per XCD.
 template <int D>
-__global__ void __launch_bounds__(D) attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int chunks) {
-    const int h = blockIdx.x, d = threadIdx.x;
+__global__ void __launch_bounds__(2 * D) attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int chunks) {
+    constexpr int U = 16;
+    __shared__ float sm[3][D];
+    const int h = blockIdx.x, d = threadIdx.x % D, half = threadIdx.x / D;
     const float *p = part + (size_t)h * chunks * (D + 2);
     float m = -INFINITY, l = 0.f, acc = 0.f;
-    for (int c0 = 0; c0 < chunks; c0 += 8) {
-        float mm[8], ll[8], aa[8];
+    for (int c0 = half; c0 < chunks; c0 += 2 * U) {
+        float mm[U], ll[U], aa[U];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const float *pc = p + (size_t)min(c0 + u, chunks - 1) * (D + 2);
+        for (int u = 0; u < U; ++u) {
+            const float *pc = p + (size_t)min(c0 + 2 * u, chunks - 1) * (D + 2);
             mm[u] = pc[D];
             ll[u] = pc[D + 1];
             aa[u] = pc[d];
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            if (c0 + u < chunks) {
+        for (int u = 0; u < U; ++u) {
+            if (c0 + 2 * u < chunks) {
                 const float mn = fmaxf(m, mm[u]);
                 const float a = __expf(m - mn), b = __expf(mm[u] - mn);
                 l = l * a + ll[u] * b;
@@ -162,7 +166,22 @@ __global__ void __launch_bounds__(D) attn_merge_kernel(const float *__restrict__
             }
         }
     }
-    out[(size_t)h * D + d] = acc / l;
+    if (half == 1) {
+        sm[0][d] = m;
+        sm[1][d] = l;
+        sm[2][d] = acc;
+    }
+    __syncthreads();
+    if (half == 0) {
+        const float m1 = sm[0][d], l1 = sm[1][d], a1 = sm[2][d];
+        if (m1 > -INFINITY) {  // the odd half saw at least one chunk
+            const float mn = fmaxf(m, m1);
+            const float a = __expf(m - mn), b = __expf(m1 - mn);
+            l = l * a + l1 * b;
+            acc = acc * a + a1 * b;
+        }
+        out[(size_t)h * D + d] = acc / l;
+    }
 }
 
 // y = silu(gate) * up, silu(v) = v / (1 + exp(-v))   (F.swiglu, F.java:1159-1161; ops/RefMath.java:114)

@@ -198,8 +198,8 @@ struct XregCall {
     float eps = 0.f;
 };
 
-int launch_xreg(const XregCall &c, hipStream_t stream) {
-    XregArgs a{};
+// kernel arguments of a call; returns the total number of rows
+int xreg_args(const XregCall &c, XregArgs &a) {
     int n = 0;
     for (int i = 0; i < 3; ++i) {
         a.w[i] = c.w[i] ? c.w[i]->dev : c.w[0]->dev;
@@ -214,6 +214,12 @@ int launch_xreg(const XregCall &c, hipStream_t stream) {
     a.eps = c.eps;
     a.k = c.w[0]->k;
     a.nib = g.nib;
+    return n;
+}
+
+int launch_xreg(const XregCall &c, hipStream_t stream) {
+    XregArgs a{};
+    const int n = xreg_args(c, a);
     const int threads = XREG_THREADS, waves = threads / 64;
     int blocks = (n + waves - 1) / waves;
     // Two workgroups (eight waves) per CU measured best for streaming: fewer, longer row streams keep HBM pages
@@ -225,6 +231,43 @@ int launch_xreg(const XregCall &c, hipStream_t stream) {
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
     const int mode = c.w2 ? 3 : c.norm_w ? 2 : c.bias ? 1 : 0;
     hipLaunchKernelGGL(pick_xreg(c.w[0]->fmt, a.k % 64 == 0, mode, pf), dim3(blocks), dim3(threads), 0, stream, a);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+typedef void (*xreg2_fn)(const XregArgs, const XregArgs, int);
+
+// the pairs of K-quant formats a Q4_K_M / Q5_K_M layer mixes, first format < second
+template <int PF>
+xreg2_fn pick_xreg2_pf(int fa, int fb) {
+    if (fa == F_Q4_K && fb == F_Q6_K) return gemv_xreg2_kernel<Unit<F_Q4_K>, 1, Unit<F_Q6_K>, 0, PF>;
+    if (fa == F_Q4_K && fb == F_Q5_K) return gemv_xreg2_kernel<Unit<F_Q4_K>, 1, Unit<F_Q5_K>, 0, PF>;
+    if (fa == F_Q5_K && fb == F_Q6_K) return gemv_xreg2_kernel<Unit<F_Q5_K>, 0, Unit<F_Q6_K>, 0, PF>;
+    return nullptr;
+}
+
+bool xreg2_ok(int fa, int fb) { return pick_xreg2_pf<1>(fa < fb ? fa : fb, fa < fb ? fb : fa) != nullptr; }
+
+// Two calls of different formats over the same normalised activations in one launch; the workgroups are shared out
+// by the bytes each call streams.
+int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
+    const bool swap = c0.w[0]->fmt > c1.w[0]->fmt;
+    const XregCall &ca = swap ? c1 : c0, &cb = swap ? c0 : c1;
+    XregArgs a{}, b{};
+    const int na = xreg_args(ca, a), nb = xreg_args(cb, b);
+    const int waves = XREG_THREADS / 64;
+    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : 2);
+    const double ba = (double)na * ca.w[0]->nbytes / ca.w[0]->n, bb = (double)nb * cb.w[0]->nbytes / cb.w[0]->n;
+    int blocks_a = (int)(cap * ba / (ba + bb) + 0.5), blocks_b;
+    if (blocks_a < 1) blocks_a = 1;
+    if (blocks_a > cap - 1) blocks_a = cap - 1;
+    blocks_b = cap - blocks_a;
+    if (blocks_a > (na + waves - 1) / waves) blocks_a = (na + waves - 1) / waves;
+    if (blocks_b > (nb + waves - 1) / waves) blocks_b = (nb + waves - 1) / waves;
+    const int rpw_a = (na + blocks_a * waves - 1) / (blocks_a * waves), rpw_b = (nb + blocks_b * waves - 1) / (blocks_b * waves);
+    const int pf = g.xreg_pf > 0 ? g.xreg_pf : ((rpw_a > rpw_b ? rpw_a : rpw_b) >= 16 ? 1 : 2);
+    xreg2_fn fn = pf == 1 ? pick_xreg2_pf<1>(ca.w[0]->fmt, cb.w[0]->fmt) : pick_xreg2_pf<2>(ca.w[0]->fmt, cb.w[0]->fmt);
+    hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(XREG_THREADS), 0, stream, a, b, blocks_a);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
@@ -827,7 +870,7 @@ void launch_attention(const jitnn_hip_llama *m, int layer, int pos, hipStream_t 
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
     hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->k, m->v, m->kc + lo, m->vc + lo, m->cosv, m->sinv,
                        m->part, m->heads, m->kv, pos, 1.0f / sqrtf((float)D));
-    hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(m->heads), dim3(D), 0, st, m->part, m->att, chunks);
+    hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(m->heads), dim3(2 * D), 0, st, m->part, m->att, chunks);
 }
 
 bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !g.force_lds; }
@@ -837,30 +880,37 @@ bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !g.force_lds; }
 // a separate RMSNorm and the general GEMV.
 int normed_linears(const jitnn_hip_llama *m, const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, const float *nw,
                    hipStream_t st) {
-    bool normed = false;
+    // runs of neighbours of one format and row length the register-resident kernel takes
+    XregCall calls[3];
+    int ncalls = 0;
+    bool all = true;
     for (int i = 0; i < count;) {
-        if (xreg_ok(ws[i])) {
-            XregCall c;
-            int j = 0;
-            while (i + j < count && j < 3 && xreg_ok(ws[i + j]) && ws[i + j]->fmt == ws[i]->fmt && ws[i + j]->k == ws[i]->k) {
-                c.w[j] = ws[i + j];
-                c.y[j] = ys[i + j];
-                ++j;
-            }
-            c.x = x;
-            c.norm_w = nw;
-            c.eps = m->eps;
-            if (int rc = launch_xreg(c, st)) return rc;
-            i += j;
-        } else {
-            if (!normed) {
-                hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, x, nw, m->xn, m->d, m->eps);
-                normed = true;
-            }
-            if (int rc = launch_gemv(ws[i], m->xn, 1, nullptr, ys[i], st)) return rc;
-            ++i;
+        if (!xreg_ok(ws[i])) {
+            all = false;
+            break;
         }
+        XregCall &c = calls[ncalls++];
+        int j = 0;
+        while (i + j < count && j < 3 && xreg_ok(ws[i + j]) && ws[i + j]->fmt == ws[i]->fmt && ws[i + j]->k == ws[i]->k) {
+            c.w[j] = ws[i + j];
+            c.y[j] = ys[i + j];
+            ++j;
+        }
+        c.x = x;
+        c.norm_w = nw;
+        c.eps = m->eps;
+        i += j;
     }
+    if (all) {
+        if (ncalls == 2 && calls[0].w[0]->k == calls[1].w[0]->k && calls[0].w[0]->k % 256 == 0 && xreg2_ok(calls[0].w[0]->fmt, calls[1].w[0]->fmt))
+            return launch_xreg2(calls[0], calls[1], st);
+        for (int c = 0; c < ncalls; ++c)
+            if (int rc = launch_xreg(calls[c], st)) return rc;
+        return JITNN_HIP_OK;
+    }
+    hipLaunchKernelGGL(rms_norm_kernel, dim3(1), dim3(256), 0, st, x, nw, m->xn, m->d, m->eps);
+    for (int i = 0; i < count; ++i)
+        if (int rc = launch_gemv(ws[i], m->xn, 1, nullptr, ys[i], st)) return rc;
     return JITNN_HIP_OK;
 }
 
