@@ -418,26 +418,48 @@ int workspace_done(hipStream_t stream) {
 }
 
 template <int FMT>
-void launch_prefill_fmt(const jitnn_hip_weight *w, const _Float16 *xh, const float *inv, int rows, const float *bias, float *y, hipStream_t s) {
-    dim3 grid((w->n + PF_BN - 1) / PF_BN, (rows + PF_BM - 1) / PF_BM);
-    hipLaunchKernelGGL(prefill_mfma_kernel<FMT>, grid, dim3(256), 0, s, w->dev, xh, inv, bias, y, rows, w->n, w->k);
+void launch_prefill_fmt(const jitnn_hip_weight *w, const _Float16 *xo, const float *inv, int rows, const float *bias, float *y, int splits,
+                        int split_steps, hipStream_t s) {
+    dim3 grid((w->n + PF_BN - 1) / PF_BN, (rows + PF_BM - 1) / PF_BM, splits);
+    hipLaunchKernelGGL(prefill_mfma_kernel<FMT>, grid, dim3(256), 0, s, w->dev, xo, inv, bias, y, rows, w->n, w->k, split_steps);
 }
 
-// rows > 8: FP16 activations + dequantise-to-LDS MFMA kernel
+// more rows than the GEMV kernels take: FP16 activations in operand order + dequantise-to-LDS MFMA kernel
 int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
-    const size_t xh_bytes = ((size_t)rows * w->k * 2 + 255) & ~(size_t)255;
+    const int mtiles = (rows + PF_BM - 1) / PF_BM, mblocks = mtiles * (PF_BM / 32);  // operands padded to whole tiles of tokens
+    const int ntiles = (w->n + PF_BN - 1) / PF_BN, nsteps = (w->k + PF_BK - 1) / PF_BK;
+    // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 16 steps writes its own
+    // partial y, a second kernel adds the slices in order.
+    int splits = 1;
+    if (w->n % 4 == 0) {
+        while (splits < 8 && ntiles * mtiles * splits * 2 <= g.cus && nsteps / (splits * 2) >= 16) splits *= 2;
+    }
+    const int split_steps = (nsteps + splits - 1) / splits;
+    const size_t xo_bytes = (size_t)mblocks * pf_ksteps(w->k) * 1024;
+    const size_t scale_bytes = ((size_t)rows * 8 + 255) & ~(size_t)255;
+    const size_t part_bytes = splits > 1 ? (size_t)splits * rows * w->n * 4 : 0;
     void *ws = nullptr;
-    if (int rc = workspace(xh_bytes + (size_t)rows * 4, stream, &ws)) return rc;
-    _Float16 *xh = (_Float16 *)ws;
-    float *inv = (float *)((uint8_t *)ws + xh_bytes);
-    hipLaunchKernelGGL(x_to_f16_kernel, dim3(rows), dim3(256), 0, stream, x, xh, inv, w->k);
+    if (int rc = workspace(xo_bytes + scale_bytes + part_bytes, stream, &ws)) return rc;
+    _Float16 *xo = (_Float16 *)ws;
+    float *scale = (float *)((uint8_t *)ws + xo_bytes), *inv = scale + rows;
+    float *part = (float *)((uint8_t *)ws + xo_bytes + scale_bytes);
+    hipLaunchKernelGGL(x_row_scale_kernel, dim3(rows), dim3(256), 0, stream, x, scale, inv, w->k);
+    hipLaunchKernelGGL(x_to_operand_kernel, dim3(mblocks, pf_ksteps(w->k) / 4), dim3(256), 0, stream, x, scale, xo, rows, w->k);
+    float *out = splits > 1 ? part : y;
+    const float *b1 = splits > 1 ? nullptr : bias;
     switch (w->fmt) {
-    case F_Q4_0: launch_prefill_fmt<F_Q4_0>(w, xh, inv, rows, bias, y, stream); break;
-    case F_Q4_1: launch_prefill_fmt<F_Q4_1>(w, xh, inv, rows, bias, y, stream); break;
-    case F_Q8_0: launch_prefill_fmt<F_Q8_0>(w, xh, inv, rows, bias, y, stream); break;
-    case F_Q4_K: launch_prefill_fmt<F_Q4_K>(w, xh, inv, rows, bias, y, stream); break;
-    case F_Q5_K: launch_prefill_fmt<F_Q5_K>(w, xh, inv, rows, bias, y, stream); break;
-    default: launch_prefill_fmt<F_Q6_K>(w, xh, inv, rows, bias, y, stream); break;
+    case F_Q4_0: launch_prefill_fmt<F_Q4_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q4_1: launch_prefill_fmt<F_Q4_1>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q8_0: launch_prefill_fmt<F_Q8_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q4_K: launch_prefill_fmt<F_Q4_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q5_K: launch_prefill_fmt<F_Q5_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    default: launch_prefill_fmt<F_Q6_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    }
+    if (splits > 1) {
+        const size_t count4 = (size_t)rows * w->n / 4;
+        size_t blocks = (count4 + 255) / 256;
+        if (blocks > (size_t)g.cus * 8) blocks = (size_t)g.cus * 8;
+        hipLaunchKernelGGL(prefill_join_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, part, bias, y, count4, w->n, splits);
     }
     HIP_TRY(hipGetLastError());
     return workspace_done(stream);

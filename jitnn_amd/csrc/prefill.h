@@ -1,14 +1,18 @@
 // Many-row linear (prefill, batches beyond the GEMV range) on raw GGUF blocks: y[M, N] = x[M, K] W[N, K]^T.
 //
 // This is the one shape on the path that is a real dense contraction, so it runs on the matrix cores:
-//   1. x_to_f16_kernel turns each activation row into FP16 with a power-of-two row scale that puts its largest
-//      magnitude in [2^13, 2^14) (no overflow for any FP32 input, no loss of small rows to FP16 subnormals);
-//   2. prefill_mfma_kernel: a workgroup of four waves owns a 128 (weight rows) x 128 (tokens) output tile and
-//      walks K in steps of 64.  Per step every thread dequantises 32 weights of one row from the raw blocks
-//      (FP32 arithmetic of the dequantiser, then one rounding to FP16) into LDS, the FP16 activations of the
-//      step are copied beside them, and each wave issues 16 v_mfma_f32_32x32x16_f16 on its 64 x 64 quadrant,
-//      accumulating in FP32; the loads of the next step are in flight meanwhile.  The epilogue undoes the row
-//      scale and adds the bias.
+//   1. x_row_scale_kernel finds, per activation row, the power-of-two scale that puts its largest magnitude in
+//      [2^13, 2^14) (no overflow for any FP32 input, no loss of small rows to FP16 subnormals), and
+//      x_to_operand_kernel writes the scaled FP16 activations in the order the matrix cores consume them: 1 KiB per
+//      (block of 32 tokens, step of 16 K values), 16 bytes per lane - a wave's B operand is one fully coalesced
+//      128-bit load from L2, no LDS involved;
+//   2. prefill_mfma_kernel: a workgroup of four waves owns a 128 (weight rows) x 256 (tokens) output tile and
+//      walks K in steps of 64.  Per step every thread dequantises 32 weights of one row from the raw blocks into a
+//      double-buffered LDS tile as FP16, and each wave issues 32 v_mfma_f32_32x32x16_f16 on its 128 x 64 slice
+//      (weight operands from LDS, each used twice; activation operands from registers loaded two steps ahead, each
+//      used four times - the shape that keeps both LDS and the vector L1 at half their bandwidth), accumulating in
+//      FP32; the raw weight bytes are requested two steps ahead and decoded after the MFMAs are issued.  The epilogue
+//      undoes the row scale and adds the bias.
 // Both FP16 roundings are relative 2^-11, so the result stays well inside the 2e-3 bar of the MFMA path.
 #pragma once
 #include "common.h"
@@ -18,34 +22,56 @@ namespace jitnn {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int PF_BN = 128, PF_BM = 128, PF_BK = 64, PF_LD = PF_BK + 8;  // LDS row pitch in halves: 144 bytes, conflict-free 16-byte reads
+constexpr int PF_BN = 128, PF_BM = 256, PF_BK = 64, PF_LD = PF_BK + 8;  // LDS row pitch in halves: 144 bytes, conflict-free 16-byte reads
 
 // position of value i (0..3) of a group of four in the FP16 operands: 0, 2, 1, 3
 __host__ __device__ constexpr int pf_perm4(int i) { return ((i & 1) << 1) | (i >> 1); }
 
-// One workgroup per activation row: amax, scale = 2^(13 - floor(log2 amax)), FP16 copy, 1/scale for the epilogue.
-__global__ void __launch_bounds__(256) x_to_f16_kernel(const float *__restrict__ x, _Float16 *__restrict__ xh, float *__restrict__ inv_scale,
-                                                        int k) {
+// One workgroup per activation row: amax -> scale = 2^(13 - floor(log2 amax)) and 1/scale for the epilogue.
+__global__ void __launch_bounds__(256) x_row_scale_kernel(const float *__restrict__ x, float *__restrict__ scale, float *__restrict__ inv_scale,
+                                                           int k) {
     __shared__ float red[4];
-    const float *xr = x + (size_t)blockIdx.x * k;
+    const float4 *xr = reinterpret_cast<const float4 *>(x + (size_t)blockIdx.x * k);  // k is a multiple of 32
     float m = 0.f;
-    for (int i = threadIdx.x; i < k; i += 256) m = fmaxf(m, fabsf(xr[i]));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    for (int i = threadIdx.x; i < (k >> 2); i += 256) {
+        const float4 v = xr[i];
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w))));
+    }
+    m = wave_max(m);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
     __syncthreads();
     m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    float scale = 1.f;
+    float sc = 1.f;
     if (m > 0.f && m < 3.0e38f) {
         int e;
         frexpf(m, &e);  // m = f * 2^e, f in [0.5, 1)
-        scale = ldexpf(1.f, 14 - e);
+        sc = ldexpf(1.f, 14 - e);
     }
-    // within each group of four values the FP16 copy is stored in the order 0, 2, 1, 3 - the order in which the weight
-    // decoder produces FP16 pairs from a dword of quants (bytes 0 and 2, then 1 and 3); a dot product does not care
-    _Float16 *o = xh + (size_t)blockIdx.x * k;
-    for (int i = threadIdx.x; i < k; i += 256) o[(i & ~3) | pf_perm4(i & 3)] = (_Float16)(xr[i] * scale);
-    if (threadIdx.x == 0) inv_scale[blockIdx.x] = 1.f / scale;
+    if (threadIdx.x == 0) {
+        scale[blockIdx.x] = sc;
+        inv_scale[blockIdx.x] = 1.f / sc;
+    }
+}
+
+// Number of 16-value K steps the operand array holds per token block: K rounded up to whole steps of PF_BK.
+__host__ __device__ constexpr int pf_ksteps(int k) { return (k + PF_BK - 1) / PF_BK * (PF_BK / 16); }
+
+// FP16 activations in matrix-core operand order: xo[token block mb][K step ks][lane][8], lane l holding token
+// 32 mb + l % 32, values 16 ks + 8 (l / 32) .. + 7, each group of four values in the order 0, 2, 1, 3 (the order in
+// which the weight decoder produces FP16 pairs from a dword of quants; a dot product only needs both to agree).
+// Tokens past m and values past k are zeros.  grid (token blocks, K / 64), 256 threads: one 16-byte piece each.
+__global__ void __launch_bounds__(256) x_to_operand_kernel(const float *__restrict__ x, const float *__restrict__ scale,
+                                                            _Float16 *__restrict__ xo, int m, int k) {
+    const int lane = threadIdx.x & 63, ks = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int tok = blockIdx.x * 32 + (lane & 31), kk = 16 * ks + 8 * (lane >> 5);
+    f16x8 o = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (tok < m && kk < k) {
+        const float sc = scale[tok];
+        const float4 a = *reinterpret_cast<const float4 *>(x + (size_t)tok * k + kk), b = *reinterpret_cast<const float4 *>(x + (size_t)tok * k + kk + 4);
+        o = f16x8{(_Float16)(a.x * sc), (_Float16)(a.z * sc), (_Float16)(a.y * sc), (_Float16)(a.w * sc),
+                  (_Float16)(b.x * sc), (_Float16)(b.z * sc), (_Float16)(b.y * sc), (_Float16)(b.w * sc)};
+    }
+    reinterpret_cast<f16x8 *>(xo)[((size_t)blockIdx.x * pf_ksteps(k) + ks) * 64 + lane] = o;
 }
 
 // 32 consecutive weights of a row, starting at value k0 (k0 % 32 == 0), in two phases so that the loads of the next
@@ -181,6 +207,14 @@ __device__ __forceinline__ void pf_decode(const PfRaw<FMT> &r, int k0, float (&o
 typedef union { uint32_t u; f16x2 h; } pf_h2;
 
 __device__ __forceinline__ f16x2 pf_pair(uint32_t u) { pf_h2 t; t.u = u; return t.h; }
+__device__ __forceinline__ uint32_t pf_bits(f16x2 h) { pf_h2 t; t.h = h; return t.u; }
+// 0x64006400 (FP16 1024.0 twice) held in a VGPR, so that (v & mask) | magic is a single v_and_or_b32: the instruction
+// takes one scalar or literal operand only, and the mask is one already
+__device__ __forceinline__ uint32_t pf_magic() {
+    uint32_t m = 0x64006400u;
+    asm("" : "+v"(m));
+    return m;
+}
 
 template <int FMT>
 __device__ __forceinline__ void pf_decode_h(const PfRaw<FMT> &r, int k0, f16x8 (&o)[4]);
@@ -190,28 +224,31 @@ __device__ __forceinline__ void pf_decode_h<F_Q4_K>(const PfRaw<F_Q4_K> &r, int 
     const int e = k0 & 255, j = e >> 6, half = (e >> 5) & 1, sub = 2 * j + half;
     int sc, mn;
     {
+        // the eight 6-bit scales and mins bytewise, then this thread's pair by a shift: no branch, so that the decode
+        // stays in the basic block of the MFMAs it is interleaved with
         const uint32_t s0 = r.h.y, s1 = r.h.z, s2 = r.h.w;
+        const uint32_t scA = s0 & 0x3f3f3f3fu, scB = (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u);
+        const uint32_t mnA = s1 & 0x3f3f3f3fu, mnB = ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u);
         const int sh = 8 * (sub & 3);
-        if (sub < 4) {
-            sc = (s0 >> sh) & 63;
-            mn = (s1 >> sh) & 63;
-        } else {
-            sc = ((s2 >> sh) & 15) | (((s0 >> sh) >> 6 & 3) << 4);
-            mn = ((s2 >> sh) >> 4 & 15) | (((s1 >> sh) >> 6 & 3) << 4);
-        }
+        sc = ((sub < 4 ? scA : scB) >> sh) & 0xff;
+        mn = ((sub < 4 ? mnA : mnB) >> sh) & 0xff;
     }
     const _Float16 ds = (_Float16)(h2f(r.h.x) * (float)sc), nm = (_Float16)(-(h2f(r.h.x >> 16) * (float)mn));
     const f16x2 ds2 = {ds, ds}, nm2 = {nm, nm}, off = {(_Float16)-1024.f, (_Float16)-1024.f};
+    const uint32_t mg = pf_magic();
 #pragma unroll
-    for (int w = 0; w < 8; ++w) {
-        const uint32_t v = (w < 4 ? r.q0[w] : r.q1[w - 4]) >> (4 * half);
-        const f16x2 a = pf_pair((v & 0x000f000fu) | 0x64006400u) + off;         // bytes 0, 2
-        const f16x2 b = pf_pair(((v >> 8) & 0x000f000fu) | 0x64006400u) + off;  // bytes 1, 3
-        const f16x2 wa = a * ds2 + nm2, wb = b * ds2 + nm2;
-        o[w >> 1][4 * (w & 1) + 0] = wa.x;
-        o[w >> 1][4 * (w & 1) + 1] = wa.y;
-        o[w >> 1][4 * (w & 1) + 2] = wb.x;
-        o[w >> 1][4 * (w & 1) + 3] = wb.y;
+    for (int c = 0; c < 4; ++c) {
+        u32x4 out;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int w = 2 * c + t;
+            const uint32_t v = (w < 4 ? r.q0[w] : r.q1[w - 4]) >> (4 * half);
+            const f16x2 a = pf_pair((v & 0x000f000fu) | mg) + off;         // bytes 0, 2
+            const f16x2 b = pf_pair(((v >> 8) & 0x000f000fu) | mg) + off;  // bytes 1, 3
+            out[2 * t] = pf_bits(__builtin_elementwise_fma(a, ds2, nm2));
+            out[2 * t + 1] = pf_bits(__builtin_elementwise_fma(b, ds2, nm2));
+        }
+        o[c] = __builtin_bit_cast(f16x8, out);
     }
 }
 
@@ -221,131 +258,179 @@ __device__ __forceinline__ void pf_decode_h<F_Q6_K>(const PfRaw<F_Q6_K> &r, int 
     const float d = h2f(r.d);
     const _Float16 a0 = (_Float16)(d * (float)(int)(int8_t)(r.sc & 0xffu)), a1 = (_Float16)(d * (float)(int)(int8_t)(r.sc >> 8));
     const f16x2 off = {(_Float16)-1056.f, (_Float16)-1056.f};  // -1024 of the exponent trick, -32 of the format
+    const uint32_t mg = pf_magic();
 #pragma unroll
-    for (int w = 0; w < 8; ++w) {
-        const uint32_t lw = (w < 4 ? r.l0[w] : r.l1[w - 4]) >> (kk < 2 ? 0 : 4);
-        const uint32_t hw = (w < 4 ? r.h0[w] : r.h1[w - 4]) >> (2 * kk);
-        const uint32_t q = (lw & 0x0f0f0f0fu) | ((hw << 4) & 0x30303030u);  // four 6-bit quants, one per byte
-        const f16x2 sc2 = w < 4 ? f16x2{a0, a0} : f16x2{a1, a1};
-        const f16x2 a = (pf_pair((q & 0x00ff00ffu) | 0x64006400u) + off) * sc2;         // bytes 0, 2
-        const f16x2 b = (pf_pair(((q >> 8) & 0x00ff00ffu) | 0x64006400u) + off) * sc2;  // bytes 1, 3
-        o[w >> 1][4 * (w & 1) + 0] = a.x;
-        o[w >> 1][4 * (w & 1) + 1] = a.y;
-        o[w >> 1][4 * (w & 1) + 2] = b.x;
-        o[w >> 1][4 * (w & 1) + 3] = b.y;
+    for (int c = 0; c < 4; ++c) {
+        u32x4 out;
+        const f16x2 sc2 = c < 2 ? f16x2{a0, a0} : f16x2{a1, a1};
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int w = 2 * c + t;
+            const uint32_t lw = (w < 4 ? r.l0[w] : r.l1[w - 4]) >> (kk < 2 ? 0 : 4);
+            const uint32_t hw = (w < 4 ? r.h0[w] : r.h1[w - 4]) >> (2 * kk);
+            const uint32_t q = (lw & 0x0f0f0f0fu) | ((hw << 4) & 0x30303030u);  // four 6-bit quants, one per byte
+            out[2 * t] = pf_bits((pf_pair((q & 0x00ff00ffu) | mg) + off) * sc2);             // bytes 0, 2
+            out[2 * t + 1] = pf_bits((pf_pair(((q >> 8) & 0x00ff00ffu) | mg) + off) * sc2);  // bytes 1, 3
+        }
+        o[c] = __builtin_bit_cast(f16x8, out);
     }
 }
 
 template <int FMT>
-__global__ void __launch_bounds__(256) prefill_mfma_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xh,
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xo,
                                                             const float *__restrict__ inv_scale, const float *__restrict__ bias,
-                                                            float *__restrict__ y, int m, int n, int k) {
-    __shared__ _Float16 As[PF_BN * PF_LD];  // dequantised weights  [row][k]
-    __shared__ _Float16 Bs[PF_BM * PF_LD];  // activations          [token][k]
+                                                            float *__restrict__ y, int m, int n, int k, int split_steps) {
+    __shared__ _Float16 As[2][PF_BN * PF_LD];  // dequantised weights [row][k], two steps
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n0 = blockIdx.x * PF_BN, m0 = blockIdx.y * PF_BM;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
     // dequantiser role: thread t fills weights [row t/2][32 * (t%2) ... +32) of the step
     const int drow = tid >> 1, dhalf = tid & 1;
     const uint8_t *wrow = W + (size_t)min(n0 + drow, n - 1) * rowbytes;
-    // copier role: thread t copies 32 halves of token t/2
-    const int xtok = min(m0 + drow, m - 1);
-    const bool xlive = m0 + drow < m;
-    const _Float16 *xrow = xh + (size_t)xtok * k;
-    // MFMA role: wave (wr, wc) owns output rows [64 wr, +64) x tokens [64 wc, +64) as 2 x 2 tiles of 32 x 32
-    const int wr = wave >> 1, wc = wave & 1;
-    f32x16 acc[2][2];
+    // MFMA role: wave w owns all 128 output rows x tokens [64 w, +64) as 4 x 2 tiles of 32 x 32: every weight operand
+    // read from LDS feeds two MFMAs, every activation operand loaded from L2 feeds four
+    const int ksteps = pf_ksteps(k);
+    // B operands of token blocks m0/32 + 2 w + {0, 1}: 16 bytes per lane, consecutive K steps 1 KiB apart (the operand
+    // array is padded to whole tiles of PF_BM tokens, so both blocks exist)
+    const f16x8 *xb = reinterpret_cast<const f16x8 *>(xo) + ((size_t)(m0 / 32 + 2 * wave) * ksteps) * 64 + lane;
+    f32x16 acc[4][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // Software pipeline over K: the raw weight bytes and the FP16 activations of step s+1 are loaded while the matrix
-    // cores work on step s, and decoded into registers (ah, bh) after the MFMAs have been issued.
-    f16x8 ah[4], bh[4];
-    PfRaw<FMT> raw;
-    auto fetch = [&](int k0) {  // issue the global loads of one step for this thread
-        const int kk = k0 + 32 * dhalf;
-        if (kk < k) {
-            pf_load<FMT>(raw, wrow, kk);
-            const f16x8 *src = reinterpret_cast<const f16x8 *>(xrow + kk);
+    // Software pipeline over K: the raw weight bytes and the B operands of a step are requested two steps ahead (a
+    // step of 32 MFMAs per wave is shorter than a trip to HBM); the weights of step s+1 are decoded into registers
+    // (ah) after the MFMAs of step s have been issued.  raw[] alternates, the B operands rotate through three sets,
+    // the LDS tile through two: the loop is unrolled six steps so that all of them are fixed registers.
+    // Nothing in a step is conditional - requests past the last step repeat the last step, a half step past the end
+    // of a row (K = 32 mod 64) re-reads the row's last block and meets the zeros the operand array holds there - so
+    // that the compiler can count the outstanding loads exactly and a step waits only for the loads it consumes.
+    f16x8 ah[4];
+    PfRaw<FMT> raw[2];
+    f16x8 bq[3][2][4];
+    // this workgroup's K steps: all of them, or slice blockIdx.z of split_steps steps when the launch splits K (then y
+    // is the slice's own [m, n] array of partial sums, to be added up by prefill_join_kernel)
+    const int sbeg = blockIdx.z * split_steps, nsteps = min((k + PF_BK - 1) / PF_BK, sbeg + split_steps);
+    y += (size_t)blockIdx.z * m * n;
+    auto wk = [&](int s) { return min(min(s, nsteps - 1) * PF_BK + 32 * dhalf, k - 32); };  // first value this thread decodes in step s
+    auto fetch_w = [&](PfRaw<FMT> &r, int s) { pf_load<FMT>(r, wrow, wk(s)); };
+    auto fetch_b = [&](f16x8(&b)[2][4], int s) {
+        const f16x8 *p = xb + (size_t)min(s, nsteps - 1) * 4 * 64;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) bh[c] = src[c];
-        }
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) b[j][ks] = p[((size_t)j * ksteps + ks) * 64];
     };
-    auto decode = [&](int k0) {  // raw -> FP16 registers, values of each group of four in the order 0, 2, 1, 3
-        const int kk = k0 + 32 * dhalf;
-        if (kk < k) {
-            if constexpr (FMT == F_Q4_K || FMT == F_Q6_K) {
-                pf_decode_h<FMT>(raw, kk, ah);
-            } else {
-                float v[32];
-                pf_decode<FMT>(raw, kk, v);
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) ah[c][(i & ~3) | pf_perm4(i & 3)] = (_Float16)v[8 * c + i];
-            }
+    auto decode = [&](const PfRaw<FMT> &r, int s) {  // raw -> FP16 registers, values of each group of four in the order 0, 2, 1, 3
+        const int kk = wk(s);
+
+        if constexpr (FMT == F_Q4_K || FMT == F_Q6_K) {
+            pf_decode_h<FMT>(r, kk, ah);
         } else {
+            float v[32];
+            pf_decode<FMT>(r, kk, v);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) ah[c] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ah[c][(i & ~3) | pf_perm4(i & 3)] = (_Float16)v[8 * c + i];
         }
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-            if (!(xlive && kk < k)) bh[c] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     };
-    fetch(0);
-    decode(0);
-    for (int k0 = 0; k0 < k; k0 += PF_BK) {
+    // one K step: publish the decoded weights, request the loads of step s+2, multiply, decode step s+1
+    auto step = [&](int s, int buf, f16x8(&bcur)[2][4], f16x8(&bfar)[2][4], PfRaw<FMT> &rfar, const PfRaw<FMT> &rnext) {
         {
-            f16x8 *da = reinterpret_cast<f16x8 *>(&As[drow * PF_LD + 32 * dhalf]);
-            f16x8 *db = reinterpret_cast<f16x8 *>(&Bs[drow * PF_LD + 32 * dhalf]);
+            f16x8 *da = reinterpret_cast<f16x8 *>(&As[buf][drow * PF_LD + 32 * dhalf]);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                da[c] = ah[c];
-                db[c] = bh[c];
-            }
+            for (int c = 0; c < 4; ++c) da[c] = ah[c];
         }
-        __syncthreads();
-        const bool more = k0 + PF_BK < k;
-        if (more) fetch(k0 + PF_BK);
-        // ---- 4 k-substeps of 16: lane l supplies row/token l%32, halves 8*(l/32) .. +8 of the substep
+        __syncthreads();  // the one barrier of the step: the other buffer was read before the previous one
+        fetch_w(rfar, s + 2);
+        fetch_b(bfar, s + 2);
+        // ---- 4 k-substeps of 16: lane l supplies row l%32, halves 8*(l/32) .. +8 of the substep.  The weight operands
+        // of a substep are read from LDS while the MFMAs of the one before run (one wave per SIMD: nobody else hides
+        // the LDS latency).
+        const _Float16 *ap = &As[buf][(lane & 31) * PF_LD + 8 * (lane >> 5)];
+        f16x8 a[2][4];
 #pragma unroll
-        for (int ks = 0; ks < PF_BK; ks += 16) {
-            f16x8 a[2], b[2];
+        for (int i = 0; i < 4; ++i) a[0][i] = *reinterpret_cast<const f16x8 *>(ap + 32 * i * PF_LD);
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                a[i] = *reinterpret_cast<const f16x8 *>(&As[(64 * wr + 32 * i + (lane & 31)) * PF_LD + ks + 8 * (lane >> 5)]);
-                b[i] = *reinterpret_cast<const f16x8 *>(&Bs[(64 * wc + 32 * i + (lane & 31)) * PF_LD + ks + 8 * (lane >> 5)]);
+        for (int ks = 0; ks < 4; ++ks) {
+            if (ks < 3) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[(ks + 1) & 1][i] = *reinterpret_cast<const f16x8 *>(ap + 32 * i * PF_LD + 16 * (ks + 1));
             }
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bcur[j][ks], a[ks & 1][i], acc[i][j], 0, 0, 0);
         }
-        __syncthreads();
-        if (more) decode(k0 + PF_BK);
+        decode(rnext, s + 1);
+        // One wave per SIMD: nobody else fills the matrix pipe while this wave decodes, or the VALU while it multiplies.
+        // Ask the scheduler for the interleaving by hand: the step's global loads first, then one MFMA, a few decode
+        // instructions and every other time one LDS operand read, 32 times over.
+        __builtin_amdgcn_sched_group_barrier(0x020, 11, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+            if (i % 2 == 0 && i < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+    fetch_w(raw[0], sbeg);
+    fetch_b(bq[0], sbeg);
+    fetch_w(raw[1], sbeg + 1);
+    fetch_b(bq[1], sbeg + 1);
+    decode(raw[0], sbeg);
+    int s0 = sbeg;
+    for (; s0 + 6 <= nsteps; s0 += 6) {
+#pragma unroll
+        for (int u = 0; u < 6; ++u) step(s0 + u, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
     }
-    // ---- epilogue: element r of a 32 x 32 accumulator is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int u = 0; u < 5; ++u)
+        if (s0 + u < nsteps) step(s0 + u, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
+    // ---- epilogue.  The activations went in as the first MFMA operand, so an accumulator holds a 32 (tokens) x 32
+    // (weight rows) block of y: element r is token 8*(r/4) + 4*(lane/32) + r%4, weight row lane%32 - the 32 lanes of a
+    // half wave store 32 consecutive floats of one token's output row.
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = n0 + 32 * i + (lane & 31);
+        const float bv = bias && row < n ? bias[row] : 0.f;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const int tok = m0 + 64 * wc + 32 * j + (lane & 31);
-            if (tok >= m) continue;
-            const float is = inv_scale[tok];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int row = n0 + 64 * wr + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row < n) {
-                    float v = acc[i][j][r] * is;
-                    if (bias) v += bias[row];
-                    y[(size_t)tok * n + row] = v;
-                }
+                const int tok = m0 + 64 * wave + 32 * j + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (row < n && tok < m) y[(size_t)tok * n + row] = acc[i][j][r] * inv_scale[tok] + bv;
             }
         }
+    }
+}
+
+// y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]), slices in order: the second half of a
+// split-K launch.  count4 = m * n / 4 (n is a multiple of 4 whenever the launch splits).
+__global__ void __launch_bounds__(256) prefill_join_kernel(const float *__restrict__ part, const float *__restrict__ bias, float *__restrict__ y,
+                                                            size_t count4, int n, int splits) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count4; i += (size_t)gridDim.x * 256) {
+        float4 a = reinterpret_cast<const float4 *>(part)[i];
+        for (int z = 1; z < splits; ++z) {
+            const float4 b = reinterpret_cast<const float4 *>(part)[(size_t)z * count4 + i];
+            a.x += b.x;
+            a.y += b.y;
+            a.z += b.z;
+            a.w += b.w;
+        }
+        if (bias) {
+            const float4 b = *reinterpret_cast<const float4 *>(bias + (i * 4) % (size_t)n);
+            a.x += b.x;
+            a.y += b.y;
+            a.z += b.z;
+            a.w += b.w;
+        }
+        reinterpret_cast<float4 *>(y)[i] = a;
     }
 }
 

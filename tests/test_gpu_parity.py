@@ -165,8 +165,8 @@ def test_small_k_32_blocks_and_many_rows(jn, fmt):
         assert norm_err(y, ref) <= bar(rows), (fmt, rows, norm_err(y, ref))
 
 
-PREFILL_SHAPES = [  # (n, k, rows): ragged tiles in every dimension, K past one step, a 32-value K tail
-    (256, 1024, 65), (131, 4096, 200), (64, 14336, 97), (130, 512, 129), (1, 256, 70),
+PREFILL_SHAPES = [  # (n, k, rows): ragged tiles in every dimension, K past one step, K split into 8 and into 4 slices
+    (256, 1024, 65), (131, 4096, 200), (64, 14336, 97), (130, 512, 129), (1, 256, 70), (384, 4096, 513),
 ]
 
 
@@ -194,10 +194,10 @@ def test_prefill_mfma_vs_oracle(jn, fmt, n, k, rows):
 
 
 @pytest.mark.parametrize("fmt", ["Q4_0", "Q8_0", "Q4_1"])
-def test_prefill_k_tail_of_32(jn, fmt):
+@pytest.mark.parametrize("n,k,rows", [(40, 32 * 7, 70), (132, 4096 + 32, 300)])  # the second: few tiles, so K is split into slices
+def test_prefill_k_tail_of_32(jn, fmt, n, k, rows):
     from oracle import oracle
     rng = np.random.default_rng(3)
-    n, k, rows = 40, 32 * 7, 70
     raw = random_valid_blocks(rng, fmt, n, k)
     x = rng.standard_normal((rows, k)).astype(np.float32)
     y = jn.Gguf.linear(jn.Tensor.of(x), weight(jn, fmt, raw, n, k), None).numpy()
