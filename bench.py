@@ -303,6 +303,39 @@ def bench_prefill(torch, lib, steps=20):
                      "pct_of_fp16_peak": flops / ms / 1e9 / 2500.0 * 100, "parity_norm_err": err}
         lib.lib.jitnn_hip_weight_free(h)
         del t, x, y
+    # the seven linears of one layer of config 5 on 512 tokens, back to back (attention and norms are not part of this path)
+    layer = [("Q4_K", 4096, 4096), ("Q4_K", 1024, 4096), ("Q6_K", 1024, 4096), ("Q4_K", 4096, 4096), ("Q4_K", 14336, 4096),
+             ("Q4_K", 14336, 4096), ("Q6_K", 4096, 14336)]
+    ws, hs, ys = [], [], []
+    for i, (fmt, n, k) in enumerate(layer):
+        t = quantized_device_weight(torch, lib, fmt, n, k, 1070 + i)
+        ws.append(t)
+        hs.append(wrap(lib, fmt, t, n, k))
+        ys.append(torch.empty(512, n, device="cuda"))
+    x4, x14 = torch.randn(512, 4096, device="cuda"), torch.randn(512, 14336, device="cuda")
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def one_layer():
+        for (fmt, n, k), h, y in zip(layer, hs, ys):
+            xin = x4 if k == 4096 else x14
+            lib.check(lib.lib.jitnn_hip_linear_dev(h, C.c_void_p(xin.data_ptr()), 512, None, C.c_void_p(y.data_ptr()), st), "linear")
+
+    for _ in range(3):
+        one_layer()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        one_layer()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    flops = sum(2.0 * 512 * n * k for _, n, k in layer)
+    res["layer_linears_512_tokens"] = {"workload": "q, k, v, o, gate, up, down of one 8B layer (Q4_K_M mix) on 512 tokens", "ms": ms,
+                                       "TFLOPs": flops / ms / 1e9, "pct_of_fp16_peak": flops / ms / 1e9 / 2500.0 * 100,
+                                       "tokens_per_s_32_layers_linears_only": 512.0 / (32 * ms * 1e-3)}
+    for h in hs:
+        lib.lib.jitnn_hip_weight_free(h)
     return res
 
 

@@ -62,16 +62,26 @@ __host__ __device__ constexpr int pf_ksteps(int k) { return (k + PF_BK - 1) / PF
 // Tokens past m and values past k are zeros.  grid (token blocks, K / 64), 256 threads: one 16-byte piece each.
 __global__ void __launch_bounds__(256) x_to_operand_kernel(const float *__restrict__ x, const float *__restrict__ scale,
                                                             _Float16 *__restrict__ xo, int m, int k) {
-    const int lane = threadIdx.x & 63, ks = blockIdx.y * 4 + (threadIdx.x >> 6);
-    const int tok = blockIdx.x * 32 + (lane & 31), kk = 16 * ks + 8 * (lane >> 5);
-    f16x8 o = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (tok < m && kk < k) {
-        const float sc = scale[tok];
-        const float4 a = *reinterpret_cast<const float4 *>(x + (size_t)tok * k + kk), b = *reinterpret_cast<const float4 *>(x + (size_t)tok * k + kk + 4);
-        o = f16x8{(_Float16)(a.x * sc), (_Float16)(a.z * sc), (_Float16)(a.y * sc), (_Float16)(a.w * sc),
-                  (_Float16)(b.x * sc), (_Float16)(b.z * sc), (_Float16)(b.y * sc), (_Float16)(b.w * sc)};
+    // 32 tokens x 64 values through LDS: the reads run along the token rows (256 contiguous bytes each), the writes
+    // along the operand order (1 KiB per K step)
+    __shared__ float4 tile[32][17];  // [token][16 quads + 1: the operand reads below walk down the tokens]
+    const int t = threadIdx.x, tok0 = blockIdx.x * 32, k0 = blockIdx.y * 64;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int idx = t + 256 * i, r = idx >> 4, q = idx & 15, tok = tok0 + r, kk = k0 + 4 * q;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (tok < m && kk < k) {
+            const float sc = scale[tok];
+            v = *reinterpret_cast<const float4 *>(x + (size_t)tok * k + kk);
+            v = make_float4(v.x * sc, v.y * sc, v.z * sc, v.w * sc);
+        }
+        tile[r][q] = v;
     }
-    reinterpret_cast<f16x8 *>(xo)[((size_t)blockIdx.x * pf_ksteps(k) + ks) * 64 + lane] = o;
+    __syncthreads();
+    const int lane = t & 63, ks = t >> 6;  // this thread's piece: token lane % 32, values 16 ks + 8 (lane / 32) .. + 7 of the tile
+    const float4 a = tile[lane & 31][4 * ks + 2 * (lane >> 5)], b = tile[lane & 31][4 * ks + 2 * (lane >> 5) + 1];
+    const f16x8 o = {(_Float16)a.x, (_Float16)a.z, (_Float16)a.y, (_Float16)a.w, (_Float16)b.x, (_Float16)b.z, (_Float16)b.y, (_Float16)b.w};
+    reinterpret_cast<f16x8 *>(xo)[((size_t)blockIdx.x * pf_ksteps(k) + blockIdx.y * 4 + ks) * 64 + lane] = o;
 }
 
 // 32 consecutive weights of a row, starting at value k0 (k0 % 32 == 0), in two phases so that the loads of the next
