@@ -267,11 +267,53 @@ struct MTile<F_Q8_0> {
     }
 };
 
+// Q6_K: 210-byte super-blocks (ql[128], qh[64], sixteen int8 scales, d); a scale covers 16 values, so the block sums
+// come from v_mfma_f32_16x16x16_f16, two per 32-value block.  Block b = 4 nh + qt holds values l = 0..31 with low
+// nibbles / high nibbles (qt >> 1) of ql[64 nh + 32 (qt & 1) + l] and bits 2 qt, 2 qt + 1 of qh[32 nh + l]
+// (GgufKernels.java: Q6_K decode).  The run is copied as 13 chunks of 16 bytes plus the two bytes of d.
+template <>
+struct MTile<F_Q6_K> {
+    static constexpr bool SUMS = false;
+    static constexpr int BYTES = 210;
+    __device__ static __forceinline__ void quad_pos(int tq, int &kq, int &h) { quad_pos_nib4(tq, kq, h); }  // half h = 16-value group
+    __device__ static __forceinline__ f32x4 mma(const uint8_t *p, int kq, const f16x8 (&xa)[8], const f16x8 &) {
+        const float d = h2f(sld16(p + 208));
+        const u32x4 scw = sld128(p + 192);
+        const uint32_t mg = magic1024();
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int nh = 0; nh < 2; ++nh) {
+#pragma unroll
+            for (int g = 0; g < 2; ++g) {
+                const uint32_t qh = sld32(p + 128 + 32 * nh + 16 * g + 4 * kq);
+#pragma unroll
+                for (int hb = 0; hb < 2; ++hb) {
+                    const uint32_t ql = sld32(p + 64 * nh + 32 * hb + 16 * g + 4 * kq);
+#pragma unroll
+                    for (int nib = 0; nib < 2; ++nib) {
+                        const int qt = 2 * nib + hb, b = 4 * nh + qt;
+                        const uint32_t q = ((ql >> (4 * nib)) & 0x0f0f0f0fu) | (((qh >> (2 * qt)) & 0x03030303u) << 4);  // four 6-bit quants
+                        const f16x2 a02 = magic_lo((q & 0x00ff00ffu) | mg, 32.f), a13 = magic_lo(((q >> 8) & 0x00ff00ffu) | mg, 32.f);
+                        const f16x4 bop = {a02.x, a02.y, a13.x, a13.y};
+                        const f16x4 aop = g ? f16x4{xa[b][4], xa[b][5], xa[b][6], xa[b][7]} : f16x4{xa[b][0], xa[b][1], xa[b][2], xa[b][3]};
+                        const f32x4 c = __builtin_amdgcn_mfma_f32_16x16x16f16(aop, bop, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        const int si = 8 * nh + 2 * qt + g;  // scale of values 16 g .. 16 g + 15 of block b
+                        const float ds = d * (float)(int)(int8_t)((scw[si >> 2] >> (8 * (si & 3))) & 0xffu);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc[i] = __builtin_fmaf(ds, c[i], acc[i]);
+                    }
+                }
+            }
+        }
+        return acc;
+    }
+};
+
 // Pitch of a tile row in a wave's LDS region: at least BYTES and an odd multiple of 16, so that the 16 rows of an
 // operand read (two dwords per lane, 64 banks) start four banks apart and never collide.
 template <int FMT>
 __host__ __device__ constexpr int mf_row_pitch() {
-    int p = MTile<FMT>::BYTES;  // a multiple of 16
+    int p = (MTile<FMT>::BYTES + 15) / 16 * 16;
     return (p / 16) % 2 ? p : p + 16;
 }
 constexpr int MF_GROUPS = 4;            // row groups whose partial sums a wave keeps before the workgroup adds them
@@ -373,7 +415,10 @@ template <int FMT>
 __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
                                                                 const float *__restrict__ bias, float *__restrict__ y, int n, int k, int rows) {
     typedef MTile<FMT> T;
-    constexpr int CH = T::BYTES / 16;           // 16-byte chunks of a tile row
+    constexpr int CH = T::BYTES / 16;           // whole 16-byte chunks of a tile row
+    constexpr int TAIL = T::BYTES % 16;         // 0, or the 2 bytes of Q6_K's d after 13 chunks
+    static_assert(TAIL == 0 || TAIL == 2, "a tile row is whole 16-byte chunks, or Q6_K's 13 chunks + d");
+    constexpr int ALIGN = TAIL ? 2 : 16;        // Q6_K rows start on even addresses only
     constexpr int PITCH = mf_row_pitch<FMT>();
     constexpr int REGION = mf_region_bytes<FMT>();
     constexpr int NL = (16 * CH + 63) / 64;     // 128-bit loads per lane and tile
@@ -408,22 +453,29 @@ __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__
             for (int i = 0; i < NL; ++i)
                 loff[c][i] = live[c] && crow[i] < 16 ? (uint32_t)(crow[i] * rowbytes + (size_t)(t0 + wave + c * MF_WAVES) * T::BYTES + (size_t)cidx[i] * 16) : 0u;
         }
-        auto fetch = [&](u32x4(&dst)[NC][NL], int grp) {
+        uint32_t toff[NC];  // TAIL: lanes 0..15 also fetch the last two bytes of their row's run
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+            toff[c] = TAIL && live[c] && lane < 16 ? (uint32_t)(lane * rowbytes + (size_t)(t0 + wave + c * MF_WAVES) * T::BYTES + 16 * CH) : 0u;
+        auto fetch = [&](u32x4(&dst)[NC][NL], uint32_t(&tl)[NC], int grp) {
             if (grp >= ngroups) return;  // workgroup-uniform
             // the last group of a ragged matrix is the last 16 rows: in bounds, its first rows computed twice, stored once
             const uint8_t *gb = W + (size_t)min(grp * 16, n - 16) * rowbytes;
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
 #pragma unroll
-                for (int i = 0; i < NL; ++i) dst[c][i] = ld128<16>(gb + loff[c][i]);
+                for (int i = 0; i < NL; ++i) dst[c][i] = ld128<ALIGN>(gb + loff[c][i]);
+                if constexpr (TAIL != 0) tl[c] = ld16(gb + toff[c]);
             }
         };
-        auto stash = [&](const u32x4(&src)[NC][NL]) {
+        auto stash = [&](const u32x4(&src)[NC][NL], const uint32_t(&tl)[NC]) {
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
 #pragma unroll
                 for (int i = 0; i < NL; ++i)
                     if (crow[i] < 16) *reinterpret_cast<u32x4 *>(reg + c * REGION + crow[i] * PITCH + cidx[i] * 16) = src[c][i];
+                if constexpr (TAIL != 0)
+                    if (lane < 16) *reinterpret_cast<uint16_t *>(reg + c * REGION + lane * PITCH + 16 * CH) = (uint16_t)tl[c];
             }
         };
 
@@ -440,8 +492,9 @@ __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__
             for (int t = 0; t < 8; ++t) v[c][t] = *reinterpret_cast<const float4 *>(xp + 32 * t);
         }
         u32x4 st[2][NC][NL];
-        fetch(st[0], blockIdx.x);
-        fetch(st[1], blockIdx.x + stride);
+        uint32_t stt[2][NC];
+        fetch(st[0], stt[0], blockIdx.x);
+        fetch(st[1], stt[1], blockIdx.x + stride);
 
         f16x8 xa[NC][8], xs[NC];
         float inv[NC][4];
@@ -456,8 +509,8 @@ __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__
                 const int grp = base + gi * stride;
                 acc[gi] = f32x4{0.f, 0.f, 0.f, 0.f};
                 if (grp < ngroups) {  // workgroup-uniform
-                    stash(st[gi & 1]);
-                    fetch(st[gi & 1], grp + 2 * stride);
+                    stash(st[gi & 1], stt[gi & 1]);
+                    fetch(st[gi & 1], stt[gi & 1], grp + 2 * stride);
                     wave_lds_sync();
 #pragma unroll
                     for (int c = 0; c < NC; ++c) {

@@ -332,6 +332,7 @@ MfmaVariant pick_mfma(int fmt) {
     case F_Q8_0: return {gemv_mfma_kernel<F_Q8_0>, gemv_mfma_lds_bytes<F_Q8_0>()};
     case F_Q4_K: return {gemv_mfma_kernel<F_Q4_K>, gemv_mfma_lds_bytes<F_Q4_K>()};
     case F_Q5_K: return {gemv_mfma_kernel<F_Q5_K>, gemv_mfma_lds_bytes<F_Q5_K>()};
+    case F_Q6_K: return {gemv_mfma_kernel<F_Q6_K>, gemv_mfma_lds_bytes<F_Q6_K>()};
     default: return {nullptr, 0};
     }
 }
@@ -347,7 +348,9 @@ int launch_gemv_mfma(const MfmaVariant &v, const jitnn_hip_weight *w, const floa
 }
 
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
-    if (rows >= 2 && rows <= 8 && w->k % 256 == 0 && w->n >= 16 && g.batch_mfma) {
+    // Q6_K pays the most per weight on the matrix-core path (6-bit quants from two arrays, 16-value scale groups): up to
+    // four rows its FP32 kernel is still ahead (measured: 33 vs 43 us at 2 rows, 151 vs 167 us at 4 rows on the output head)
+    if (rows >= (w->fmt == F_Q6_K ? 5 : 2) && rows <= 8 && w->k % 256 == 0 && w->n >= 16 && g.batch_mfma) {
         const MfmaVariant v = pick_mfma(w->fmt);
         if (v.fn && v.lds <= g.max_lds) return launch_gemv_mfma(v, w, x, rows, bias, y, stream);
     }
