@@ -57,6 +57,14 @@ struct XReg {
     __device__ __forceinline__ float4 q(int, int g) const { return x[g]; }
     __device__ __forceinline__ float s(int, int i) const { return sm[i]; }
 };
+// the same for two batch rows (128 VGPRs of activations per lane)
+template <int UQ, int NS>
+struct XReg2 {
+    float4 x[2][UQ];
+    float sm[2][NS];
+    __device__ __forceinline__ float4 q(int b, int g) const { return x[b][g]; }
+    __device__ __forceinline__ float s(int b, int i) const { return sm[b][i]; }
+};
 
 template <int FMT>
 struct Unit;
@@ -783,6 +791,109 @@ template <class UA, int CVA, class UB, int CVB, int PF>
 __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg2_kernel(const XregArgs a, const XregArgs b, const int split) {
     if ((int)blockIdx.x < split) gemv_xreg_body<UA, CVA, PF, false, true, false>(a, blockIdx.x, split);
     else gemv_xreg_body<UB, CVB, PF, false, true, false>(b, blockIdx.x - split, gridDim.x - split);
+}
+
+// Batch 2, rows of at most 4096 values: gemv_xreg_kernel's scheme with the activations of both rows in registers.
+// Every decoded weight meets two activations, so the kernel stays close to the batch-1 time where the FP32 kernel
+// with activations in LDS and the matrix-core kernel (built for up to eight rows) both take half as long again.
+//   x [2, k], y [2, n]; bias (BIAS) is added to both rows.
+template <class U, int CV, int PF, bool BIAS>
+__global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_b2_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
+                                                                    const float *__restrict__ bias, float *__restrict__ y, int n, int k, float nib) {
+    constexpr int FMT = U::FMT, STEPS = 64 / U::UV;
+    constexpr int UQ = U::UV / 4, NS = U::NS, SG = U::SG, NB = PF + 1;
+    __shared__ float4 xl[2][STEPS * 64 * (UQ + 1)];
+    __shared__ float sums[2][STEPS * 64 * NS];
+    constexpr int nwaves = XREG_THREADS / 64;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int units = k / U::UV;
+    const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
+    const int stride = gridDim.x * nwaves;
+    const int row0 = blockIdx.x * nwaves + wave;
+    int uc[STEPS];
+    uint32_t off[STEPS][U::NOFF];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+        uc[s] = min(s * 64 + lane, units - 1);  // lanes past the row end: last unit, zeroed x
+        U::offsets(uc[s], off[s]);
+    }
+    auto fill = [&](typename U::Raw(&dst)[STEPS], float &bdst, int r) {
+        const bool live = r < n;  // a row past the end is "loaded" from the first bytes of the matrix: one cache line
+        const uint8_t *rp = W + (live ? (size_t)r * rowbytes : 0);
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            uint32_t o[U::NOFF];
+#pragma unroll
+            for (int i = 0; i < U::NOFF; ++i) o[i] = live ? off[s][i] : 0u;
+            U::load(dst[s], rp, o);
+        }
+        if (BIAS) bdst = bias[live ? r : 0];
+    };
+    // ---- activations first (their loads must not queue behind the first weight rows), then the ring's first rows
+    constexpr int QUADS = STEPS * 64 * UQ, PER = QUADS / XREG_THREADS;
+    static_assert(QUADS % XREG_THREADS == 0, "whole passes");
+    float4 xv[2][PER];
+    {
+        const int kq = k >> 2;
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                const int f = tid + i * XREG_THREADS;
+                xv[b][i] = f < kq ? reinterpret_cast<const float4 *>(x + (size_t)b * k)[f] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+    }
+    typename U::Raw buf[NB][STEPS];
+    float bv[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        bv[b] = 0.f;
+        fill(buf[b], bv[b], row0 + b * stride);
+    }
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int f = tid + i * XREG_THREADS;
+            int u, g;
+            U::slot(f, u, g);
+            xl[b][u * (UQ + 1) + g] = xv[b][i];
+            const float sm = group_sum<SG>((xv[b][i].x + xv[b][i].y) + (xv[b][i].z + xv[b][i].w));
+            if ((f & (SG - 1)) == 0) sums[b][u * NS + g / SG] = sm;
+        }
+    __syncthreads();
+    XReg2<UQ, NS> xs[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int g = 0; g < UQ; ++g) xs[s].x[b][g] = xl[b][(s * 64 + lane) * (UQ + 1) + g];
+#pragma unroll
+            for (int i = 0; i < NS; ++i) xs[s].sm[b][i] = sums[b][(s * 64 + lane) * NS + i];
+        }
+
+    for (int base = row0; base < n; base += NB * stride) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int row = base + b * stride;
+            if (row < n) {  // wave-uniform
+                float acc[1][2] = {{0.f, 0.f}};
+#pragma unroll
+                for (int s = 0; s < STEPS; ++s) {
+                    const typename U::Raw(&w1)[1] = reinterpret_cast<const typename U::Raw(&)[1]>(buf[b][s]);
+                    U::template dot<2, 1, CV>(w1, uc[s], xs[s], acc, nib);
+                }
+                const float t0 = wave_sum(acc[0][0]), t1 = wave_sum(acc[0][1]);
+                if (lane == 0) {
+                    y[row] = BIAS ? t0 + bv[b] : t0;
+                    y[(size_t)n + row] = BIAS ? t1 + bv[b] : t1;
+                }
+            }
+            fill(buf[b], bv[b], row + NB * stride);
+        }
+    }
 }
 
 // Batch-1 GEMV for rows longer than 4096 values: the row is cut into slices of 4096 values, one per wave of

@@ -67,6 +67,7 @@ struct State {
     int gemv_max_rows = 64;
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
+    bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
 };
 State g;
 std::mutex g_mu;
@@ -318,6 +319,34 @@ int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *b
     return JITNN_HIP_OK;
 }
 
+template <int PF, bool BIAS>
+gemv1_fn pick_xreg_b2_fmt(int fmt, bool pairs) {
+    switch (fmt) {
+    case F_Q4_0: return pairs ? gemv_xreg_b2_kernel<UnitPair<F_Q4_0>, 1, PF, BIAS> : gemv_xreg_b2_kernel<Unit<F_Q4_0>, 1, PF, BIAS>;
+    case F_Q4_1: return pairs ? gemv_xreg_b2_kernel<UnitPair<F_Q4_1>, 1, PF, BIAS> : gemv_xreg_b2_kernel<Unit<F_Q4_1>, 1, PF, BIAS>;
+    case F_Q8_0: return pairs ? gemv_xreg_b2_kernel<UnitPair<F_Q8_0>, 0, PF, BIAS> : gemv_xreg_b2_kernel<Unit<F_Q8_0>, 0, PF, BIAS>;
+    case F_Q4_K: return gemv_xreg_b2_kernel<Unit<F_Q4_K>, 1, PF, BIAS>;
+    case F_Q5_K: return gemv_xreg_b2_kernel<Unit<F_Q5_K>, 0, PF, BIAS>;
+    default: return gemv_xreg_b2_kernel<Unit<F_Q6_K>, 0, PF, BIAS>;
+    }
+}
+
+// Batch 2, rows of at most 4096 values: both activation rows in registers.
+int launch_gemv_xreg_b2(const jitnn_hip_weight *w, const float *x, const float *bias, float *y, hipStream_t stream) {
+    const int waves = XREG_THREADS / 64;
+    int blocks = (w->n + waves - 1) / waves;
+    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : 2);
+    if (blocks > cap) blocks = cap;
+    const int rows_per_wave = (w->n + blocks * waves - 1) / (blocks * waves);
+    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
+    const bool pairs = w->k % 64 == 0;
+    gemv1_fn fn = bias ? (pf == 1 ? pick_xreg_b2_fmt<1, true>(w->fmt, pairs) : pick_xreg_b2_fmt<2, true>(w->fmt, pairs))
+                       : (pf == 1 ? pick_xreg_b2_fmt<1, false>(w->fmt, pairs) : pick_xreg_b2_fmt<2, false>(w->fmt, pairs));
+    hipLaunchKernelGGL(fn, dim3(blocks), dim3(XREG_THREADS), 0, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
 typedef void (*mfma_fn)(const uint8_t *, const float *, const float *, float *, int, int, int);
 
 struct MfmaVariant {
@@ -348,6 +377,7 @@ int launch_gemv_mfma(const MfmaVariant &v, const jitnn_hip_weight *w, const floa
 }
 
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    if (rows == 2 && w->k <= 4096 && !g.force_lds && g.batch2_xreg) return launch_gemv_xreg_b2(w, x, bias, y, stream);
     // Q6_K pays the most per weight on the matrix-core path (6-bit quants from two arrays, 16-value scale groups): up to
     // four rows its FP32 kernel is still ahead (measured: 33 vs 43 us at 2 rows, 151 vs 167 us at 4 rows on the output head)
     if (rows >= (w->fmt == F_Q6_K ? 5 : 2) && rows <= 8 && w->k % 256 == 0 && w->n >= 16 && g.batch_mfma) {
@@ -557,6 +587,7 @@ int jitnn_hip_init(int device_ordinal) {
     }
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
     g.device = device_ordinal;
     g.ready = true;
     return JITNN_HIP_OK;
