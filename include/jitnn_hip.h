@@ -11,7 +11,9 @@
  *
  * Conventions
  *  - fmt is the ggml type id stored in GGUF files (gguf/GgmlType.java:27-65):
- *    Q4_0=2 Q4_1=3 Q8_0=8 Q4_K=12 Q5_K=13 Q6_K=14.
+ *    Q4_0=2 Q4_1=3 Q8_0=8 Q4_K=12 Q5_K=13 Q6_K=14 (the quantised-linear path proper: tuned kernels), and
+ *    Q5_0=6 Q5_1=7 Q2_K=10 Q3_K=11 (the other block formats the reference dequantises,
+ *    core/kernels/GgufKernels.java:147-198: bit-exact dequantiser and a plain GEMV).
  *  - A weight is [n, k] row-major rows of k/block_values blocks, byte-for-byte as in the GGUF file
  *    (core/Tensor.java:249-278); it stays in that layout in HBM.
  *  - Activations and outputs are FP32 row-major: x [rows, k], y [rows, n], bias [n].
@@ -63,7 +65,7 @@ JITNN_HIP_API int jitnn_hip_sync(void);
 
 /* ---- block formats (no device needed) ------------------------------------------------------------ */
 
-/* Values per block / bytes per block of a format, 0 when fmt is not one of the six
+/* Values per block / bytes per block of a format, 0 when fmt is not one of the ten
  * (core/DType.java:75-98, gguf/GgmlType.java:113-118). */
 JITNN_HIP_API int jitnn_hip_block_values(int fmt);
 JITNN_HIP_API int jitnn_hip_block_bytes(int fmt);

@@ -8,14 +8,21 @@
 namespace jitnn {
 
 // ggml type ids as stored in GGUF files (reference: gguf/GgmlType.java:27-65)
-enum : int { F_Q4_0 = 2, F_Q4_1 = 3, F_Q8_0 = 8, F_Q4_K = 12, F_Q5_K = 13, F_Q6_K = 14 };
+// The first six are the formats of the quantised-linear path proper (tuned kernels); Q5_0, Q5_1, Q2_K and Q3_K are the
+// other block formats the reference dequantises (core/kernels/GgufKernels.java:147-198): bit-exact dequantiser and a
+// plain GEMV, so that every block tensor of a GGUF file is usable.
+enum : int { F_Q4_0 = 2, F_Q4_1 = 3, F_Q8_0 = 8, F_Q4_K = 12, F_Q5_K = 13, F_Q6_K = 14, F_Q5_0 = 6, F_Q5_1 = 7, F_Q2_K = 10, F_Q3_K = 11 };
+
+__host__ __device__ constexpr bool is_extra_format(int fmt) { return fmt == F_Q5_0 || fmt == F_Q5_1 || fmt == F_Q2_K || fmt == F_Q3_K; }
 
 __host__ __device__ constexpr int block_values(int fmt) {
-    return (fmt == F_Q4_0 || fmt == F_Q4_1 || fmt == F_Q8_0) ? 32 : (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K) ? 256 : 0;
+    return (fmt == F_Q4_0 || fmt == F_Q4_1 || fmt == F_Q8_0 || fmt == F_Q5_0 || fmt == F_Q5_1) ? 32
+           : (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K || fmt == F_Q2_K || fmt == F_Q3_K) ? 256 : 0;
 }
 
 __host__ __device__ constexpr int block_bytes(int fmt) {
-    return fmt == F_Q4_0 ? 18 : fmt == F_Q4_1 ? 20 : fmt == F_Q8_0 ? 34 : fmt == F_Q4_K ? 144 : fmt == F_Q5_K ? 176 : fmt == F_Q6_K ? 210 : 0;
+    return fmt == F_Q4_0 ? 18 : fmt == F_Q4_1 ? 20 : fmt == F_Q8_0 ? 34 : fmt == F_Q4_K ? 144 : fmt == F_Q5_K ? 176 : fmt == F_Q6_K ? 210
+           : fmt == F_Q5_0 ? 22 : fmt == F_Q5_1 ? 24 : fmt == F_Q2_K ? 84 : fmt == F_Q3_K ? 110 : 0;
 }
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

@@ -63,6 +63,55 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
             float a = ds * (float)q;
             o[t] = a - m;
         }
+    } else if constexpr (FMT == F_Q5_0 || FMT == F_Q5_1) {
+        // 22 / 24 bytes: f16 d (, f16 m), 32 fifth bits, 16 bytes of nibbles; value e: nibble e % 16 (low for e < 16) + 16 *
+        // bit e, then (q - 16) * d or q * d + m (GgufKernels.java:143-163)
+        constexpr int NB = FMT == F_Q5_0 ? 22 : 24, QH = FMT == F_Q5_0 ? 2 : 4, QS = QH + 4;
+        const uint8_t *b = w + (i >> 5) * NB;
+        const int e = (int)(i & 31);
+        const float d = h2f(ld16(b));
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int v = b[QS + ((e + t) & 15)];
+            const int q = (e < 16 ? (v & 15) : (v >> 4)) + 16 * ((b[QH + ((e + t) >> 3)] >> ((e + t) & 7)) & 1);
+            if constexpr (FMT == F_Q5_0) {
+                o[t] = (float)(q - 16) * d;
+            } else {
+                const float p = (float)q * d;
+                o[t] = p + h2f(ld16(b + 2));
+            }
+        }
+    } else if constexpr (FMT == F_Q2_K) {
+        // 84 bytes: 16 scale bytes (low nibble scale, high nibble min), 64 bytes of 2-bit quants, f16 d, f16 dmin
+        // (GgufKernels.java:166-175)
+        const uint8_t *b = w + (i >> 8) * 84;
+        const int e = (int)(i & 255);
+        const int n = e >> 7, j = (e & 127) >> 5, l = e & 31;
+        const int sc = b[n * 8 + j * 2 + (l >> 4)];
+        const float ds = h2f(ld16(b + 80)) * (float)(sc & 15);
+        const float m = h2f(ld16(b + 82)) * (float)(sc >> 4);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int q = (b[16 + n * 32 + l + t] >> (2 * j)) & 3;
+            const float a = ds * (float)q;
+            o[t] = a - m;
+        }
+    } else if constexpr (FMT == F_Q3_K) {
+        // 110 bytes: 32 bytes of high bits, 64 bytes of 2-bit quants, 12 bytes of 6-bit scales, f16 d
+        // (GgufKernels.java:181-198)
+        const uint8_t *b = w + (i >> 8) * 110;
+        const int e = (int)(i & 255);
+        const int n = e >> 7, j = (e & 127) >> 5, l = e & 31;
+        const int is = n * 8 + j * 2 + (l >> 4);
+        const int low = is < 8 ? (b[96 + is] & 15) : (b[96 + is - 8] >> 4);
+        const int high = (b[96 + 8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+        const float a = h2f(ld16(b + 108)) * (float)(low + 16 * high - 32);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int q = (b[32 + n * 32 + l + t] >> (2 * j)) & 3;
+            const int hb = (b[l + t] >> (4 * n + j)) & 1;
+            o[t] = a * (float)(q - (hb == 1 ? 0 : 4));
+        }
     } else {  // F_Q6_K
         const uint8_t *b = w + (i >> 8) * 210;
         const int e = (int)(i & 255);
@@ -84,6 +133,39 @@ template <int FMT>
 __global__ void __launch_bounds__(256) dequant_kernel(const uint8_t *__restrict__ w, float *__restrict__ y, size_t quads) {
     for (size_t f = (size_t)blockIdx.x * blockDim.x + threadIdx.x; f < quads; f += (size_t)gridDim.x * blockDim.x) {
         reinterpret_cast<float4 *>(y)[f] = dequant4<FMT>(w, f * 4);
+    }
+}
+
+// Plain GEMV for the formats without a tuned kernel: one wave per weight row, every lane dequantises quads of the row
+// with the bit-exact decoder and multiplies them with up to eight activation rows; a fixed DPP tree adds the lanes.
+//   y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]), b < rows <= 8.  grid: any; waves take rows round-robin.
+template <int FMT>
+__global__ void __launch_bounds__(256) gemv_plain_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, const float *__restrict__ bias,
+                                                          float *__restrict__ y, int n, int k, int rows) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
+    for (int row = blockIdx.x * 4 + wave; row < n; row += gridDim.x * 4) {
+        const uint8_t *wr = W + (size_t)row * rowbytes;
+        float acc[8];
+#pragma unroll
+        for (int b = 0; b < 8; ++b) acc[b] = 0.f;
+        for (int f = lane; f < (k >> 2); f += 64) {
+            const float4 v = dequant4<FMT>(wr, (size_t)f * 4);
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+                if (b < rows) {
+                    const float4 xv = reinterpret_cast<const float4 *>(x + (size_t)b * k)[f];
+                    acc[b] = __builtin_fmaf(v.w, xv.w, __builtin_fmaf(v.z, xv.z, __builtin_fmaf(v.y, xv.y, __builtin_fmaf(v.x, xv.x, acc[b]))));
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            if (b < rows) {
+                const float t = wave_sum(acc[b]);
+                if (lane == 0) y[(size_t)b * n + row] = bias ? t + bias[row] : t;
+            }
+        }
     }
 }
 

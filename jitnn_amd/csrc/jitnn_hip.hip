@@ -376,7 +376,20 @@ int launch_gemv_mfma(const MfmaVariant &v, const jitnn_hip_weight *w, const floa
     return JITNN_HIP_OK;
 }
 
+// Formats without a tuned kernel (Q5_0, Q5_1, Q2_K, Q3_K): one wave per row on the bit-exact decoder.
+int launch_gemv_plain(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    int blocks = (w->n + 3) / 4;
+    if (blocks > g.cus * 8) blocks = g.cus * 8;
+    typedef void (*fn_t)(const uint8_t *, const float *, const float *, float *, int, int, int);
+    fn_t fn = w->fmt == F_Q5_0 ? gemv_plain_kernel<F_Q5_0> : w->fmt == F_Q5_1 ? gemv_plain_kernel<F_Q5_1> : w->fmt == F_Q2_K ? gemv_plain_kernel<F_Q2_K>
+                                                                                                                             : gemv_plain_kernel<F_Q3_K>;
+    hipLaunchKernelGGL(fn, dim3(blocks), dim3(256), 0, stream, w->dev, x, bias, y, w->n, w->k, rows);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    if (is_extra_format(w->fmt)) return launch_gemv_plain(w, x, rows, bias, y, stream);
     if (rows == 2 && w->k <= 4096 && !g.force_lds && g.batch2_xreg) return launch_gemv_xreg_b2(w, x, bias, y, stream);
     // Q6_K pays the most per weight on the matrix-core path (6-bit quants from two arrays, 16-value scale groups): up to
     // four rows its FP32 kernel is still ahead (measured: 33 vs 43 us at 2 rows, 151 vs 167 us at 4 rows on the output head)
@@ -530,7 +543,7 @@ int jitnn_hip_block_values(int fmt) { return block_values(fmt); }
 int jitnn_hip_block_bytes(int fmt) { return block_bytes(fmt); }
 
 long long jitnn_hip_weight_nbytes(int fmt, long long n, long long k) {
-    if (!known(fmt)) return fail(JITNN_HIP_EINVAL, "ggml type id %d is not one of Q4_0, Q4_1, Q8_0, Q4_K, Q5_K, Q6_K", fmt);
+    if (!known(fmt)) return fail(JITNN_HIP_EINVAL, "ggml type id %d is not one of Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K, Q4_K, Q5_K, Q6_K", fmt);
     if (n < 1 || k < 1) return fail(JITNN_HIP_EINVAL, "weight shape [%lld, %lld] is empty", n, k);
     if (k % block_values(fmt) != 0)
         return fail(JITNN_HIP_EINVAL, "format %d weight of shape [%lld, %lld]: last axis not a multiple of its block of %d", fmt, n, k,
@@ -669,6 +682,10 @@ int jitnn_hip_dequantize_dev(const jitnn_hip_weight *w, float *y_dev, void *stre
     case F_Q8_0: launch_dequant<F_Q8_0>(w, y_dev, s); break;
     case F_Q4_K: launch_dequant<F_Q4_K>(w, y_dev, s); break;
     case F_Q5_K: launch_dequant<F_Q5_K>(w, y_dev, s); break;
+    case F_Q5_0: launch_dequant<F_Q5_0>(w, y_dev, s); break;
+    case F_Q5_1: launch_dequant<F_Q5_1>(w, y_dev, s); break;
+    case F_Q2_K: launch_dequant<F_Q2_K>(w, y_dev, s); break;
+    case F_Q3_K: launch_dequant<F_Q3_K>(w, y_dev, s); break;
     default: launch_dequant<F_Q6_K>(w, y_dev, s); break;
     }
     HIP_TRY(hipGetLastError());
@@ -696,7 +713,7 @@ int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows
     if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
     if (int rc = check_ready()) return rc;
     hipStream_t s = (hipStream_t)stream;
-    if (rows > g.gemv_max_rows) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s);
+    if (rows > g.gemv_max_rows && !is_extra_format(w->fmt)) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s);
     for (int r0 = 0; r0 < rows; r0 += 8) {
         const int nb = rows - r0 < 8 ? rows - r0 : 8;
         if (int rc = launch_gemv(w, x_dev + (size_t)r0 * w->k, nb, bias_dev, y_dev + (size_t)r0 * w->n, s)) return rc;
@@ -929,7 +946,7 @@ void launch_attention(const jitnn_hip_llama *m, int layer, int pos, hipStream_t 
     hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(m->heads), dim3(2 * D), 0, st, m->part, m->att, chunks);
 }
 
-bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !g.force_lds; }
+bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !g.force_lds && !is_extra_format(w->fmt); }
 
 // y_i = W_i RMSNorm(x; nw) for `count` (at most 3) weights over the same x.  Weights the register-resident kernel
 // takes get the norm fused into their launch, neighbours of one format share the launch; anything else goes through

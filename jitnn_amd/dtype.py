@@ -15,6 +15,12 @@ class DType(Enum):
     Q4_K = (12, 256, 144)
     Q5_K = (13, 256, 176)
     Q6_K = (14, 256, 210)
+    # the other block formats the reference dequantises (core/kernels/GgufKernels.java:147-198): bit-exact dequantiser and
+    # a plain GEMV, no tuned kernels
+    Q5_0 = (6, 32, 22)
+    Q5_1 = (7, 32, 24)
+    Q2_K = (10, 256, 84)
+    Q3_K = (11, 256, 110)
 
     @property
     def ggml_id(self) -> int:

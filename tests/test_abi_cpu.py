@@ -27,13 +27,14 @@ def test_header_symbols_are_exported_and_bound():
 
 def test_block_metadata_matches_reference_table():
     from jitnn_amd import DType, _lib
-    table = {2: (32, 18), 3: (32, 20), 8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210)}  # DType.java:75-98
+    table = {2: (32, 18), 3: (32, 20), 8: (32, 34), 12: (256, 144), 13: (256, 176), 14: (256, 210),  # DType.java:75-98
+             6: (32, 22), 7: (32, 24), 10: (256, 84), 11: (256, 110)}
     for fid, (qk, nb) in table.items():
         assert _lib.lib.jitnn_hip_block_values(fid) == qk
         assert _lib.lib.jitnn_hip_block_bytes(fid) == nb
         t = DType.from_ggml_id(fid)
         assert (t.block_values(), t.block_bytes()) == (qk, nb)
-    for fid in (0, 1, 6, 7, 10, 11, 15, 99, -1):
+    for fid in (0, 1, 9, 15, 30, 99, -1):  # F32, F16, Q8_1, Q8_K, BF16: no block tensor type
         assert _lib.lib.jitnn_hip_block_values(fid) == 0 and _lib.lib.jitnn_hip_block_bytes(fid) == 0
 
 

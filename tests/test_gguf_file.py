@@ -13,7 +13,7 @@ import jitnn_amd
 from jitnn_amd import DType, GgufFile, UnsupportedTypeError
 
 FIXTURE = GOLDEN_DIR / "fixture.gguf"
-PATH_FORMATS = ["Q8_0", "Q4_0", "Q4_1", "Q4_K", "Q5_K", "Q6_K"]
+PATH_FORMATS = ["Q8_0", "Q4_0", "Q4_1", "Q4_K", "Q5_K", "Q6_K", "Q5_0", "Q5_1", "Q2_K", "Q3_K"]
 
 
 @pytest.fixture(scope="module")

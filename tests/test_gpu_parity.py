@@ -258,3 +258,33 @@ def test_quantize_q8_0_bit_exact_vs_oracle(jn):
     b = rng.standard_normal(64).astype(np.float32)
     y = jn.F.linear_q8(jn.Tensor.of(xin), q, jn.Tensor.of(b)).numpy()
     assert norm_err(y, oracle.gguf_linear(8, xin, exp, b, 64, 256)) <= 1e-5
+
+
+# ------------------------------------------------------------------------------------------ the other dequantisable formats
+
+EXTRA_FORMATS = ["Q5_0", "Q5_1", "Q2_K", "Q3_K"]  # bit-exact dequantiser + plain GEMV, no tuned kernels
+
+
+@pytest.mark.parametrize("fmt", EXTRA_FORMATS)
+def test_extra_format_dequant_fixture_bit_exact(jn, gguf_fixture, fmt):
+    """w.<T> of the reference's fixture.gguf dequantises to expect.<T> bit for bit (GgufChecks.java:58-75)."""
+    got = weight(jn, fmt, gguf_fixture.raw("w." + fmt), 3, 512).to_float_array()
+    expect = gguf_fixture.f32("expect." + fmt).reshape(-1)
+    assert np.array_equal(bits(got), bits(expect))
+
+
+@pytest.mark.parametrize("fmt", EXTRA_FORMATS)
+def test_extra_format_dequant_and_linear_vs_oracle(jn, fmt):
+    from oracle import oracle
+    rng = np.random.default_rng(500 + GGML_ID[fmt])
+    n, k = 37, 1024
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    assert np.array_equal(bits(w.to_float_array()), bits(oracle.dequantize(GGML_ID[fmt], raw, n * k)))
+    bias = rng.standard_normal(n).astype(np.float32)
+    for rows in (1, 3, 8, 11, 70):  # 70: past the GEMV range of the tuned formats; these stay on the plain kernel
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, bias if rows % 2 else None, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias) if rows % 2 else None).numpy()
+        assert y.shape == (rows, n)
+        assert norm_err(y, ref) <= GEMV_BAR, (fmt, rows, norm_err(y, ref))
