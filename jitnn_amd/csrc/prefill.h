@@ -378,15 +378,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         }
         decode(rnext, s + 1);
         // One wave per SIMD: nobody else fills the matrix pipe while this wave decodes, or the VALU while it multiplies.
-        // Ask the scheduler for the interleaving by hand: the step's global loads first, then one MFMA, a few decode
-        // instructions and every other time one LDS operand read, 32 times over.
-        __builtin_amdgcn_sched_group_barrier(0x020, 11, 0);
+        // Ask the scheduler for the interleaving by hand: 32 times one MFMA and a few decode instructions, every other
+        // time also one LDS operand read and one of the step's global loads.  The loads are spread over the step on
+        // purpose: issued in one burst after the barrier, the four waves' 44 requests queue up at the CU's one
+        // address unit and the waves stall at the issue while the matrix pipe idles.
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
             if (i % 2 == 0 && i < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
     };
     fetch_w(raw[0], sbeg);
@@ -404,17 +406,33 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         if (s0 + u < nsteps) step(s0 + u, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
     // ---- epilogue.  The activations went in as the first MFMA operand, so an accumulator holds a 32 (tokens) x 32
     // (weight rows) block of y: element r is token 8*(r/4) + 4*(lane/32) + r%4, weight row lane%32 - the 32 lanes of a
-    // half wave store 32 consecutive floats of one token's output row.
+    // half wave store 32 consecutive floats of one token's output row.  The 32 token scales of the lane are read
+    // first, in one batch (index clamped, so the loads are unconditional): a load between the stores would make
+    // every store wait for the one before it, stores and loads being counted by the same counter.
+    const int tok0 = m0 + 64 * wave + 4 * (lane >> 5);
+    float isc[2][16];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) isc[j][r] = inv_scale[min(tok0 + 32 * j + 8 * (r >> 2) + (r & 3), m - 1)];
+    float bv[4];
+    {
+        const float *bp = bias ? bias : inv_scale;  // some readable address when there is no bias: the value is dropped
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float b = bp[bias ? min(n0 + 32 * i + (lane & 31), n - 1) : 0];
+            bv[i] = bias ? b : 0.f;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = n0 + 32 * i + (lane & 31);
-        const float bv = bias && row < n ? bias[row] : 0.f;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int tok = m0 + 64 * wave + 32 * j + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row < n && tok < m) y[(size_t)tok * n + row] = acc[i][j][r] * inv_scale[tok] + bv;
+                const int tok = tok0 + 32 * j + 8 * (r >> 2) + (r & 3);
+                if (row < n && tok < m) y[(size_t)tok * n + row] = acc[i][j][r] * isc[j][r] + bv[i];
             }
         }
     }
