@@ -489,8 +489,15 @@ int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const fl
     _Float16 *xo = (_Float16 *)ws;
     float *scale = (float *)((uint8_t *)ws + xo_bytes), *inv = scale + rows;
     float *part = (float *)((uint8_t *)ws + xo_bytes + scale_bytes);
-    hipLaunchKernelGGL(x_row_scale_kernel, dim3(rows), dim3(256), 0, stream, x, scale, inv, w->k);
-    hipLaunchKernelGGL(x_to_operand_kernel, dim3(mblocks, pf_ksteps(w->k) / 4), dim3(256), 0, stream, x, scale, xo, rows, w->k);
+    if (w->k <= XP_MAXK) {
+        const int pieces = pf_ksteps(w->k) * 2;  // per row; 256 threads take J each
+        if (pieces <= 512) hipLaunchKernelGGL(x_prepare_kernel<2>, dim3(mblocks * 32), dim3(256), 0, stream, x, inv, xo, rows, w->k);
+        else if (pieces <= 1024) hipLaunchKernelGGL(x_prepare_kernel<4>, dim3(mblocks * 32), dim3(256), 0, stream, x, inv, xo, rows, w->k);
+        else hipLaunchKernelGGL(x_prepare_kernel<8>, dim3(mblocks * 32), dim3(256), 0, stream, x, inv, xo, rows, w->k);
+    } else {
+        hipLaunchKernelGGL(x_row_scale_kernel, dim3(rows), dim3(256), 0, stream, x, scale, inv, w->k);
+        hipLaunchKernelGGL(x_to_operand_kernel, dim3(mblocks, pf_ksteps(w->k) / 4), dim3(256), 0, stream, x, scale, xo, rows, w->k);
+    }
     float *out = splits > 1 ? part : y;
     const float *b1 = splits > 1 ? nullptr : bias;
     switch (w->fmt) {

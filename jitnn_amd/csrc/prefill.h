@@ -84,6 +84,61 @@ __global__ void __launch_bounds__(256) x_to_operand_kernel(const float *__restri
     reinterpret_cast<f16x8 *>(xo)[((size_t)blockIdx.x * pf_ksteps(k) + blockIdx.y * 4 + ks) * 64 + lane] = o;
 }
 
+// The two kernels above in one launch, for rows of up to XP_MAXK values: one workgroup per token keeps the row in
+// registers between finding its scale and writing its FP16 pieces (16 bytes each, 512 bytes apart in operand order).
+// Eight consecutive tokens share every 128-byte line of the operand array, and consecutive workgroups run on
+// different XCDs, each with its own L2: the workgroup -> token map keeps the eight writers of a line on one XCD, so
+// that the line leaves its L2 whole.  grid = padded tokens (a multiple of 64); padding tokens write zeros.
+// J = 8-value pieces per thread: a row holds at most 256 J of them.
+constexpr int XP_MAXJ = 8, XP_MAXK = XP_MAXJ * 256 * 8;
+template <int J>
+__global__ void __launch_bounds__(256) x_prepare_kernel(const float *__restrict__ x, float *__restrict__ inv_scale, _Float16 *__restrict__ xo,
+                                                         int m, int k) {
+    __shared__ float red[4];
+    const int b = blockIdx.x, tok = (b & ~63) | ((b & 7) << 3) | ((b >> 3) & 7), t = threadIdx.x;
+    const int ksteps = pf_ksteps(k), npieces = 2 * ksteps;  // 8-value pieces of a row, zero padding included
+    const float *xr = x + (size_t)min(tok, m - 1) * k;
+    float4 v[J][2];
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {  // unconditional loads (index clamped), so that all of them are in flight at once
+        const int kk = 8 * (t + 256 * j);
+        const float4 *src = reinterpret_cast<const float4 *>(xr + min(kk, k - 8));
+        v[j][0] = src[0];
+        v[j][1] = src[1];
+    }
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const bool in = tok < m && 8 * (t + 256 * j) < k;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (!in) v[j][h] = make_float4(0.f, 0.f, 0.f, 0.f);
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j][h].x), fabsf(v[j][h].y)), fmaxf(fabsf(v[j][h].z), fabsf(v[j][h].w))));
+        }
+    }
+    amax = wave_max(amax);
+    if ((t & 63) == 0) red[t >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float sc = 1.f;
+    if (amax > 0.f && amax < 3.0e38f) {
+        int e;
+        frexpf(amax, &e);
+        sc = ldexpf(1.f, 14 - e);
+    }
+    if (t == 0 && tok < m) inv_scale[tok] = 1.f / sc;
+    f16x8 *dst = reinterpret_cast<f16x8 *>(xo) + (size_t)(tok >> 5) * ksteps * 64 + (tok & 31);
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const int p = t + 256 * j;  // values 8 p .. 8 p + 7: K step p / 2, lane half p % 2
+        if (p < npieces) {
+            const float4 a = v[j][0], c = v[j][1];
+            dst[(size_t)(p >> 1) * 64 + 32 * (p & 1)] = f16x8{(_Float16)(a.x * sc), (_Float16)(a.z * sc), (_Float16)(a.y * sc), (_Float16)(a.w * sc),
+                                                             (_Float16)(c.x * sc), (_Float16)(c.z * sc), (_Float16)(c.y * sc), (_Float16)(c.w * sc)};
+        }
+    }
+}
+
 // 32 consecutive weights of a row, starting at value k0 (k0 % 32 == 0), in two phases so that the loads of the next
 // K step can be in flight while the matrix cores work on the current one: pf_load fetches the raw bytes, pf_decode
 // turns them into FP32 values in the dequantiser's arithmetic.
