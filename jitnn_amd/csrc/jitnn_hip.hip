@@ -464,10 +464,13 @@ int workspace_done(hipStream_t stream) {
 }
 
 template <int FMT>
-void launch_prefill_fmt(const jitnn_hip_weight *w, const _Float16 *xo, const float *inv, int rows, const float *bias, float *y, int splits,
-                        int split_steps, hipStream_t s) {
+int launch_prefill_fmt(const jitnn_hip_weight *w, const _Float16 *xo, const float *inv, int rows, const float *bias, float *y, int splits,
+                       int split_steps, hipStream_t s) {
+    constexpr size_t lds = pf_lds_bytes<FMT>();
+    if (int rc = allow_lds((const void *)prefill_mfma_kernel<FMT>, lds)) return rc;
     dim3 grid((w->n + PF_BN - 1) / PF_BN, (rows + PF_BM - 1) / PF_BM, splits);
-    hipLaunchKernelGGL(prefill_mfma_kernel<FMT>, grid, dim3(256), 0, s, w->dev, xo, inv, bias, y, rows, w->n, w->k, split_steps);
+    hipLaunchKernelGGL(prefill_mfma_kernel<FMT>, grid, dim3(256), lds, s, w->dev, xo, inv, bias, y, rows, w->n, w->k, split_steps);
+    return JITNN_HIP_OK;
 }
 
 // more rows than the GEMV kernels take: FP16 activations in operand order + dequantise-to-LDS MFMA kernel
@@ -480,7 +483,9 @@ int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const fl
     if (w->n % 4 == 0) {
         while (splits < 8 && ntiles * mtiles * splits * 2 <= g.cus && nsteps / (splits * 2) >= 16) splits *= 2;
     }
-    const int split_steps = (nsteps + splits - 1) / splits;
+    // slices of the 256-value formats start on whole blocks (four steps): the kernel stages their raw bytes by block
+    int split_steps = (nsteps + splits - 1) / splits;
+    if (block_values(w->fmt) == 256) split_steps = (split_steps + 3) & ~3;
     const size_t xo_bytes = (size_t)mblocks * pf_ksteps(w->k) * 1024;
     const size_t scale_bytes = ((size_t)rows * 8 + 255) & ~(size_t)255;
     const size_t part_bytes = splits > 1 ? (size_t)splits * rows * w->n * 4 : 0;
@@ -500,13 +505,18 @@ int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const fl
     }
     float *out = splits > 1 ? part : y;
     const float *b1 = splits > 1 ? nullptr : bias;
+    int rc = JITNN_HIP_OK;
     switch (w->fmt) {
-    case F_Q4_0: launch_prefill_fmt<F_Q4_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q4_1: launch_prefill_fmt<F_Q4_1>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q8_0: launch_prefill_fmt<F_Q8_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q4_K: launch_prefill_fmt<F_Q4_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q5_K: launch_prefill_fmt<F_Q5_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    default: launch_prefill_fmt<F_Q6_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q4_0: rc = launch_prefill_fmt<F_Q4_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q4_1: rc = launch_prefill_fmt<F_Q4_1>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q8_0: rc = launch_prefill_fmt<F_Q8_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q4_K: rc = launch_prefill_fmt<F_Q4_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    case F_Q5_K: rc = launch_prefill_fmt<F_Q5_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    default: rc = launch_prefill_fmt<F_Q6_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
+    }
+    if (rc) {
+        workspace_done(stream);
+        return rc;
     }
     if (splits > 1) {
         const size_t count4 = (size_t)rows * w->n / 4;

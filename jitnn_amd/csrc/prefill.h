@@ -317,6 +317,40 @@ __device__ __forceinline__ void pf_decode_h<F_Q4_K>(const PfRaw<F_Q4_K> &r, int 
     }
 }
 
+// Q5_K: the Q4_K decoder with the fifth bit of every quant (bit `sub` of the qh byte of its position) put above the
+// nibble before the exponent trick.
+template <>
+__device__ __forceinline__ void pf_decode_h<F_Q5_K>(const PfRaw<F_Q5_K> &r, int k0, f16x8 (&o)[4]) {
+    const int e = k0 & 255, j = e >> 6, half = (e >> 5) & 1, sub = 2 * j + half;
+    int sc, mn;
+    {
+        const uint32_t s0 = r.h.y, s1 = r.h.z, s2 = r.h.w;
+        const uint32_t scA = s0 & 0x3f3f3f3fu, scB = (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u);
+        const uint32_t mnA = s1 & 0x3f3f3f3fu, mnB = ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u);
+        const int sh = 8 * (sub & 3);
+        sc = ((sub < 4 ? scA : scB) >> sh) & 0xff;
+        mn = ((sub < 4 ? mnA : mnB) >> sh) & 0xff;
+    }
+    const _Float16 ds = (_Float16)(h2f(r.h.x) * (float)sc), nm = (_Float16)(-(h2f(r.h.x >> 16) * (float)mn));
+    const f16x2 ds2 = {ds, ds}, nm2 = {nm, nm}, off = {(_Float16)-1024.f, (_Float16)-1024.f};
+    const uint32_t mg = pf_magic();
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        u32x4 out;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int w = 2 * c + t;
+            const uint32_t v = (w < 4 ? r.q0[w] : r.q1[w - 4]) >> (4 * half);
+            const uint32_t hb = ((w < 4 ? r.qh0[w] : r.qh1[w - 4]) >> sub) << 4;  // bit 4 of bytes 0 .. 3 at bits 4, 12, 20, 28
+            const f16x2 a = pf_pair((v & 0x000f000fu) | (hb & 0x00100010u) | mg) + off;                // bytes 0, 2
+            const f16x2 b = pf_pair(((v >> 8) & 0x000f000fu) | ((hb >> 8) & 0x00100010u) | mg) + off;  // bytes 1, 3
+            out[2 * t] = pf_bits(__builtin_elementwise_fma(a, ds2, nm2));
+            out[2 * t + 1] = pf_bits(__builtin_elementwise_fma(b, ds2, nm2));
+        }
+        o[c] = __builtin_bit_cast(f16x8, out);
+    }
+}
+
 template <>
 __device__ __forceinline__ void pf_decode_h<F_Q6_K>(const PfRaw<F_Q6_K> &r, int k0, f16x8 (&o)[4]) {
     const int kk = ((k0 & 255) >> 5) & 3;
@@ -341,11 +375,63 @@ __device__ __forceinline__ void pf_decode_h<F_Q6_K>(const PfRaw<F_Q6_K> &r, int 
     }
 }
 
+// The 256-value formats reach LDS in two hops.  A thread's 32 weights of a step are a few 16-byte fields scattered
+// over its row's block, so fetching them straight from global memory makes every load instruction of a wave touch
+// 32 to 64 cache lines (one or two per row), and the CU's one vector L1 spends more cycles on tag look-ups than the
+// matrix cores spend on the step.  Instead the workgroup copies the whole blocks of its 128 rows once per 256 values
+// (four steps), consecutive lanes taking consecutive 16-byte chunks of a row (CPR per row; a Q6_K block is 13
+// chunks and a 2-byte tail), into a double-buffered LDS area with a row pitch of RP bytes (16 x odd: conflict-free
+// 16-byte reads, and every field a decoder reads with one 16-byte load is 16-byte aligned relative to the block);
+// each step's decoder then reads its fields from there.
+template <int FMT>
+struct PfStage { static constexpr bool ON = false; static constexpr int NB = 16, CPR = 1, RP = 16, TAIL = 0, ALIGN = 16, NRAW = 0; };
+template <>
+struct PfStage<F_Q4_K> { static constexpr bool ON = false; static constexpr int NB = 144, CPR = 9, RP = 144, TAIL = 0, ALIGN = 16, NRAW = 3; };
+template <>
+struct PfStage<F_Q5_K> { static constexpr bool ON = true; static constexpr int NB = 176, CPR = 11, RP = 176, TAIL = 0, ALIGN = 16, NRAW = 5; };
+template <>
+struct PfStage<F_Q6_K> { static constexpr bool ON = true; static constexpr int NB = 210, CPR = 13, RP = 240, TAIL = 1, ALIGN = 2, NRAW = 6; };
+
+// dynamic LDS of prefill_mfma_kernel<FMT>: the FP16 weight tile of two steps, then the staged raw blocks of two
+// groups of four steps
+template <int FMT>
+constexpr size_t pf_lds_bytes() { return (size_t)2 * PF_BN * PF_LD * 2 + (PfStage<FMT>::ON ? (size_t)2 * PF_BN * PfStage<FMT>::RP : 0); }
+
+// pf_load from a staged block: b = the row's block in LDS, e = first value within the block (a multiple of 32)
+template <int FMT>
+__device__ __forceinline__ void pf_load_lds(PfRaw<FMT> &r, const uint8_t *b, int e) {
+    auto q = [&](int off) { return *reinterpret_cast<const u32x4 *>(b + off); };
+    if constexpr (FMT == F_Q4_K || FMT == F_Q5_K) {
+        constexpr int QS = FMT == F_Q4_K ? 16 : 48;
+        const int j = e >> 6;
+        r.h = q(0);
+        r.q0 = q(QS + 32 * j);
+        r.q1 = q(QS + 32 * j + 16);
+        if constexpr (FMT == F_Q5_K) {
+            r.qh0 = q(16);
+            r.qh1 = q(32);
+        }
+    } else {
+        static_assert(FMT == F_Q6_K, "staged formats");
+        const int n = e >> 7, kk = (e >> 5) & 3;
+        r.l0 = q(64 * n + 32 * (kk & 1));
+        r.l1 = q(64 * n + 32 * (kk & 1) + 16);
+        r.h0 = q(128 + 32 * n);
+        r.h1 = q(128 + 32 * n + 16);
+        r.sc = *reinterpret_cast<const uint16_t *>(b + 192 + 8 * n + 2 * kk);
+        r.d = *reinterpret_cast<const uint16_t *>(b + 208);
+    }
+}
+
 template <int FMT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xo,
                                                             const float *__restrict__ inv_scale, const float *__restrict__ bias,
                                                             float *__restrict__ y, int m, int n, int k, int split_steps) {
-    __shared__ _Float16 As[2][PF_BN * PF_LD];  // dequantised weights [row][k], two steps
+    using Stage = PfStage<FMT>;
+    constexpr bool STAGED = Stage::ON;
+    extern __shared__ __align__(16) uint8_t pf_smem[];  // pf_lds_bytes<FMT>()
+    _Float16(*As)[PF_BN * PF_LD] = reinterpret_cast<_Float16(*)[PF_BN * PF_LD]>(pf_smem);  // dequantised weights [row][k], two steps
+    uint8_t *Rs = pf_smem + 2 * PF_BN * PF_LD * 2;                                         // staged raw blocks [2][row][RP]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n0 = blockIdx.x * PF_BN, m0 = blockIdx.y * PF_BM;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
@@ -366,10 +452,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // Software pipeline over K: the raw weight bytes and the B operands of a step are requested two steps ahead (a
-    // step of 32 MFMAs per wave is shorter than a trip to HBM); the weights of step s+1 are decoded into registers
-    // (ah) after the MFMAs of step s have been issued.  raw[] alternates, the B operands rotate through three sets,
-    // the LDS tile through two: the loop is unrolled six steps so that all of them are fixed registers.
+    // Software pipeline over K: the B operands of a step are requested two steps ahead (a step of 32 MFMAs per wave
+    // is shorter than a trip to memory), and so are the raw weight bytes of the 32-value formats (raw[] alternates);
+    // the 256-value formats request the blocks of the next four steps during the first of four, park them in
+    // registers (stg) and hand them to LDS during the third.  The weights of step s+1 are decoded into registers
+    // (ah) after the MFMAs of step s have been issued.  The B operands rotate through three sets, the FP16 tile
+    // through two, the staged blocks have a period of four steps: the loop is unrolled twelve steps so that all of
+    // them are fixed registers and addresses.
     // Nothing in a step is conditional - requests past the last step repeat the last step, a half step past the end
     // of a row (K = 32 mod 64) re-reads the row's last block and meets the zeros the operand array holds there - so
     // that the compiler can count the outstanding loads exactly and a step waits only for the loads it consumes.
@@ -377,7 +466,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     PfRaw<FMT> raw[2];
     f16x8 bq[3][2][4];
     // this workgroup's K steps: all of them, or slice blockIdx.z of split_steps steps when the launch splits K (then y
-    // is the slice's own [m, n] array of partial sums, to be added up by prefill_join_kernel)
+    // is the slice's own [m, n] array of partial sums, to be added up by prefill_join_kernel; a slice of a staged
+    // format starts on a multiple of four steps)
     const int sbeg = blockIdx.z * split_steps, nsteps = min((k + PF_BK - 1) / PF_BK, sbeg + split_steps);
     y += (size_t)blockIdx.z * m * n;
     auto wk = [&](int s) { return min(min(s, nsteps - 1) * PF_BK + 32 * dhalf, k - 32); };  // first value this thread decodes in step s
@@ -389,10 +479,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) b[j][ks] = p[((size_t)j * ksteps + ks) * 64];
     };
-    auto decode = [&](const PfRaw<FMT> &r, int s) {  // raw -> FP16 registers, values of each group of four in the order 0, 2, 1, 3
-        const int kk = wk(s);
-
-        if constexpr (FMT == F_Q4_K || FMT == F_Q6_K) {
+    auto decode = [&](const PfRaw<FMT> &r, int kk) {  // raw -> FP16 registers, values of each group of four in the order 0, 2, 1, 3
+        if constexpr (FMT == F_Q4_K || FMT == F_Q5_K || FMT == F_Q6_K) {
             pf_decode_h<FMT>(r, kk, ah);
         } else {
             float v[32];
@@ -403,15 +491,57 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                 for (int i = 0; i < 8; ++i) ah[c][(i & ~3) | pf_perm4(i & 3)] = (_Float16)v[8 * c + i];
         }
     };
-    // one K step: publish the decoded weights, request the loads of step s+2, multiply, decode step s+1
-    auto step = [&](int s, int buf, f16x8(&bcur)[2][4], f16x8(&bfar)[2][4], PfRaw<FMT> &rfar, const PfRaw<FMT> &rnext) {
+    // ---- staging of the 256-value formats: the two threads of a row take its even and its odd 16-byte chunks (every
+    // address is the row's plus a constant); the odd thread of a Q6_K row ends with the block's last two bytes
+    constexpr int NCH = STAGED ? (Stage::CPR + Stage::TAIL + 1) / 2 : 1, RBUF = PF_BN * Stage::RP;
+    const int nblk = k >> 8;
+    u32x4 stg[NCH];
+    auto stage_fetch = [&](int blk) {  // block number blk of the row (clamped: past the end, the last again)
+        const uint8_t *p = wrow + (size_t)min(blk, nblk - 1) * Stage::NB + 16 * dhalf;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            if (32 * i + 32 <= Stage::NB) {
+                stg[i] = ld128<Stage::ALIGN>(p + 32 * i);
+            } else if constexpr (Stage::TAIL) {  // 16 bytes for the even thread, 2 for the odd one
+                const uint8_t *q = p + 32 * i - 14 * dhalf;  // odd: the block's last 16 bytes, the tail in its top half-word
+                stg[i] = ld128<Stage::ALIGN>(q);
+            } else {  // the even thread's last chunk; the odd thread repeats its previous one
+                stg[i] = ld128<Stage::ALIGN>(p + 32 * i - 32 * dhalf);
+            }
+        }
+    };
+    auto stage_store = [&](int buf) {
+        uint8_t *d = Rs + buf * RBUF + drow * Stage::RP + 16 * dhalf;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            if (32 * i + 32 <= Stage::NB) {
+                *reinterpret_cast<u32x4 *>(d + 32 * i) = stg[i];
+            } else if constexpr (Stage::TAIL) {
+                if (dhalf == 0) *reinterpret_cast<u32x4 *>(d + 32 * i) = stg[i];
+                else *reinterpret_cast<uint16_t *>(d + 32 * i) = (uint16_t)(stg[i].w >> 16);
+            } else {
+                if (dhalf == 0) *reinterpret_cast<u32x4 *>(d + 32 * i) = stg[i];
+            }
+        }
+    };
+    // one K step: publish the decoded weights, request the loads of step s+2, multiply, decode step s+1.  ph = s % 4.
+    auto step = [&](int s, int ph, int buf, f16x8(&bcur)[2][4], f16x8(&bfar)[2][4], PfRaw<FMT> &rfar, const PfRaw<FMT> &rnext) {
         {
             f16x8 *da = reinterpret_cast<f16x8 *>(&As[buf][drow * PF_LD + 32 * dhalf]);
 #pragma unroll
             for (int c = 0; c < 4; ++c) da[c] = ah[c];
         }
         __syncthreads();  // the one barrier of the step: the other buffer was read before the previous one
-        fetch_w(rfar, s + 2);
+        PfRaw<FMT> rl;
+        if constexpr (STAGED) {
+            // the staged buffer of steps 4 S .. 4 S + 3 is number S % 2: written during step 4 S - 2, read (for the
+            // decode of the step after) during steps 4 S - 1 .. 4 S + 2, every pair a barrier apart
+            if (ph == 0) stage_fetch((s >> 2) + 1);
+            if (ph == 2) stage_store(((s >> 2) + 1) & 1);
+            pf_load_lds<FMT>(rl, Rs + (((s + 1) >> 2) & 1) * RBUF + drow * Stage::RP, 64 * ((ph + 1) & 3) + 32 * dhalf);
+        } else {
+            fetch_w(rfar, s + 2);
+        }
         fetch_b(bfar, s + 2);
         // ---- 4 k-substeps of 16: lane l supplies row l%32, halves 8*(l/32) .. +8 of the substep.  The weight operands
         // of a substep are read from LDS while the MFMAs of the one before run (one wave per SIMD: nobody else hides
@@ -431,13 +561,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bcur[j][ks], a[ks & 1][i], acc[i][j], 0, 0, 0);
         }
-        decode(rnext, s + 1);
+        if constexpr (STAGED) decode(rl, 64 * ((ph + 1) & 3) + 32 * dhalf);
+        else decode(rnext, wk(s + 1));
         // One wave per SIMD: nobody else fills the matrix pipe while this wave decodes, or the VALU while it multiplies.
         // Ask the scheduler for the interleaving by hand: 32 times one MFMA and a few decode instructions, every other
         // time also one LDS operand read and one of the step's global loads.  The loads are spread over the step on
-        // purpose: issued in one burst after the barrier, the four waves' 44 requests queue up at the CU's one
+        // purpose: issued in one burst after the barrier, the four waves' requests queue up at the CU's one
         // address unit and the waves stall at the issue while the matrix pipe idles.
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4 + Stage::NRAW, 0);
 #pragma unroll
         for (int i = 0; i < 32; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -446,19 +577,29 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
             if (i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
     };
-    fetch_w(raw[0], sbeg);
-    fetch_b(bq[0], sbeg);
-    fetch_w(raw[1], sbeg + 1);
-    fetch_b(bq[1], sbeg + 1);
-    decode(raw[0], sbeg);
+    if constexpr (STAGED) {
+        stage_fetch(sbeg >> 2);
+        stage_store((sbeg >> 2) & 1);
+        __syncthreads();
+        pf_load_lds<FMT>(raw[0], Rs + ((sbeg >> 2) & 1) * RBUF + drow * Stage::RP, 32 * dhalf);
+        fetch_b(bq[0], sbeg);
+        fetch_b(bq[1], sbeg + 1);
+        decode(raw[0], 32 * dhalf);
+    } else {
+        fetch_w(raw[0], sbeg);
+        fetch_b(bq[0], sbeg);
+        fetch_w(raw[1], sbeg + 1);
+        fetch_b(bq[1], sbeg + 1);
+        decode(raw[0], wk(sbeg));
+    }
     int s0 = sbeg;
-    for (; s0 + 6 <= nsteps; s0 += 6) {
+    for (; s0 + 12 <= nsteps; s0 += 12) {
 #pragma unroll
-        for (int u = 0; u < 6; ++u) step(s0 + u, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
+        for (int u = 0; u < 12; ++u) step(s0 + u, u & 3, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
     }
 #pragma unroll
-    for (int u = 0; u < 5; ++u)
-        if (s0 + u < nsteps) step(s0 + u, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
+    for (int u = 0; u < 11; ++u)
+        if (s0 + u < nsteps) step(s0 + u, u & 3, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
     // ---- epilogue.  The activations went in as the first MFMA operand, so an accumulator holds a 32 (tokens) x 32
     // (weight rows) block of y: element r is token 8*(r/4) + 4*(lane/32) + r%4, weight row lane%32 - the 32 lanes of a
     // half wave store 32 consecutive floats of one token's output row.  The 32 token scales of the lane are read
