@@ -165,8 +165,9 @@ def test_small_k_32_blocks_and_many_rows(jn, fmt):
         assert norm_err(y, ref) <= bar(rows), (fmt, rows, norm_err(y, ref))
 
 
-PREFILL_SHAPES = [  # (n, k, rows): ragged tiles in every dimension, K past one step, K split into 8 and into 4 slices
-    (256, 1024, 65), (131, 4096, 200), (64, 14336, 97), (130, 512, 129), (1, 256, 70), (384, 4096, 513),
+PREFILL_SHAPES = [  # (n, k, rows): ragged tiles in every dimension, K past one step, K split into 8 and into 4 slices,
+    # and (the last) into four slices of unequal length: 17 blocks of 256 over slices of whole blocks
+    (256, 1024, 65), (131, 4096, 200), (64, 14336, 97), (130, 512, 129), (1, 256, 70), (384, 4096, 513), (130, 4352, 129),
 ]
 
 
