@@ -172,7 +172,7 @@ __global__ void __launch_bounds__(256) gemv_plain_kernel(const uint8_t *__restri
 // FP32 -> Q8_0, one thread per block of 32 values, in the reference quantiser's arithmetic
 // (core/ops/Quant.java:102-118): amax in double, d = (float)(amax / 127.0) stored as binary16 (round to
 // nearest even), quants = round-half-away(x / (double)d) with the unrounded float d, clamped to +-127.
-__global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restrict__ x, uint8_t *__restrict__ q, size_t blocks) {
+static __global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restrict__ x, uint8_t *__restrict__ q, size_t blocks) {
     for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < blocks; b += (size_t)gridDim.x * blockDim.x) {
         const float *xb = x + b * 32;
         float v[32];

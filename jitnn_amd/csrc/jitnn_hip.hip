@@ -21,6 +21,7 @@
 #include "gguf_file.h"
 #include "glue.h"
 #include "prefill.h"
+#include "tu.h"
 
 using namespace jitnn;
 
@@ -347,31 +348,13 @@ int launch_gemv_xreg_b2(const jitnn_hip_weight *w, const float *x, const float *
     return JITNN_HIP_OK;
 }
 
-typedef void (*mfma_fn)(const uint8_t *, const float *, const float *, float *, int, int, int);
-
-struct MfmaVariant {
-    mfma_fn fn;
-    size_t lds;
-};
-
-MfmaVariant pick_mfma(int fmt) {
-    switch (fmt) {
-    case F_Q4_0: return {gemv_mfma_kernel<F_Q4_0>, gemv_mfma_lds_bytes<F_Q4_0>()};
-    case F_Q4_1: return {gemv_mfma_kernel<F_Q4_1>, gemv_mfma_lds_bytes<F_Q4_1>()};
-    case F_Q8_0: return {gemv_mfma_kernel<F_Q8_0>, gemv_mfma_lds_bytes<F_Q8_0>()};
-    case F_Q4_K: return {gemv_mfma_kernel<F_Q4_K>, gemv_mfma_lds_bytes<F_Q4_K>()};
-    case F_Q5_K: return {gemv_mfma_kernel<F_Q5_K>, gemv_mfma_lds_bytes<F_Q5_K>()};
-    case F_Q6_K: return {gemv_mfma_kernel<F_Q6_K>, gemv_mfma_lds_bytes<F_Q6_K>()};
-    default: return {nullptr, 0};
-    }
-}
-
-// Batch 2..8, rows a multiple of 256 values long: block sums on the matrix cores, one workgroup of 16 waves per CU.
-int launch_gemv_mfma(const MfmaVariant &v, const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
-    if (int rc = allow_lds((const void *)v.fn, v.lds)) return rc;
+// Batch 2..8, rows a multiple of 256 values long: block sums on the matrix cores, one workgroup of 8 waves per CU
+// (the kernels live in gemv_mfma.hip).
+int launch_gemv_mfma(const KernelRef &v, const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    if (int rc = allow_lds(v.fn, v.lds)) return rc;
     const int groups = (w->n + 15) / 16;
     const int blocks = groups < g.cus ? groups : g.cus;
-    hipLaunchKernelGGL(v.fn, dim3(blocks), dim3(MF_THREADS), v.lds, stream, w->dev, x, bias, y, w->n, w->k, rows);
+    gemv_mfma_launch(w->fmt, (unsigned)blocks, stream, w->dev, x, bias, y, w->n, w->k, rows);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
@@ -394,7 +377,7 @@ int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float
     // Q6_K pays the most per weight on the matrix-core path (6-bit quants from two arrays, 16-value scale groups): up to
     // four rows its FP32 kernel is still ahead (measured: 33 vs 43 us at 2 rows, 151 vs 167 us at 4 rows on the output head)
     if (rows >= (w->fmt == F_Q6_K ? 5 : 2) && rows <= 8 && w->k % 256 == 0 && w->n >= 16 && g.batch_mfma) {
-        const MfmaVariant v = pick_mfma(w->fmt);
+        const KernelRef v = gemv_mfma_kernel_ref(w->fmt);
         if (v.fn && v.lds <= g.max_lds) return launch_gemv_mfma(v, w, x, rows, bias, y, stream);
     }
     if (rows == 1 && !g.force_lds) {
@@ -463,18 +446,13 @@ int workspace_done(hipStream_t stream) {
     return JITNN_HIP_OK;
 }
 
-template <int FMT>
-int launch_prefill_fmt(const jitnn_hip_weight *w, const _Float16 *xo, const float *inv, int rows, const float *bias, float *y, int splits,
-                       int split_steps, hipStream_t s) {
-    constexpr size_t lds = pf_lds_bytes<FMT>();
-    if (int rc = allow_lds((const void *)prefill_mfma_kernel<FMT>, lds)) return rc;
-    dim3 grid((w->n + PF_BN - 1) / PF_BN, (rows + PF_BM - 1) / PF_BM, splits);
-    hipLaunchKernelGGL(prefill_mfma_kernel<FMT>, grid, dim3(256), lds, s, w->dev, xo, inv, bias, y, rows, w->n, w->k, split_steps);
-    return JITNN_HIP_OK;
-}
-
 // more rows than the GEMV kernels take: FP16 activations in operand order + dequantise-to-LDS MFMA kernel
 int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    // (the kernels live in prefill_k.hip and prefill_q32.hip)
+    const bool kq = block_values(w->fmt) == 256;
+    const KernelRef kr = kq ? prefill_kernel_k(w->fmt) : prefill_kernel_q32(w->fmt);
+    if (!kr.fn) return fail(JITNN_HIP_EUNSUPPORTED, "no many-row kernel for format %d", w->fmt);
+    if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
     const int mtiles = (rows + PF_BM - 1) / PF_BM, mblocks = mtiles * (PF_BM / 32);  // operands padded to whole tiles of tokens
     const int ntiles = (w->n + PF_BN - 1) / PF_BN, nsteps = (w->k + PF_BK - 1) / PF_BK;
     // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 16 steps writes its own
@@ -494,35 +472,17 @@ int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const fl
     _Float16 *xo = (_Float16 *)ws;
     float *scale = (float *)((uint8_t *)ws + xo_bytes), *inv = scale + rows;
     float *part = (float *)((uint8_t *)ws + xo_bytes + scale_bytes);
-    if (w->k <= XP_MAXK) {
-        const int pieces = pf_ksteps(w->k) * 2;  // per row; 256 threads take J each
-        if (pieces <= 512) hipLaunchKernelGGL(x_prepare_kernel<2>, dim3(mblocks * 32), dim3(256), 0, stream, x, inv, xo, rows, w->k);
-        else if (pieces <= 1024) hipLaunchKernelGGL(x_prepare_kernel<4>, dim3(mblocks * 32), dim3(256), 0, stream, x, inv, xo, rows, w->k);
-        else hipLaunchKernelGGL(x_prepare_kernel<8>, dim3(mblocks * 32), dim3(256), 0, stream, x, inv, xo, rows, w->k);
-    } else {
-        hipLaunchKernelGGL(x_row_scale_kernel, dim3(rows), dim3(256), 0, stream, x, scale, inv, w->k);
-        hipLaunchKernelGGL(x_to_operand_kernel, dim3(mblocks, pf_ksteps(w->k) / 4), dim3(256), 0, stream, x, scale, xo, rows, w->k);
-    }
+    prefill_prepare_launch(x, scale, inv, xo, rows, w->k, mblocks, stream);
     float *out = splits > 1 ? part : y;
     const float *b1 = splits > 1 ? nullptr : bias;
-    int rc = JITNN_HIP_OK;
-    switch (w->fmt) {
-    case F_Q4_0: rc = launch_prefill_fmt<F_Q4_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q4_1: rc = launch_prefill_fmt<F_Q4_1>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q8_0: rc = launch_prefill_fmt<F_Q8_0>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q4_K: rc = launch_prefill_fmt<F_Q4_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    case F_Q5_K: rc = launch_prefill_fmt<F_Q5_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    default: rc = launch_prefill_fmt<F_Q6_K>(w, xo, inv, rows, b1, out, splits, split_steps, stream); break;
-    }
-    if (rc) {
-        workspace_done(stream);
-        return rc;
-    }
+    const dim3 grid(ntiles, mtiles, splits);
+    if (kq) prefill_launch_k(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, w->k, split_steps);
+    else prefill_launch_q32(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, w->k, split_steps);
     if (splits > 1) {
         const size_t count4 = (size_t)rows * w->n / 4;
         size_t blocks = (count4 + 255) / 256;
         if (blocks > (size_t)g.cus * 8) blocks = (size_t)g.cus * 8;
-        hipLaunchKernelGGL(prefill_join_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, part, bias, y, count4, w->n, splits);
+        prefill_join_launch(part, bias, y, count4, w->n, splits, (unsigned)blocks, stream);
     }
     HIP_TRY(hipGetLastError());
     return workspace_done(stream);

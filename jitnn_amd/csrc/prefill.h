@@ -28,7 +28,7 @@ constexpr int PF_BN = 128, PF_BM = 256, PF_BK = 64, PF_LD = PF_BK + 8;  // LDS r
 __host__ __device__ constexpr int pf_perm4(int i) { return ((i & 1) << 1) | (i >> 1); }
 
 // One workgroup per activation row: amax -> scale = 2^(13 - floor(log2 amax)) and 1/scale for the epilogue.
-__global__ void __launch_bounds__(256) x_row_scale_kernel(const float *__restrict__ x, float *__restrict__ scale, float *__restrict__ inv_scale,
+static __global__ void __launch_bounds__(256) x_row_scale_kernel(const float *__restrict__ x, float *__restrict__ scale, float *__restrict__ inv_scale,
                                                            int k) {
     __shared__ float red[4];
     const float4 *xr = reinterpret_cast<const float4 *>(x + (size_t)blockIdx.x * k);  // k is a multiple of 32
@@ -60,7 +60,7 @@ __host__ __device__ constexpr int pf_ksteps(int k) { return (k + PF_BK - 1) / PF
 // 32 mb + l % 32, values 16 ks + 8 (l / 32) .. + 7, each group of four values in the order 0, 2, 1, 3 (the order in
 // which the weight decoder produces FP16 pairs from a dword of quants; a dot product only needs both to agree).
 // Tokens past m and values past k are zeros.  grid (token blocks, K / 64), 256 threads: one 16-byte piece each.
-__global__ void __launch_bounds__(256) x_to_operand_kernel(const float *__restrict__ x, const float *__restrict__ scale,
+static __global__ void __launch_bounds__(256) x_to_operand_kernel(const float *__restrict__ x, const float *__restrict__ scale,
                                                             _Float16 *__restrict__ xo, int m, int k) {
     // 32 tokens x 64 values through LDS: the reads run along the token rows (256 contiguous bytes each), the writes
     // along the operand order (1 KiB per K step)
@@ -457,8 +457,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     // the 256-value formats request the blocks of the next four steps during the first of four, park them in
     // registers (stg) and hand them to LDS during the third.  The weights of step s+1 are decoded into registers
     // (ah) after the MFMAs of step s have been issued.  The B operands rotate through three sets, the FP16 tile
-    // through two, the staged blocks have a period of four steps: the loop is unrolled twelve steps so that all of
-    // them are fixed registers and addresses.
+    // through two, the staged blocks have a period of four steps: the loop is unrolled six steps (twelve for the
+    // staged formats) so that all of them are fixed registers and addresses.
     // Nothing in a step is conditional - requests past the last step repeat the last step, a half step past the end
     // of a row (K = 32 mod 64) re-reads the row's last block and meets the zeros the operand array holds there - so
     // that the compiler can count the outstanding loads exactly and a step waits only for the loads it consumes.
@@ -592,13 +592,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
         fetch_b(bq[1], sbeg + 1);
         decode(raw[0], wk(sbeg));
     }
+    constexpr int UNR = STAGED ? 12 : 6;  // lcm of the rotation periods: 3 operand sets, 2 tiles (and raw sets), 4 steps per staged block
     int s0 = sbeg;
-    for (; s0 + 12 <= nsteps; s0 += 12) {
+    for (; s0 + UNR <= nsteps; s0 += UNR) {
 #pragma unroll
-        for (int u = 0; u < 12; ++u) step(s0 + u, u & 3, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
+        for (int u = 0; u < UNR; ++u) step(s0 + u, u & 3, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
     }
 #pragma unroll
-    for (int u = 0; u < 11; ++u)
+    for (int u = 0; u < UNR - 1; ++u)
         if (s0 + u < nsteps) step(s0 + u, u & 3, u & 1, bq[u % 3], bq[(u + 2) % 3], raw[u & 1], raw[(u + 1) & 1]);
     // ---- epilogue.  The activations went in as the first MFMA operand, so an accumulator holds a 32 (tokens) x 32
     // (weight rows) block of y: element r is token 8*(r/4) + 4*(lane/32) + r%4, weight row lane%32 - the 32 lanes of a
@@ -636,7 +637,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 
 // y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]), slices in order: the second half of a
 // split-K launch.  count4 = m * n / 4 (n is a multiple of 4 whenever the launch splits).
-__global__ void __launch_bounds__(256) prefill_join_kernel(const float *__restrict__ part, const float *__restrict__ bias, float *__restrict__ y,
+static __global__ void __launch_bounds__(256) prefill_join_kernel(const float *__restrict__ part, const float *__restrict__ bias, float *__restrict__ y,
                                                             size_t count4, int n, int splits) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count4; i += (size_t)gridDim.x * 256) {
         float4 a = reinterpret_cast<const float4 *>(part)[i];

@@ -1,0 +1,26 @@
+// prefill_mfma_kernel for the 256-value formats.
+#include "prefill.h"
+#include "tu.h"
+
+namespace jitnn {
+
+KernelRef prefill_kernel_k(int fmt) {
+    switch (fmt) {
+    case F_Q4_K: return {(const void *)prefill_mfma_kernel<F_Q4_K>, pf_lds_bytes<F_Q4_K>()};
+    case F_Q5_K: return {(const void *)prefill_mfma_kernel<F_Q5_K>, pf_lds_bytes<F_Q5_K>()};
+    case F_Q6_K: return {(const void *)prefill_mfma_kernel<F_Q6_K>, pf_lds_bytes<F_Q6_K>()};
+    default: return {nullptr, 0};
+    }
+}
+
+void prefill_launch_k(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const _Float16 *xo, const float *inv_scale, const float *bias, float *y,
+                      int m, int n, int k, int split_steps) {
+    switch (fmt) {
+    case F_Q4_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_K>, grid, dim3(256), pf_lds_bytes<F_Q4_K>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
+    case F_Q5_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q5_K>, grid, dim3(256), pf_lds_bytes<F_Q5_K>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
+    case F_Q6_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q6_K>, grid, dim3(256), pf_lds_bytes<F_Q6_K>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
+    default: break;
+    }
+}
+
+}  // namespace jitnn

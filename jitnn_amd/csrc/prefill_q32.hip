@@ -1,0 +1,42 @@
+// prefill_mfma_kernel for the 32-value formats, the activation preparation and the join of K slices.
+#include "prefill.h"
+#include "tu.h"
+
+namespace jitnn {
+
+KernelRef prefill_kernel_q32(int fmt) {
+    switch (fmt) {
+    case F_Q4_0: return {(const void *)prefill_mfma_kernel<F_Q4_0>, pf_lds_bytes<F_Q4_0>()};
+    case F_Q4_1: return {(const void *)prefill_mfma_kernel<F_Q4_1>, pf_lds_bytes<F_Q4_1>()};
+    case F_Q8_0: return {(const void *)prefill_mfma_kernel<F_Q8_0>, pf_lds_bytes<F_Q8_0>()};
+    default: return {nullptr, 0};
+    }
+}
+
+void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const _Float16 *xo, const float *inv_scale, const float *bias, float *y,
+                        int m, int n, int k, int split_steps) {
+    switch (fmt) {
+    case F_Q4_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_0>, grid, dim3(256), pf_lds_bytes<F_Q4_0>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
+    case F_Q4_1: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_1>, grid, dim3(256), pf_lds_bytes<F_Q4_1>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
+    case F_Q8_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q8_0>, grid, dim3(256), pf_lds_bytes<F_Q8_0>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
+    default: break;
+    }
+}
+
+void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, hipStream_t s) {
+    if (k <= XP_MAXK) {
+        const int pieces = pf_ksteps(k) * 2;  // per row; 256 threads take J each
+        if (pieces <= 512) hipLaunchKernelGGL(x_prepare_kernel<2>, dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k);
+        else if (pieces <= 1024) hipLaunchKernelGGL(x_prepare_kernel<4>, dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k);
+        else hipLaunchKernelGGL(x_prepare_kernel<8>, dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k);
+    } else {
+        hipLaunchKernelGGL(x_row_scale_kernel, dim3(rows), dim3(256), 0, s, x, scale, inv_scale, k);
+        hipLaunchKernelGGL(x_to_operand_kernel, dim3(mblocks, pf_ksteps(k) / 4), dim3(256), 0, s, x, scale, xo, rows, k);
+    }
+}
+
+void prefill_join_launch(const float *part, const float *bias, float *y, size_t count4, int n, int splits, unsigned blocks, hipStream_t s) {
+    hipLaunchKernelGGL(prefill_join_kernel, dim3(blocks), dim3(256), 0, s, part, bias, y, count4, n, splits);
+}
+
+}  // namespace jitnn

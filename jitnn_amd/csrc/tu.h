@@ -1,0 +1,33 @@
+// Host entry points of the translation units that hold the matrix-core kernels.  The library is several .hip files so
+// that it builds in parallel: every kernel template is instantiated in exactly one of them, the others reach it
+// through the plain functions below (C++ linkage, hidden like everything that is not in include/jitnn_hip.h).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace jitnn {
+
+// a kernel and the dynamic LDS it needs (for hipFuncSetAttribute when that is more than 64 KiB); fn == nullptr: no such format
+struct KernelRef {
+    const void *fn;
+    size_t lds;
+};
+
+// ---- prefill_k.hip (Q4_K, Q5_K, Q6_K) and prefill_q32.hip (Q4_0, Q4_1, Q8_0): prefill_mfma_kernel<fmt>
+KernelRef prefill_kernel_k(int fmt);
+KernelRef prefill_kernel_q32(int fmt);
+void prefill_launch_k(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const _Float16 *xo, const float *inv_scale, const float *bias, float *y,
+                      int m, int n, int k, int split_steps);
+void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const _Float16 *xo, const float *inv_scale, const float *bias, float *y,
+                        int m, int n, int k, int split_steps);
+// activation preparation and the join of K slices (prefill_q32.hip)
+void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, hipStream_t s);
+void prefill_join_launch(const float *part, const float *bias, float *y, size_t count4, int n, int splits, unsigned blocks, hipStream_t s);
+
+// ---- gemv_mfma.hip: gemv_mfma_kernel<fmt>
+KernelRef gemv_mfma_kernel_ref(int fmt);
+void gemv_mfma_launch(int fmt, unsigned blocks, hipStream_t s, const uint8_t *W, const float *x, const float *bias, float *y, int n, int k, int rows);
+
+}  // namespace jitnn
