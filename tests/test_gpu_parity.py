@@ -166,8 +166,9 @@ def test_small_k_32_blocks_and_many_rows(jn, fmt):
 
 
 PREFILL_SHAPES = [  # (n, k, rows): ragged tiles in every dimension, K past one step, K split into 8 and into 4 slices,
-    # and (the last) into four slices of unequal length: 17 blocks of 256 over slices of whole blocks
+    # and (130 x 4352) into four slices of unequal length: 17 blocks of 256 over slices of whole blocks
     (256, 1024, 65), (131, 4096, 200), (64, 14336, 97), (130, 512, 129), (1, 256, 70), (384, 4096, 513), (130, 4352, 129),
+    (40, 16640, 70),  # rows longer than the one-launch activation preparation takes: scale and conversion in two launches
 ]
 
 
