@@ -263,6 +263,30 @@ def bench_decode(torch, lib, steps, warmup):
         out["graph_matches_direct"] = bool(torch.equal(ref, logits))
     except Exception as e:  # report, never hide
         out["graph_error"] = f"{type(e).__name__}: {e}"
+    # the prompt side of config 5: 512 tokens through the same 32 layers in one call (linears on the matrix-core path,
+    # causal attention, keys and values appended), then the last token's logits against 512 single-token steps
+    try:
+        xs = torch.randn(512, 4096, device="cuda", generator=torch.Generator(device="cuda").manual_seed(12))
+        pl = torch.empty(cfg["vocab"], device="cuda")
+        for _ in range(2):
+            dec.prefill_dev(xs.data_ptr(), 0, 512, pl.data_ptr(), st)
+        torch.cuda.synchronize()
+        reps = 5
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            dec.prefill_dev(xs.data_ptr(), 0, 512, pl.data_ptr(), st)
+        torch.cuda.synchronize()
+        pw = (time.perf_counter() - t0) / reps
+        for t in range(512):
+            dec.decode_dev(xs[t].data_ptr(), t, logits.data_ptr(), st)
+        torch.cuda.synchronize()
+        err = float((pl - logits).abs().max() / logits.abs().max())
+        flops = 2.0 * 512 * sum(n * k for _, n, k in shapes) * cfg["layers"] + 2.0 * cfg["vocab"] * 4096
+        out["prefill_512"] = {"workload": "the same model on a 512-token prompt from an empty cache, one call", "ms": pw * 1e3,
+                              "tokens_per_s": 512 / pw, "linear_TFLOPs": flops / pw / 1e12,
+                              "last_logits_vs_512_decode_steps_norm_err": err, "logits_finite": bool(torch.isfinite(pl).all().item())}
+    except Exception as e:  # report, never hide
+        out["prefill_512_error"] = f"{type(e).__name__}: {e}"
     for h in handles + [hh]:
         lib.lib.jitnn_hip_weight_free(h)
     dec.close()

@@ -210,6 +210,16 @@ JITNN_HIP_API int jitnn_hip_llama_kv_read(const jitnn_hip_llama *m, int layer, i
 JITNN_HIP_API int jitnn_hip_llama_decode(jitnn_hip_llama *m, const float *x_host, int pos, float *logits_host);
 JITNN_HIP_API int jitnn_hip_llama_decode_dev(jitnn_hip_llama *m, const float *x_dev, int pos, float *logits_dev, void *stream);
 
+/* Many tokens at once (the prompt): x [tokens, d_model] are the embeddings of the tokens at positions pos0 ..
+ * pos0 + tokens - 1 (the cache must hold positions 0..pos0-1); every layer runs its linears on all rows (more than 64
+ * rows: the matrix-core path of jitnn_hip_linear_dev), attention is causal; appends all keys and values and writes the
+ * logits [vocab] of the last token (logits may be NULL).  Same arithmetic per token as jitnn_hip_llama_decode, i.e.
+ * Llama.Block.forward (jitnn-nn/.../nn/models/Llama.java:209-222) on a [1, tokens, d_model] input.  The first call, and
+ * any call with more tokens than every call before, allocates the model's many-token buffers (so it is not for HIP
+ * graph capture). */
+JITNN_HIP_API int jitnn_hip_llama_prefill(jitnn_hip_llama *m, const float *x_host, int pos0, int tokens, float *logits_host);
+JITNN_HIP_API int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0, int tokens, float *logits_dev, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

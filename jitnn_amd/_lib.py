@@ -66,6 +66,8 @@ def _bind() -> C.CDLL:
         "jitnn_hip_llama_kv_read": (i, [vp, i, i, i, vp, vp]),
         "jitnn_hip_llama_decode": (i, [vp, vp, i, vp]),
         "jitnn_hip_llama_decode_dev": (i, [vp, vp, i, vp, vp]),
+        "jitnn_hip_llama_prefill": (i, [vp, vp, i, i, vp]),
+        "jitnn_hip_llama_prefill_dev": (i, [vp, vp, i, i, vp, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol

@@ -140,11 +140,10 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
 // A separate launch on purpose: publishing the partial results to another workgroup inside one kernel needs
 // device-scope fences, which cost several times this kernel on a part with one L2 per XCD.
 template <int D>
-__global__ void __launch_bounds__(2 * D) attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int chunks) {
+__device__ __forceinline__ void attn_merge_body(const float *__restrict__ p, float *__restrict__ out, int chunks) {
     constexpr int U = 16;
     __shared__ float sm[3][D];
-    const int h = blockIdx.x, d = threadIdx.x % D, half = threadIdx.x / D;
-    const float *p = part + (size_t)h * chunks * (D + 2);
+    const int d = threadIdx.x % D, half = threadIdx.x / D;
     float m = -INFINITY, l = 0.f, acc = 0.f;
     for (int c0 = half; c0 < chunks; c0 += 2 * U) {
         float mm[U], ll[U], aa[U];
@@ -180,7 +179,218 @@ __global__ void __launch_bounds__(2 * D) attn_merge_kernel(const float *__restri
             l = l * a + l1 * b;
             acc = acc * a + a1 * b;
         }
-        out[(size_t)h * D + d] = acc / l;
+        out[d] = acc / l;
+    }
+}
+
+template <int D>
+__global__ void __launch_bounds__(2 * D) attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int chunks) {
+    const int h = blockIdx.x;
+    attn_merge_body<D>(part + (size_t)h * chunks * (D + 2), out + (size_t)h * D, chunks);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Many tokens at once (prefill): the same operators row by row.  T tokens at positions pos0 .. pos0 + T - 1 attend
+// causally to the cache (which must hold positions 0 .. pos0 - 1) and to one another.
+
+// y[r] = RMSNorm(x[r]) for every row: one workgroup of 256 per row (ops/RowNorm.java:286-306, RMS branch).
+__global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float *__restrict__ x, const float *__restrict__ w, float *__restrict__ y, int n,
+                                                             float eps) {
+    __shared__ float red[4];
+    const float *xr = x + (size_t)blockIdx.x * n;
+    float *yr = y + (size_t)blockIdx.x * n;
+    float s = 0.f;
+#pragma unroll 8
+    for (int i = threadIdx.x; i < n; i += 256) s = __builtin_fmaf(xr[i], xr[i], s);
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    s = (red[0] + red[1]) + (red[2] + red[3]);
+    const float is = 1.f / sqrtf(s / (float)n + eps);
+#pragma unroll 8
+    for (int i = threadIdx.x; i < n; i += 256) yr[i] = xr[i] * is * w[i];
+}
+
+// Rotary embedding of the query heads in place (q [T, heads, D]) and of the key heads on their way into the cache,
+// values copied into the cache: token t = blockIdx.x sits at position pos0 + t.  Same rotation as attn_decode_kernel.
+__global__ void __launch_bounds__(256) rope_append_rows_kernel(float *__restrict__ q, const float *__restrict__ k, const float *__restrict__ v,
+                                                                float *__restrict__ kcache, float *__restrict__ vcache,
+                                                                const float *__restrict__ cosv, const float *__restrict__ sinv, int heads, int kv_heads,
+                                                                int D, int pos0) {
+    const int t = blockIdx.x, pos = pos0 + t, half = D / 2;
+    const float *cp = cosv + (size_t)pos * half, *sp = sinv + (size_t)pos * half;
+    float *qt = q + (size_t)t * heads * D;
+    for (int i = threadIdx.x; i < heads * half; i += 256) {
+        const int h = i / half, p = i - h * half;
+        const float a = qt[h * D + p], b = qt[h * D + p + half], cs = cp[p], sn = sp[p];
+        qt[h * D + p] = a * cs - b * sn;
+        qt[h * D + p + half] = a * sn + b * cs;
+    }
+    const float *kt = k + (size_t)t * kv_heads * D, *vt = v + (size_t)t * kv_heads * D;
+    float *kc = kcache + (size_t)pos * kv_heads * D, *vc = vcache + (size_t)pos * kv_heads * D;
+    for (int i = threadIdx.x; i < kv_heads * half; i += 256) {
+        const int h = i / half, p = i - h * half;
+        const float a = kt[h * D + p], b = kt[h * D + p + half], cs = cp[p], sn = sp[p];
+        kc[h * D + p] = a * cs - b * sn;
+        kc[h * D + p + half] = a * sn + b * cs;
+    }
+    for (int i = threadIdx.x; i < kv_heads * D; i += 256) vc[i] = vt[i];
+}
+
+// Attention of a block of consecutive tokens over one chunk of CH keys: the (token, query head) pairs of one
+// key/value head - ATT_ROWS = 64 rows, i.e. 64 / group tokens - share the LDS copy of the chunk; row r = tq * group + h
+// sees key j when j <= pos0 + t0 + tq (causal).  q is already rotated, every key comes from the cache.
+// Register tiles instead of one LDS read per multiply-add: a thread owns 4 rows x CH/16 keys of the scores (the 16
+// threads of a DPP row hold all keys of their 4 rows, so the softmax statistics are two DPP reductions and the
+// probabilities go to the weighted value sum through LDS without a workgroup barrier) and 4 rows x D/16 values of the
+// output.  Per-chunk results go to `part` for attn_merge_rows_kernel, as in the one-token kernels.
+//   grid (chunks of the last token, kv_heads, token blocks), 256 threads, attn_prefill_lds_bytes<D>() of dynamic LDS;
+//   part [T, heads, chunks_max, D + 2].
+constexpr int ATT_ROWS = 64;
+template <int D>
+constexpr size_t attn_prefill_lds_bytes() {
+    return sizeof(float) * ((size_t)ATT_ROWS * D + (size_t)AttCfg<D>::CH * (D + 4) + (size_t)AttCfg<D>::CH * D + (size_t)AttCfg<D>::CH * (ATT_ROWS + 4));
+}
+template <int D>
+__global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restrict__ q, const float *__restrict__ kcache,
+                                                            const float *__restrict__ vcache, float *__restrict__ part, int heads, int kv_heads, int pos0,
+                                                            int T, int chunks_max, float scale) {
+    constexpr int CH = AttCfg<D>::CH, DQ = D / 4, KN = CH / 16, DV = D / 16, KP = D + 4, PP = ATT_ROWS + 4;
+    static_assert(D % 64 == 0 && CH % 16 == 0, "tiles of 16 threads");
+    extern __shared__ __align__(16) float att_smem[];
+    float *Qs = att_smem;             // [ATT_ROWS][D]
+    float *Ks = Qs + ATT_ROWS * D;    // [CH][D + 4]
+    float *Vs = Ks + CH * KP;         // [CH][D]
+    float *Pt = Vs + CH * D;          // [CH][ATT_ROWS + 4]: probabilities, key-major
+    const int tid = threadIdx.x, rg = tid >> 4, kl = tid & 15;
+    const int group = heads / kv_heads, QT = ATT_ROWS / group, rows = QT * group;
+    const int g = blockIdx.y, c = blockIdx.x, t0 = blockIdx.z * QT;
+    const int tl = min(t0 + QT, T) - 1;  // last token of the block
+    const int j0 = c * CH;
+    if (j0 > pos0 + tl) return;  // no key of this chunk is visible to any token of the block (uniform)
+    const int nk = min(CH, pos0 + tl + 1 - j0);
+    for (int i = tid; i < ATT_ROWS * DQ; i += 256) {
+        const int r = i / DQ, e = (i - r * DQ) * 4, tq = r / group, h = r - tq * group;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (r < rows && t0 + tq < T) v = *reinterpret_cast<const float4 *>(q + ((size_t)(t0 + tq) * heads + g * group + h) * D + e);
+        *reinterpret_cast<float4 *>(&Qs[r * D + e]) = v;
+    }
+    for (int i = tid; i < CH * DQ; i += 256) {
+        const int j = i / DQ, e = (i - j * DQ) * 4;
+        float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), vv = kk;
+        if (j < nk) {
+            const size_t row = ((size_t)(j0 + j) * kv_heads + g) * D;
+            kk = *reinterpret_cast<const float4 *>(kcache + row + e);
+            vv = *reinterpret_cast<const float4 *>(vcache + row + e);
+        }
+        *reinterpret_cast<float4 *>(&Ks[j * KP + e]) = kk;
+        *reinterpret_cast<float4 *>(&Vs[j * D + e]) = vv;
+    }
+    __syncthreads();
+    // ---- scores of rows 4 rg .. + 3 against keys kl + 16 n
+    float sc[4][KN];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int n = 0; n < KN; ++n) sc[i][n] = 0.f;
+#pragma unroll 4
+    for (int d4 = 0; d4 < DQ; ++d4) {
+        float4 qv[4], kv[KN];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const float4 *>(&Qs[(4 * rg + i) * D + 4 * d4]);
+#pragma unroll
+        for (int n = 0; n < KN; ++n) kv[n] = *reinterpret_cast<const float4 *>(&Ks[(kl + 16 * n) * KP + 4 * d4]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int n = 0; n < KN; ++n) {
+                sc[i][n] = __builtin_fmaf(qv[i].x, kv[n].x, sc[i][n]);
+                sc[i][n] = __builtin_fmaf(qv[i].y, kv[n].y, sc[i][n]);
+                sc[i][n] = __builtin_fmaf(qv[i].z, kv[n].z, sc[i][n]);
+                sc[i][n] = __builtin_fmaf(qv[i].w, kv[n].w, sc[i][n]);
+            }
+    }
+    // ---- softmax statistics of each row over the chunk (the row's keys sit in the 16 lanes of this DPP row)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = 4 * rg + i, tq = r / group, h = r - tq * group;
+        const bool live = r < rows && t0 + tq < T;
+        float m = -INFINITY;
+#pragma unroll
+        for (int n = 0; n < KN; ++n) {
+            const bool seen = live && j0 + kl + 16 * n <= pos0 + t0 + tq;
+            sc[i][n] = seen ? sc[i][n] * scale : -INFINITY;
+            m = fmaxf(m, sc[i][n]);
+        }
+        m = row_max(m);
+        float l = 0.f;
+#pragma unroll
+        for (int n = 0; n < KN; ++n) {
+            const float p = sc[i][n] > -INFINITY ? __expf(sc[i][n] - m) : 0.f;
+            Pt[(kl + 16 * n) * PP + r] = p;
+            l += p;
+        }
+        l = row_sum(l);
+        if (kl == 0 && live) {
+            float *o = part + (((size_t)(t0 + tq) * heads + g * group + h) * chunks_max + c) * (D + 2);
+            o[D] = m;
+            o[D + 1] = l;
+        }
+    }
+    // the probabilities of rows 4 rg .. + 3 were written by the 16 lanes that read them below: a wave-level hand-off
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // ---- unnormalised weighted value sums: rows 4 rg .. + 3, values DV kl .. + DV - 1
+    float4 acc[4][DV / 4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int e = 0; e < DV / 4; ++e) acc[i][e] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+    for (int j = 0; j < CH; ++j) {
+        const float4 p = *reinterpret_cast<const float4 *>(&Pt[j * PP + 4 * rg]);
+        const float pr[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+        for (int e = 0; e < DV / 4; ++e) {
+            const float4 v = *reinterpret_cast<const float4 *>(&Vs[j * D + DV * kl + 4 * e]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[i][e].x = __builtin_fmaf(pr[i], v.x, acc[i][e].x);
+                acc[i][e].y = __builtin_fmaf(pr[i], v.y, acc[i][e].y);
+                acc[i][e].z = __builtin_fmaf(pr[i], v.z, acc[i][e].z);
+                acc[i][e].w = __builtin_fmaf(pr[i], v.w, acc[i][e].w);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = 4 * rg + i, tq = r / group, h = r - tq * group;
+        if (r < rows && t0 + tq < T) {
+            float *o = part + (((size_t)(t0 + tq) * heads + g * group + h) * chunks_max + c) * (D + 2) + DV * kl;
+#pragma unroll
+            for (int e = 0; e < DV / 4; ++e) {  // (D + 2 floats per record: 8-byte aligned, so two 64-bit stores)
+                *reinterpret_cast<float2 *>(o + 4 * e) = make_float2(acc[i][e].x, acc[i][e].y);
+                *reinterpret_cast<float2 *>(o + 4 * e + 2) = make_float2(acc[i][e].z, acc[i][e].w);
+            }
+        }
+    }
+}
+
+// attn_merge_kernel per (query head, token): token t merges the chunks that hold keys up to its own position.
+template <int D>
+__global__ void __launch_bounds__(2 * D) attn_merge_rows_kernel(const float *__restrict__ part, float *__restrict__ out, int heads, int pos0,
+                                                                 int chunks_max) {
+    const int h = blockIdx.x, t = blockIdx.y;
+    const int chunks = (pos0 + t + AttCfg<D>::CH) / AttCfg<D>::CH;  // ceil((pos0 + t + 1) / CH)
+    attn_merge_body<D>(part + ((size_t)t * heads + h) * chunks_max * (D + 2), out + ((size_t)t * heads + h) * D, chunks);
+}
+
+// y = a + b, four values per thread (the residual connections of many rows)
+__global__ void __launch_bounds__(256) add_rows_kernel(const float4 *__restrict__ a, const float4 *__restrict__ b, float4 *__restrict__ y, size_t count4) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count4; i += (size_t)gridDim.x * 256) {
+        const float4 u = a[i], w = b[i];
+        y[i] = make_float4(u.x + w.x, u.y + w.y, u.z + w.z, u.w + w.w);
     }
 }
 

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -910,6 +911,9 @@ struct jitnn_hip_llama {
     float *cosv, *sinv;          // [max_ctx][hd/2]
     float *xin, *xa, *xb, *xn, *q, *k, *v, *att, *gate, *up, *h, *part, *logits;
     int chunks_max;
+    // many-token (prefill) buffers, [pf_cap, ...] each, allocated by the first prefill call and grown when a longer one comes
+    int pf_cap, pf_chunks;
+    float *pf[11];  // xn, q, k, v, att, xa, xb, gate, up, h, part
 };
 
 namespace {
@@ -970,6 +974,47 @@ int check_model(const jitnn_hip_llama *m) {
         for (int i = 0; i < 7; ++i)
             if (!m->w[l * 7 + i]) return fail(JITNN_HIP_EINVAL, "layer %d has no weight %d", l, i);
     if (!m->w_out) return fail(JITNN_HIP_EINVAL, "no output weight");
+    return JITNN_HIP_OK;
+}
+
+// The many-token buffers of a model, for at least `tokens` rows.
+int ensure_prefill(jitnn_hip_llama *m, int tokens) {
+    if (tokens <= m->pf_cap) return JITNN_HIP_OK;
+    HIP_TRY(hipDeviceSynchronize());  // earlier calls may still use the old buffers
+    for (float *&b : m->pf) {
+        if (b) (void)hipFree(b);
+        b = nullptr;
+    }
+    m->pf_cap = 0;
+    const int ch = m->hd <= 128 ? 32 : 16;  // AttCfg<D>::CH
+    m->pf_chunks = (m->max_ctx + ch - 1) / ch;
+    const size_t qd = (size_t)m->heads * m->hd, kd = (size_t)m->kv * m->hd;
+    const size_t per[11] = {(size_t)m->d, qd, kd, kd, qd, (size_t)m->d, (size_t)m->d, (size_t)m->ffn, (size_t)m->ffn, (size_t)m->ffn,
+                            (size_t)m->heads * m->pf_chunks * (m->hd + 2)};
+    for (int i = 0; i < 11; ++i) {
+        if (hipMalloc(&m->pf[i], per[i] * tokens * sizeof(float)) != hipSuccess) {
+            (void)hipGetLastError();
+            for (float *&b : m->pf) {
+                if (b) (void)hipFree(b);
+                b = nullptr;
+            }
+            return fail(JITNN_HIP_ENOMEM, "allocating the buffers of a %d-token prefill failed", tokens);
+        }
+    }
+    m->pf_cap = tokens;
+    return JITNN_HIP_OK;
+}
+
+template <int D>
+int launch_attention_rows(const jitnn_hip_llama *m, int layer, int pos0, int tokens, const float *q, float *part, float *att, hipStream_t st) {
+    const int group = m->heads / m->kv, qt = ATT_ROWS / group;
+    const int chunks = (pos0 + tokens + AttCfg<D>::CH - 1) / AttCfg<D>::CH;  // of the last token
+    const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
+    constexpr size_t lds = attn_prefill_lds_bytes<D>();
+    if (int rc = allow_lds((const void *)attn_prefill_kernel<D>, lds)) return rc;
+    hipLaunchKernelGGL(attn_prefill_kernel<D>, dim3(chunks, m->kv, (tokens + qt - 1) / qt), dim3(256), lds, st, q, m->kc + lo, m->vc + lo, part, m->heads,
+                       m->kv, pos0, tokens, m->pf_chunks, 1.0f / sqrtf((float)D));
+    hipLaunchKernelGGL(attn_merge_rows_kernel<D>, dim3(m->heads, tokens), dim3(2 * D), 0, st, part, att, m->heads, pos0, m->pf_chunks);
     return JITNN_HIP_OK;
 }
 
@@ -1037,6 +1082,8 @@ int jitnn_hip_llama_free(jitnn_hip_llama *m) {
     if (!m) return JITNN_HIP_OK;
     float *bufs[] = {m->norms, m->kc, m->vc, m->cosv, m->sinv, m->xin, m->xa, m->xb, m->xn, m->q, m->k, m->v, m->att, m->gate, m->up, m->h, m->part, m->logits};
     for (float *b : bufs)
+        if (b) (void)hipFree(b);
+    for (float *b : m->pf)
         if (b) (void)hipFree(b);
     delete[] m->w;
     delete m;
@@ -1147,6 +1194,84 @@ int jitnn_hip_llama_decode_dev(jitnn_hip_llama *m, const float *x_dev, int pos, 
     }
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0, int tokens, float *logits_dev, void *stream) {
+    if (int rc = check_model(m)) return rc;
+    if (!x_dev) return fail(JITNN_HIP_EINVAL, "input is NULL");
+    if (tokens < 1 || pos0 < 0 || pos0 > m->max_ctx - tokens)
+        return fail(JITNN_HIP_EINVAL, "%d tokens from position %d in a cache of %d", tokens, pos0, m->max_ctx);
+    if (m->d % 4 != 0) return fail(JITNN_HIP_EUNSUPPORTED, "d_model %d is not a multiple of 4", m->d);
+    if (int rc = ensure_prefill(m, tokens)) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const int d = m->d, T = tokens, qd = m->heads * m->hd;
+    float *xn = m->pf[0], *q = m->pf[1], *k = m->pf[2], *v = m->pf[3], *att = m->pf[4], *xa = m->pf[5], *xb = m->pf[6], *gate = m->pf[7],
+          *up = m->pf[8], *h = m->pf[9], *part = m->pf[10];
+    const unsigned add_blocks = (unsigned)std::min<size_t>(((size_t)T * d / 4 + 255) / 256, (size_t)g.cus * 8);
+    const float *x = x_dev;
+    for (int l = 0; l < m->layers; ++l) {
+        const jitnn_hip_weight *const *w = m->w + (size_t)l * 7;
+        const float *nw = m->norms + (size_t)l * 2 * d;
+        const size_t lo = (size_t)l * m->max_ctx * m->kv * m->hd;
+        hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(T), dim3(256), 0, st, x, nw, xn, d, m->eps);
+        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_Q], xn, T, nullptr, q, stream)) return rc;
+        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_K], xn, T, nullptr, k, stream)) return rc;
+        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_V], xn, T, nullptr, v, stream)) return rc;
+        hipLaunchKernelGGL(rope_append_rows_kernel, dim3(T), dim3(256), 0, st, q, k, v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads, m->kv, m->hd,
+                           pos0);
+        int arc;
+        switch (m->hd) {
+        case 64: arc = launch_attention_rows<64>(m, l, pos0, T, q, part, att, st); break;
+        case 128: arc = launch_attention_rows<128>(m, l, pos0, T, q, part, att, st); break;
+        case 192: arc = launch_attention_rows<192>(m, l, pos0, T, q, part, att, st); break;
+        default: arc = launch_attention_rows<256>(m, l, pos0, T, q, part, att, st); break;
+        }
+        if (arc) return arc;
+        // xa = x + Wo att, xb = xa + W2 (silu(W1 n) * (W3 n)), n = RMSNorm(xa)
+        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_O], att, T, nullptr, xn, stream)) return rc;
+        hipLaunchKernelGGL(add_rows_kernel, dim3(add_blocks), dim3(256), 0, st, reinterpret_cast<const float4 *>(x), reinterpret_cast<const float4 *>(xn),
+                           reinterpret_cast<float4 *>(xa), (size_t)T * d / 4);
+        hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(T), dim3(256), 0, st, xa, nw + d, xn, d, m->eps);
+        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_FFN_GATE], xn, T, nullptr, gate, stream)) return rc;
+        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_FFN_UP], xn, T, nullptr, up, stream)) return rc;
+        {
+            const long long count = (long long)T * m->ffn;
+            const unsigned blocks = (unsigned)std::min<long long>((count + 1023) / 1024, (long long)g.cus * 16);
+            hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, st, gate, up, h, (int)count);
+        }
+        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_FFN_DOWN], h, T, nullptr, xn, stream)) return rc;
+        hipLaunchKernelGGL(add_rows_kernel, dim3(add_blocks), dim3(256), 0, st, reinterpret_cast<const float4 *>(xa), reinterpret_cast<const float4 *>(xn),
+                           reinterpret_cast<float4 *>(xb), (size_t)T * d / 4);
+        x = xb;
+    }
+    (void)qd;
+    if (logits_dev) {  // the last token's logits
+        const jitnn_hip_weight *ws[1] = {m->w_out};
+        float *ys[1] = {logits_dev};
+        if (int rc = normed_linears(m, ws, ys, 1, x + (size_t)(T - 1) * d, m->norms + (size_t)m->layers * 2 * d, st)) return rc;
+    }
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_prefill(jitnn_hip_llama *m, const float *x_host, int pos0, int tokens, float *logits_host) {
+    if (int rc = check_model(m)) return rc;
+    if (!x_host) return fail(JITNN_HIP_EINVAL, "input is NULL");
+    if (tokens < 1) return fail(JITNN_HIP_EINVAL, "%d tokens", tokens);
+    float *x = nullptr;
+    const size_t bytes = (size_t)tokens * m->d * 4;
+    if (hipMalloc(&x, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(JITNN_HIP_ENOMEM, "allocating %zu bytes of embeddings failed", bytes);
+    }
+    int rc = JITNN_HIP_OK;
+    if (hipMemcpy(x, x_host, bytes, hipMemcpyHostToDevice) != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "copying the embeddings failed");
+    if (!rc) rc = jitnn_hip_llama_prefill_dev(m, x, pos0, tokens, logits_host ? m->logits : nullptr, nullptr);
+    if (!rc && hipDeviceSynchronize() != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "the prefill step failed: %s", hipGetErrorString(hipGetLastError()));
+    if (!rc && logits_host && hipMemcpy(logits_host, m->logits, (size_t)m->vocab * 4, hipMemcpyDeviceToHost) != hipSuccess)
+        rc = fail(JITNN_HIP_EDEVICE, "copying the logits failed");
+    (void)hipFree(x);
+    return rc;
 }
 
 int jitnn_hip_llama_decode(jitnn_hip_llama *m, const float *x_host, int pos, float *logits_host) {

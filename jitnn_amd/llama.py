@@ -82,3 +82,18 @@ class LlamaDecoder:
     def decode_dev(self, x_ptr: int, pos: int, logits_ptr: int, stream_ptr: int = 0) -> None:
         _lib.check(_lib.lib.jitnn_hip_llama_decode_dev(self._h, C.c_void_p(x_ptr), pos, C.c_void_p(logits_ptr), C.c_void_p(stream_ptr)),
                    "jitnn_hip_llama_decode_dev")
+
+    def prefill(self, x, pos0: int = 0, logits: bool = True):
+        """Runs the tokens whose embeddings are the rows of x [tokens, d_model] through the stack at positions
+        pos0 .. pos0 + tokens - 1 (causal attention over the cache and one another), appends their keys and values,
+        and returns the logits [vocab] of the last token (None when logits is False)."""
+        a = np.ascontiguousarray(x, dtype=np.float32)
+        if a.ndim != 2 or a.shape[1] != self.cfg["d_model"]:
+            raise ValueError(f"embeddings of shape {a.shape} for d_model {self.cfg['d_model']}")
+        y = np.empty(self.cfg["vocab"], dtype=np.float32) if logits else None
+        _lib.check(_lib.lib.jitnn_hip_llama_prefill(self._h, _p(a), pos0, a.shape[0], _p(y) if logits else None), "jitnn_hip_llama_prefill")
+        return y
+
+    def prefill_dev(self, x_ptr: int, pos0: int, tokens: int, logits_ptr: int = 0, stream_ptr: int = 0) -> None:
+        _lib.check(_lib.lib.jitnn_hip_llama_prefill_dev(self._h, C.c_void_p(x_ptr), pos0, tokens, C.c_void_p(logits_ptr), C.c_void_p(stream_ptr)),
+                   "jitnn_hip_llama_prefill_dev")

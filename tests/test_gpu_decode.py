@@ -106,3 +106,70 @@ def test_decode_argument_checks(jn):
     with pytest.raises(ValueError):
         jn.LlamaDecoder(**{**cfg, "head_dim": 80})
     dec.close()
+
+
+@pytest.mark.parametrize("pos0,tokens,bar", [(5, 3, 1e-4), (0, 20, 1e-4), (9, 70, 1e-2)])
+def test_prefill_matches_token_by_token_reference(jn, pos0, tokens, bar):
+    """Many tokens at once against the oracle's decode step run token by token on the same cache: the last token's
+    logits and every appended key and value.  Up to 64 tokens the linears are the FP32-grade GEMV kernels (bar 1e-4);
+    beyond, the FP16-operand matrix-core path (2e-3 per linear, two layers deep: 1e-2 on the logits)."""
+    cfg = dict(layers=2, d_model=512, heads=8, kv_heads=2, head_dim=64, ffn=1024, vocab=1000, max_ctx=96, rms_eps=1e-5, rope_theta=5e5)
+    dec, layers, out_norm, out_w = build(jn, cfg, 11)
+    rng = np.random.default_rng(3)
+    kc = np.zeros((cfg["layers"], cfg["max_ctx"], cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :pos0] = rng.standard_normal(kc[:, :pos0].shape)
+    vc[:, :pos0] = rng.standard_normal(vc[:, :pos0].shape)
+    for li in range(cfg["layers"]):
+        if pos0:
+            dec.kv_write(li, 0, kc[li, :pos0], vc[li, :pos0])
+    x = rng.standard_normal((tokens, cfg["d_model"])).astype(np.float32)
+    ref = None
+    for t in range(tokens):
+        ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x[t], pos0 + t)
+    y = dec.prefill(x, pos0)
+    assert norm_err(y, ref) <= bar, norm_err(y, ref)
+    for li in range(cfg["layers"]):
+        k, v = dec.kv_read(li, pos0, tokens)
+        assert norm_err(k, kc[li, pos0:pos0 + tokens]) <= bar and norm_err(v, vc[li, pos0:pos0 + tokens]) <= bar, li
+    # decoding goes on from the prefilled cache
+    xn = rng.standard_normal(cfg["d_model"]).astype(np.float32)
+    ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, xn, pos0 + tokens)
+    assert norm_err(dec.decode(xn, pos0 + tokens), ref) <= bar
+    dec.close()
+
+
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(4, 2, 128), (6, 2, 64), (2, 2, 192), (2, 1, 256)])
+def test_prefill_head_shapes(jn, heads, kv_heads, head_dim):
+    """Every head size the attention kernels are built for, groups of 1, 2 and 3 query heads per key/value head; 40 tokens
+    after 7 cached positions (several key chunks, the last one partly filled)."""
+    cfg = dict(layers=1, d_model=512, heads=heads, kv_heads=kv_heads, head_dim=head_dim, ffn=512, vocab=300, max_ctx=64, rms_eps=1e-5,
+               rope_theta=5e5)
+    dec, layers, out_norm, out_w = build(jn, cfg, 17, {s: "Q8_0" for s in SLOTS}, "Q8_0")
+    rng = np.random.default_rng(4)
+    pos0, tokens = 7, 40
+    kc = np.zeros((1, cfg["max_ctx"], kv_heads, head_dim), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :pos0] = rng.standard_normal(kc[:, :pos0].shape)
+    vc[:, :pos0] = rng.standard_normal(vc[:, :pos0].shape)
+    dec.kv_write(0, 0, kc[0, :pos0], vc[0, :pos0])
+    x = rng.standard_normal((tokens, cfg["d_model"])).astype(np.float32)
+    for t in range(tokens):
+        ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x[t], pos0 + t)
+    y = dec.prefill(x, pos0)
+    assert norm_err(y, ref) <= 1e-4, norm_err(y, ref)
+    k, v = dec.kv_read(0, pos0, tokens)
+    assert norm_err(k, kc[0, pos0:pos0 + tokens]) <= 1e-4 and norm_err(v, vc[0, pos0:pos0 + tokens]) <= 1e-4
+    dec.close()
+
+
+def test_prefill_argument_checks(jn):
+    cfg = dict(layers=1, d_model=256, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=64, max_ctx=8, rms_eps=1e-5, rope_theta=1e4)
+    dec, *_ = build(jn, cfg, 13, {s: "Q8_0" for s in SLOTS}, "Q8_0")
+    x = np.zeros((4, 256), dtype=np.float32)
+    with pytest.raises(ValueError):
+        dec.prefill(x, 5)  # positions 5..8 of a cache of 8
+    with pytest.raises(ValueError):
+        dec.prefill(np.zeros((4, 128), dtype=np.float32), 0)
+    assert dec.prefill(x, 4, logits=False) is None
+    dec.close()
