@@ -237,15 +237,15 @@ __global__ void __launch_bounds__(256) rope_append_rows_kernel(float *__restrict
     for (int i = threadIdx.x; i < kv_heads * D; i += 256) vc[i] = vt[i];
 }
 
-// Attention of a block of consecutive tokens over one chunk of CH keys: the (token, query head) pairs of one
-// key/value head - ATT_ROWS = 64 rows, i.e. 64 / group tokens - share the LDS copy of the chunk; row r = tq * group + h
-// sees key j when j <= pos0 + t0 + tq (causal).  q is already rotated, every key comes from the cache.
-// Register tiles instead of one LDS read per multiply-add: a thread owns 4 rows x CH/16 keys of the scores (the 16
-// threads of a DPP row hold all keys of their 4 rows, so the softmax statistics are two DPP reductions and the
-// probabilities go to the weighted value sum through LDS without a workgroup barrier) and 4 rows x D/16 values of the
-// output.  Per-chunk results go to `part` for attn_merge_rows_kernel, as in the one-token kernels.
-//   grid (chunks of the last token, kv_heads, token blocks), 256 threads, attn_prefill_lds_bytes<D>() of dynamic LDS;
-//   part [T, heads, chunks_max, D + 2].
+// Causal attention of a block of consecutive tokens: the (token, query head) pairs of one key/value head - ATT_ROWS =
+// 64 rows, i.e. 64 / group tokens - walk the keys in chunks of CH, each chunk staged once in LDS for all of them; row
+// r = tq * group + h sees key j when j <= pos0 + t0 + tq.  q is already rotated, every key comes from the cache.
+// Register tiles instead of one LDS read per multiply-add: a thread owns 4 rows x CH/16 keys of the scores and 4 rows
+// x D/16 values of the output.  The 16 threads of a DPP row hold all keys of their 4 rows and all of these rows'
+// output, so the running softmax (maximum, sum, rescaling of the output so far) stays inside the row of lanes: two DPP
+// reductions per chunk, the probabilities handed from the score tile to the value tile through LDS without a
+// workgroup barrier, no partial results in memory and no merge pass.
+//   grid (token blocks, kv_heads), 256 threads, attn_prefill_lds_bytes<D>() of dynamic LDS; out [T, heads, D].
 constexpr int ATT_ROWS = 64;
 template <int D>
 constexpr size_t attn_prefill_lds_bytes() {
@@ -253,8 +253,8 @@ constexpr size_t attn_prefill_lds_bytes() {
 }
 template <int D>
 __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restrict__ q, const float *__restrict__ kcache,
-                                                            const float *__restrict__ vcache, float *__restrict__ part, int heads, int kv_heads, int pos0,
-                                                            int T, int chunks_max, float scale) {
+                                                            const float *__restrict__ vcache, float *__restrict__ out, int heads, int kv_heads, int pos0,
+                                                            int T, float scale) {
     constexpr int CH = AttCfg<D>::CH, DQ = D / 4, KN = CH / 16, DV = D / 16, KP = D + 4, PP = ATT_ROWS + 4;
     static_assert(D % 64 == 0 && CH % 16 == 0, "tiles of 16 threads");
     extern __shared__ __align__(16) float att_smem[];
@@ -264,102 +264,108 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
     float *Pt = Vs + CH * D;          // [CH][ATT_ROWS + 4]: probabilities, key-major
     const int tid = threadIdx.x, rg = tid >> 4, kl = tid & 15;
     const int group = heads / kv_heads, QT = ATT_ROWS / group, rows = QT * group;
-    const int g = blockIdx.y, c = blockIdx.x, t0 = blockIdx.z * QT;
-    const int tl = min(t0 + QT, T) - 1;  // last token of the block
-    const int j0 = c * CH;
-    if (j0 > pos0 + tl) return;  // no key of this chunk is visible to any token of the block (uniform)
-    const int nk = min(CH, pos0 + tl + 1 - j0);
+    const int g = blockIdx.y, t0 = blockIdx.x * QT;
+    const int tl = min(t0 + QT, T) - 1;                // last token of the block
+    const int nchunks = (pos0 + tl + CH) / CH;         // chunks that hold keys up to its position
     for (int i = tid; i < ATT_ROWS * DQ; i += 256) {
         const int r = i / DQ, e = (i - r * DQ) * 4, tq = r / group, h = r - tq * group;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (r < rows && t0 + tq < T) v = *reinterpret_cast<const float4 *>(q + ((size_t)(t0 + tq) * heads + g * group + h) * D + e);
         *reinterpret_cast<float4 *>(&Qs[r * D + e]) = v;
     }
-    for (int i = tid; i < CH * DQ; i += 256) {
-        const int j = i / DQ, e = (i - j * DQ) * 4;
-        float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), vv = kk;
-        if (j < nk) {
-            const size_t row = ((size_t)(j0 + j) * kv_heads + g) * D;
-            kk = *reinterpret_cast<const float4 *>(kcache + row + e);
-            vv = *reinterpret_cast<const float4 *>(vcache + row + e);
-        }
-        *reinterpret_cast<float4 *>(&Ks[j * KP + e]) = kk;
-        *reinterpret_cast<float4 *>(&Vs[j * D + e]) = vv;
+    float mrun[4], lrun[4];
+    float4 acc[4][DV / 4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        mrun[i] = -INFINITY;
+        lrun[i] = 0.f;
+#pragma unroll
+        for (int e = 0; e < DV / 4; ++e) acc[i][e] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    __syncthreads();
-    // ---- scores of rows 4 rg .. + 3 against keys kl + 16 n
-    float sc[4][KN];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int n = 0; n < KN; ++n) sc[i][n] = 0.f;
-#pragma unroll 4
-    for (int d4 = 0; d4 < DQ; ++d4) {
-        float4 qv[4], kv[KN];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const float4 *>(&Qs[(4 * rg + i) * D + 4 * d4]);
-#pragma unroll
-        for (int n = 0; n < KN; ++n) kv[n] = *reinterpret_cast<const float4 *>(&Ks[(kl + 16 * n) * KP + 4 * d4]);
+    for (int c = 0; c < nchunks; ++c) {
+        const int j0 = c * CH, nk = min(CH, pos0 + tl + 1 - j0);
+        __syncthreads();  // the chunk before has been read (first turn: nothing to wait for but the barrier below needs its twin)
+        for (int i = tid; i < CH * DQ; i += 256) {
+            const int j = i / DQ, e = (i - j * DQ) * 4;
+            float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), vv = kk;
+            if (j < nk) {
+                const size_t row = ((size_t)(j0 + j) * kv_heads + g) * D;
+                kk = *reinterpret_cast<const float4 *>(kcache + row + e);
+                vv = *reinterpret_cast<const float4 *>(vcache + row + e);
+            }
+            *reinterpret_cast<float4 *>(&Ks[j * KP + e]) = kk;
+            *reinterpret_cast<float4 *>(&Vs[j * D + e]) = vv;
+        }
+        __syncthreads();
+        // ---- scores of rows 4 rg .. + 3 against keys kl + 16 n
+        float sc[4][KN];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int n = 0; n < KN; ++n) {
-                sc[i][n] = __builtin_fmaf(qv[i].x, kv[n].x, sc[i][n]);
-                sc[i][n] = __builtin_fmaf(qv[i].y, kv[n].y, sc[i][n]);
-                sc[i][n] = __builtin_fmaf(qv[i].z, kv[n].z, sc[i][n]);
-                sc[i][n] = __builtin_fmaf(qv[i].w, kv[n].w, sc[i][n]);
-            }
-    }
-    // ---- softmax statistics of each row over the chunk (the row's keys sit in the 16 lanes of this DPP row)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = 4 * rg + i, tq = r / group, h = r - tq * group;
-        const bool live = r < rows && t0 + tq < T;
-        float m = -INFINITY;
-#pragma unroll
-        for (int n = 0; n < KN; ++n) {
-            const bool seen = live && j0 + kl + 16 * n <= pos0 + t0 + tq;
-            sc[i][n] = seen ? sc[i][n] * scale : -INFINITY;
-            m = fmaxf(m, sc[i][n]);
-        }
-        m = row_max(m);
-        float l = 0.f;
-#pragma unroll
-        for (int n = 0; n < KN; ++n) {
-            const float p = sc[i][n] > -INFINITY ? __expf(sc[i][n] - m) : 0.f;
-            Pt[(kl + 16 * n) * PP + r] = p;
-            l += p;
-        }
-        l = row_sum(l);
-        if (kl == 0 && live) {
-            float *o = part + (((size_t)(t0 + tq) * heads + g * group + h) * chunks_max + c) * (D + 2);
-            o[D] = m;
-            o[D + 1] = l;
-        }
-    }
-    // the probabilities of rows 4 rg .. + 3 were written by the 16 lanes that read them below: a wave-level hand-off
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // ---- unnormalised weighted value sums: rows 4 rg .. + 3, values DV kl .. + DV - 1
-    float4 acc[4][DV / 4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int e = 0; e < DV / 4; ++e) acc[i][e] = make_float4(0.f, 0.f, 0.f, 0.f);
+            for (int n = 0; n < KN; ++n) sc[i][n] = 0.f;
 #pragma unroll 4
-    for (int j = 0; j < CH; ++j) {
-        const float4 p = *reinterpret_cast<const float4 *>(&Pt[j * PP + 4 * rg]);
-        const float pr[4] = {p.x, p.y, p.z, p.w};
+        for (int d4 = 0; d4 < DQ; ++d4) {
+            float4 qv[4], kv[KN];
 #pragma unroll
-        for (int e = 0; e < DV / 4; ++e) {
-            const float4 v = *reinterpret_cast<const float4 *>(&Vs[j * D + DV * kl + 4 * e]);
+            for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const float4 *>(&Qs[(4 * rg + i) * D + 4 * d4]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[i][e].x = __builtin_fmaf(pr[i], v.x, acc[i][e].x);
-                acc[i][e].y = __builtin_fmaf(pr[i], v.y, acc[i][e].y);
-                acc[i][e].z = __builtin_fmaf(pr[i], v.z, acc[i][e].z);
-                acc[i][e].w = __builtin_fmaf(pr[i], v.w, acc[i][e].w);
+            for (int n = 0; n < KN; ++n) kv[n] = *reinterpret_cast<const float4 *>(&Ks[(kl + 16 * n) * KP + 4 * d4]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int n = 0; n < KN; ++n) {
+                    sc[i][n] = __builtin_fmaf(qv[i].x, kv[n].x, sc[i][n]);
+                    sc[i][n] = __builtin_fmaf(qv[i].y, kv[n].y, sc[i][n]);
+                    sc[i][n] = __builtin_fmaf(qv[i].z, kv[n].z, sc[i][n]);
+                    sc[i][n] = __builtin_fmaf(qv[i].w, kv[n].w, sc[i][n]);
+                }
+        }
+        // ---- running softmax of each row (its keys sit in the 16 lanes of this DPP row, and so does its output)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 4 * rg + i, tq = r / group;
+            const bool live = r < rows && t0 + tq < T;
+            float mc = -INFINITY;
+#pragma unroll
+            for (int n = 0; n < KN; ++n) {
+                const bool seen = live && j0 + kl + 16 * n <= pos0 + t0 + tq;
+                sc[i][n] = seen ? sc[i][n] * scale : -INFINITY;
+                mc = fmaxf(mc, sc[i][n]);
+            }
+            const float mn = fmaxf(mrun[i], row_max(mc));
+            const float alpha = mrun[i] > -INFINITY ? __expf(mrun[i] - mn) : 0.f;  // (nothing seen so far: nothing to rescale)
+            float ls = 0.f;
+#pragma unroll
+            for (int n = 0; n < KN; ++n) {
+                const float p = sc[i][n] > -INFINITY ? __expf(sc[i][n] - mn) : 0.f;
+                Pt[(kl + 16 * n) * PP + r] = p;
+                ls += p;
+            }
+            lrun[i] = lrun[i] * alpha + row_sum(ls);
+            mrun[i] = mn;
+#pragma unroll
+            for (int e = 0; e < DV / 4; ++e)
+                acc[i][e] = make_float4(acc[i][e].x * alpha, acc[i][e].y * alpha, acc[i][e].z * alpha, acc[i][e].w * alpha);
+        }
+        // the probabilities of rows 4 rg .. + 3 were written by the 16 lanes that read them below: a wave-level hand-off
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // ---- weighted value sums: rows 4 rg .. + 3, values DV kl .. + DV - 1
+#pragma unroll 4
+        for (int j = 0; j < CH; ++j) {
+            const float4 p = *reinterpret_cast<const float4 *>(&Pt[j * PP + 4 * rg]);
+            const float pr[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+            for (int e = 0; e < DV / 4; ++e) {
+                const float4 v = *reinterpret_cast<const float4 *>(&Vs[j * D + DV * kl + 4 * e]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[i][e].x = __builtin_fmaf(pr[i], v.x, acc[i][e].x);
+                    acc[i][e].y = __builtin_fmaf(pr[i], v.y, acc[i][e].y);
+                    acc[i][e].z = __builtin_fmaf(pr[i], v.z, acc[i][e].z);
+                    acc[i][e].w = __builtin_fmaf(pr[i], v.w, acc[i][e].w);
+                }
             }
         }
     }
@@ -367,23 +373,13 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
     for (int i = 0; i < 4; ++i) {
         const int r = 4 * rg + i, tq = r / group, h = r - tq * group;
         if (r < rows && t0 + tq < T) {
-            float *o = part + (((size_t)(t0 + tq) * heads + g * group + h) * chunks_max + c) * (D + 2) + DV * kl;
+            float *o = out + ((size_t)(t0 + tq) * heads + g * group + h) * D + DV * kl;
+            const float il = 1.f / lrun[i];
 #pragma unroll
-            for (int e = 0; e < DV / 4; ++e) {  // (D + 2 floats per record: 8-byte aligned, so two 64-bit stores)
-                *reinterpret_cast<float2 *>(o + 4 * e) = make_float2(acc[i][e].x, acc[i][e].y);
-                *reinterpret_cast<float2 *>(o + 4 * e + 2) = make_float2(acc[i][e].z, acc[i][e].w);
-            }
+            for (int e = 0; e < DV / 4; ++e)
+                *reinterpret_cast<float4 *>(o + 4 * e) = make_float4(acc[i][e].x * il, acc[i][e].y * il, acc[i][e].z * il, acc[i][e].w * il);
         }
     }
-}
-
-// attn_merge_kernel per (query head, token): token t merges the chunks that hold keys up to its own position.
-template <int D>
-__global__ void __launch_bounds__(2 * D) attn_merge_rows_kernel(const float *__restrict__ part, float *__restrict__ out, int heads, int pos0,
-                                                                 int chunks_max) {
-    const int h = blockIdx.x, t = blockIdx.y;
-    const int chunks = (pos0 + t + AttCfg<D>::CH) / AttCfg<D>::CH;  // ceil((pos0 + t + 1) / CH)
-    attn_merge_body<D>(part + ((size_t)t * heads + h) * chunks_max * (D + 2), out + ((size_t)t * heads + h) * D, chunks);
 }
 
 // y = a + b, four values per thread (the residual connections of many rows)

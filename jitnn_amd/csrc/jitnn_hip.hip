@@ -912,8 +912,8 @@ struct jitnn_hip_llama {
     float *xin, *xa, *xb, *xn, *q, *k, *v, *att, *gate, *up, *h, *part, *logits;
     int chunks_max;
     // many-token (prefill) buffers, [pf_cap, ...] each, allocated by the first prefill call and grown when a longer one comes
-    int pf_cap, pf_chunks;
-    float *pf[11];  // xn, q, k, v, att, xa, xb, gate, up, h, part
+    int pf_cap;
+    float *pf[10];  // xn, q, k, v, att, xa, xb, gate, up, h
 };
 
 namespace {
@@ -986,12 +986,9 @@ int ensure_prefill(jitnn_hip_llama *m, int tokens) {
         b = nullptr;
     }
     m->pf_cap = 0;
-    const int ch = m->hd <= 128 ? 32 : 16;  // AttCfg<D>::CH
-    m->pf_chunks = (m->max_ctx + ch - 1) / ch;
     const size_t qd = (size_t)m->heads * m->hd, kd = (size_t)m->kv * m->hd;
-    const size_t per[11] = {(size_t)m->d, qd, kd, kd, qd, (size_t)m->d, (size_t)m->d, (size_t)m->ffn, (size_t)m->ffn, (size_t)m->ffn,
-                            (size_t)m->heads * m->pf_chunks * (m->hd + 2)};
-    for (int i = 0; i < 11; ++i) {
+    const size_t per[10] = {(size_t)m->d, qd, kd, kd, qd, (size_t)m->d, (size_t)m->d, (size_t)m->ffn, (size_t)m->ffn, (size_t)m->ffn};
+    for (int i = 0; i < 10; ++i) {
         if (hipMalloc(&m->pf[i], per[i] * tokens * sizeof(float)) != hipSuccess) {
             (void)hipGetLastError();
             for (float *&b : m->pf) {
@@ -1006,15 +1003,13 @@ int ensure_prefill(jitnn_hip_llama *m, int tokens) {
 }
 
 template <int D>
-int launch_attention_rows(const jitnn_hip_llama *m, int layer, int pos0, int tokens, const float *q, float *part, float *att, hipStream_t st) {
+int launch_attention_rows(const jitnn_hip_llama *m, int layer, int pos0, int tokens, const float *q, float *att, hipStream_t st) {
     const int group = m->heads / m->kv, qt = ATT_ROWS / group;
-    const int chunks = (pos0 + tokens + AttCfg<D>::CH - 1) / AttCfg<D>::CH;  // of the last token
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
     constexpr size_t lds = attn_prefill_lds_bytes<D>();
     if (int rc = allow_lds((const void *)attn_prefill_kernel<D>, lds)) return rc;
-    hipLaunchKernelGGL(attn_prefill_kernel<D>, dim3(chunks, m->kv, (tokens + qt - 1) / qt), dim3(256), lds, st, q, m->kc + lo, m->vc + lo, part, m->heads,
-                       m->kv, pos0, tokens, m->pf_chunks, 1.0f / sqrtf((float)D));
-    hipLaunchKernelGGL(attn_merge_rows_kernel<D>, dim3(m->heads, tokens), dim3(2 * D), 0, st, part, att, m->heads, pos0, m->pf_chunks);
+    hipLaunchKernelGGL(attn_prefill_kernel<D>, dim3((tokens + qt - 1) / qt, m->kv), dim3(256), lds, st, q, m->kc + lo, m->vc + lo, att, m->heads, m->kv,
+                       pos0, tokens, 1.0f / sqrtf((float)D));
     return JITNN_HIP_OK;
 }
 
@@ -1206,7 +1201,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
     hipStream_t st = (hipStream_t)stream;
     const int d = m->d, T = tokens, qd = m->heads * m->hd;
     float *xn = m->pf[0], *q = m->pf[1], *k = m->pf[2], *v = m->pf[3], *att = m->pf[4], *xa = m->pf[5], *xb = m->pf[6], *gate = m->pf[7],
-          *up = m->pf[8], *h = m->pf[9], *part = m->pf[10];
+          *up = m->pf[8], *h = m->pf[9];
     const unsigned add_blocks = (unsigned)std::min<size_t>(((size_t)T * d / 4 + 255) / 256, (size_t)g.cus * 8);
     const float *x = x_dev;
     for (int l = 0; l < m->layers; ++l) {
@@ -1221,10 +1216,10 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
                            pos0);
         int arc;
         switch (m->hd) {
-        case 64: arc = launch_attention_rows<64>(m, l, pos0, T, q, part, att, st); break;
-        case 128: arc = launch_attention_rows<128>(m, l, pos0, T, q, part, att, st); break;
-        case 192: arc = launch_attention_rows<192>(m, l, pos0, T, q, part, att, st); break;
-        default: arc = launch_attention_rows<256>(m, l, pos0, T, q, part, att, st); break;
+        case 64: arc = launch_attention_rows<64>(m, l, pos0, T, q, att, st); break;
+        case 128: arc = launch_attention_rows<128>(m, l, pos0, T, q, att, st); break;
+        case 192: arc = launch_attention_rows<192>(m, l, pos0, T, q, att, st); break;
+        default: arc = launch_attention_rows<256>(m, l, pos0, T, q, att, st); break;
         }
         if (arc) return arc;
         // xa = x + Wo att, xb = xa + W2 (silu(W1 n) * (W3 n)), n = RMSNorm(xa)
