@@ -237,16 +237,17 @@ __global__ void __launch_bounds__(256) rope_append_rows_kernel(float *__restrict
     for (int i = threadIdx.x; i < kv_heads * D; i += 256) vc[i] = vt[i];
 }
 
-// Causal attention of a block of consecutive tokens: the (token, query head) pairs of one key/value head - ATT_ROWS =
-// 64 rows, i.e. 64 / group tokens - walk the keys in chunks of CH, each chunk staged once in LDS for all of them; row
+// Causal attention of a block of consecutive tokens: the (token, query head) pairs of one key/value head - ATT_ROWS
+// rows, i.e. ATT_ROWS / group tokens - walk the keys in chunks of CH, each chunk staged once in LDS for all of them; row
 // r = tq * group + h sees key j when j <= pos0 + t0 + tq.  q is already rotated, every key comes from the cache.
-// Register tiles instead of one LDS read per multiply-add: a thread owns 4 rows x CH/16 keys of the scores and 4 rows
-// x D/16 values of the output.  The 16 threads of a DPP row hold all keys of their 4 rows and all of these rows'
+// Register tiles instead of one LDS read per multiply-add: a thread owns ATT_RT rows x CH/16 keys of the scores and ATT_RT rows
+// x D/16 values of the output.  The 16 threads of a DPP row hold all keys of their rows and all of these rows'
 // output, so the running softmax (maximum, sum, rescaling of the output so far) stays inside the row of lanes: two DPP
 // reductions per chunk, the probabilities handed from the score tile to the value tile through LDS without a
 // workgroup barrier, no partial results in memory and no merge pass.
 //   grid (token blocks, kv_heads), 256 threads, attn_prefill_lds_bytes<D>() of dynamic LDS; out [T, heads, D].
-constexpr int ATT_ROWS = 64;
+constexpr int ATT_ROWS = 32;  // 16 row groups of ATT_RT rows
+constexpr int ATT_RT = ATT_ROWS / 16;
 template <int D>
 constexpr size_t attn_prefill_lds_bytes() {
     return sizeof(float) * ((size_t)ATT_ROWS * D + (size_t)AttCfg<D>::CH * (D + 4) + (size_t)AttCfg<D>::CH * D + (size_t)AttCfg<D>::CH * (ATT_ROWS + 4));
@@ -264,7 +265,11 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
     float *Pt = Vs + CH * D;          // [CH][ATT_ROWS + 4]: probabilities, key-major
     const int tid = threadIdx.x, rg = tid >> 4, kl = tid & 15;
     const int group = heads / kv_heads, QT = ATT_ROWS / group, rows = QT * group;
-    const int g = blockIdx.y, t0 = blockIdx.x * QT;
+    const int g = blockIdx.y;
+    // two workgroups share a CU and the early token blocks have few keys to walk: the upper half of the key/value heads
+    // takes the blocks in reverse, so that the pair a CU is likely to hold has one long and one short walk
+    const int tb = 2 * (int)blockIdx.y < kv_heads ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int t0 = tb * QT;
     const int tl = min(t0 + QT, T) - 1;                // last token of the block
     const int nchunks = (pos0 + tl + CH) / CH;         // chunks that hold keys up to its position
     for (int i = tid; i < ATT_ROWS * DQ; i += 256) {
@@ -273,10 +278,10 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
         if (r < rows && t0 + tq < T) v = *reinterpret_cast<const float4 *>(q + ((size_t)(t0 + tq) * heads + g * group + h) * D + e);
         *reinterpret_cast<float4 *>(&Qs[r * D + e]) = v;
     }
-    float mrun[4], lrun[4];
-    float4 acc[4][DV / 4];
+    float mrun[ATT_RT], lrun[ATT_RT];
+    float4 acc[ATT_RT][DV / 4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < ATT_RT; ++i) {
         mrun[i] = -INFINITY;
         lrun[i] = 0.f;
 #pragma unroll
@@ -284,7 +289,8 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
     }
     for (int c = 0; c < nchunks; ++c) {
         const int j0 = c * CH, nk = min(CH, pos0 + tl + 1 - j0);
-        __syncthreads();  // the chunk before has been read (first turn: nothing to wait for but the barrier below needs its twin)
+        __syncthreads();  // the chunk before has been read (first turn: the barrier below needs its twin)
+        // (requesting the chunk one turn ahead into registers was tried: slower, it costs the second workgroup of the CU)
         for (int i = tid; i < CH * DQ; i += 256) {
             const int j = i / DQ, e = (i - j * DQ) * 4;
             float4 kk = make_float4(0.f, 0.f, 0.f, 0.f), vv = kk;
@@ -297,21 +303,21 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
             *reinterpret_cast<float4 *>(&Vs[j * D + e]) = vv;
         }
         __syncthreads();
-        // ---- scores of rows 4 rg .. + 3 against keys kl + 16 n
-        float sc[4][KN];
+        // ---- scores of rows ATT_RT rg .. against keys kl + 16 n
+        float sc[ATT_RT][KN];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < ATT_RT; ++i)
 #pragma unroll
             for (int n = 0; n < KN; ++n) sc[i][n] = 0.f;
 #pragma unroll 4
         for (int d4 = 0; d4 < DQ; ++d4) {
-            float4 qv[4], kv[KN];
+            float4 qv[ATT_RT], kv[KN];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) qv[i] = *reinterpret_cast<const float4 *>(&Qs[(4 * rg + i) * D + 4 * d4]);
+            for (int i = 0; i < ATT_RT; ++i) qv[i] = *reinterpret_cast<const float4 *>(&Qs[(ATT_RT * rg + i) * D + 4 * d4]);
 #pragma unroll
             for (int n = 0; n < KN; ++n) kv[n] = *reinterpret_cast<const float4 *>(&Ks[(kl + 16 * n) * KP + 4 * d4]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < ATT_RT; ++i)
 #pragma unroll
                 for (int n = 0; n < KN; ++n) {
                     sc[i][n] = __builtin_fmaf(qv[i].x, kv[n].x, sc[i][n]);
@@ -322,8 +328,8 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
         }
         // ---- running softmax of each row (its keys sit in the 16 lanes of this DPP row, and so does its output)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = 4 * rg + i, tq = r / group;
+        for (int i = 0; i < ATT_RT; ++i) {
+            const int r = ATT_RT * rg + i, tq = r / group;
             const bool live = r < rows && t0 + tq < T;
             float mc = -INFINITY;
 #pragma unroll
@@ -347,20 +353,21 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
             for (int e = 0; e < DV / 4; ++e)
                 acc[i][e] = make_float4(acc[i][e].x * alpha, acc[i][e].y * alpha, acc[i][e].z * alpha, acc[i][e].w * alpha);
         }
-        // the probabilities of rows 4 rg .. + 3 were written by the 16 lanes that read them below: a wave-level hand-off
+        // the probabilities of this row group were written by the 16 lanes that read them below: a wave-level hand-off
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        // ---- weighted value sums: rows 4 rg .. + 3, values DV kl .. + DV - 1
+        // ---- weighted value sums: rows ATT_RT rg .., values DV kl .. + DV - 1
 #pragma unroll 4
         for (int j = 0; j < CH; ++j) {
-            const float4 p = *reinterpret_cast<const float4 *>(&Pt[j * PP + 4 * rg]);
-            const float pr[4] = {p.x, p.y, p.z, p.w};
+            float pr[ATT_RT];
+#pragma unroll
+            for (int i = 0; i < ATT_RT; ++i) pr[i] = Pt[j * PP + ATT_RT * rg + i];
 #pragma unroll
             for (int e = 0; e < DV / 4; ++e) {
                 const float4 v = *reinterpret_cast<const float4 *>(&Vs[j * D + DV * kl + 4 * e]);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
+                for (int i = 0; i < ATT_RT; ++i) {
                     acc[i][e].x = __builtin_fmaf(pr[i], v.x, acc[i][e].x);
                     acc[i][e].y = __builtin_fmaf(pr[i], v.y, acc[i][e].y);
                     acc[i][e].z = __builtin_fmaf(pr[i], v.z, acc[i][e].z);
@@ -370,8 +377,8 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
         }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = 4 * rg + i, tq = r / group, h = r - tq * group;
+    for (int i = 0; i < ATT_RT; ++i) {
+        const int r = ATT_RT * rg + i, tq = r / group, h = r - tq * group;
         if (r < rows && t0 + tq < T) {
             float *o = out + ((size_t)(t0 + tq) * heads + g * group + h) * D + DV * kl;
             const float il = 1.f / lrun[i];
