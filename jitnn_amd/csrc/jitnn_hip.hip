@@ -447,46 +447,73 @@ int workspace_done(hipStream_t stream) {
     return JITNN_HIP_OK;
 }
 
-// more rows than the GEMV kernels take: FP16 activations in operand order + dequantise-to-LDS MFMA kernel
-int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+// More rows than the GEMV kernels take: FP16 activations in operand order + dequantise-to-LDS MFMA kernel.
+// `count` weights of one row length share the activations x [rows, k] (prepared once): ys[i] = x ws[i]^T (+ bias, one
+// weight only).  norm_w != nullptr: the RMSNorm in front of the linears is fused into the preparation (rows of at most
+// XP_MAXK values; the caller checks with prefill_prepare_fuses_norm).
+int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias,
+                         const float *norm_w, float eps, hipStream_t stream) {
     // (the kernels live in prefill_k.hip and prefill_q32.hip)
-    const bool kq = block_values(w->fmt) == 256;
-    const KernelRef kr = kq ? prefill_kernel_k(w->fmt) : prefill_kernel_q32(w->fmt);
-    if (!kr.fn) return fail(JITNN_HIP_EUNSUPPORTED, "no many-row kernel for format %d", w->fmt);
-    if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
+    struct Plan {
+        bool kq;
+        int ntiles, splits, split_steps;
+        size_t part_bytes;
+    } plan[4];
+    if (count < 1 || count > 4) return fail(JITNN_HIP_EINVAL, "%d weights on one activation", count);
+    const int k = ws[0]->k;
     const int mtiles = (rows + PF_BM - 1) / PF_BM, mblocks = mtiles * (PF_BM / 32);  // operands padded to whole tiles of tokens
-    const int ntiles = (w->n + PF_BN - 1) / PF_BN, nsteps = (w->k + PF_BK - 1) / PF_BK;
-    // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 16 steps writes its own
-    // partial y, a second kernel adds the slices in order.
-    int splits = 1;
-    if (w->n % 4 == 0) {
-        while (splits < 8 && ntiles * mtiles * splits * 2 <= g.cus && nsteps / (splits * 2) >= 16) splits *= 2;
+    const int nsteps = (k + PF_BK - 1) / PF_BK;
+    size_t part_max = 0;
+    for (int i = 0; i < count; ++i) {
+        const jitnn_hip_weight *w = ws[i];
+        if (w->k != k) return fail(JITNN_HIP_EINVAL, "weights of %d and %d values per row on one activation", k, w->k);
+        Plan &p = plan[i];
+        p.kq = block_values(w->fmt) == 256;
+        const KernelRef kr = p.kq ? prefill_kernel_k(w->fmt) : prefill_kernel_q32(w->fmt);
+        if (!kr.fn) return fail(JITNN_HIP_EUNSUPPORTED, "no many-row kernel for format %d", w->fmt);
+        if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
+        p.ntiles = (w->n + PF_BN - 1) / PF_BN;
+        // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 16 steps writes its
+        // own partial y, a second kernel adds the slices in order.
+        p.splits = 1;
+        if (w->n % 4 == 0) {
+            while (p.splits < 8 && p.ntiles * mtiles * p.splits * 2 <= g.cus && nsteps / (p.splits * 2) >= 16) p.splits *= 2;
+        }
+        // slices of the 256-value formats start on whole blocks (four steps): the kernel stages their raw bytes by block
+        p.split_steps = (nsteps + p.splits - 1) / p.splits;
+        if (p.kq) p.split_steps = (p.split_steps + 3) & ~3;
+        p.part_bytes = p.splits > 1 ? (size_t)p.splits * rows * w->n * 4 : 0;
+        if (p.part_bytes > part_max) part_max = p.part_bytes;
     }
-    // slices of the 256-value formats start on whole blocks (four steps): the kernel stages their raw bytes by block
-    int split_steps = (nsteps + splits - 1) / splits;
-    if (block_values(w->fmt) == 256) split_steps = (split_steps + 3) & ~3;
-    const size_t xo_bytes = (size_t)mblocks * pf_ksteps(w->k) * 1024;
+    const size_t xo_bytes = (size_t)mblocks * pf_ksteps(k) * 1024;
     const size_t scale_bytes = ((size_t)rows * 8 + 255) & ~(size_t)255;
-    const size_t part_bytes = splits > 1 ? (size_t)splits * rows * w->n * 4 : 0;
-    void *ws = nullptr;
-    if (int rc = workspace(xo_bytes + scale_bytes + part_bytes, stream, &ws)) return rc;
-    _Float16 *xo = (_Float16 *)ws;
-    float *scale = (float *)((uint8_t *)ws + xo_bytes), *inv = scale + rows;
-    float *part = (float *)((uint8_t *)ws + xo_bytes + scale_bytes);
-    prefill_prepare_launch(x, scale, inv, xo, rows, w->k, mblocks, stream);
-    float *out = splits > 1 ? part : y;
-    const float *b1 = splits > 1 ? nullptr : bias;
-    const dim3 grid(ntiles, mtiles, splits);
-    if (kq) prefill_launch_k(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, w->k, split_steps);
-    else prefill_launch_q32(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, w->k, split_steps);
-    if (splits > 1) {
-        const size_t count4 = (size_t)rows * w->n / 4;
-        size_t blocks = (count4 + 255) / 256;
-        if (blocks > (size_t)g.cus * 8) blocks = (size_t)g.cus * 8;
-        prefill_join_launch(part, bias, y, count4, w->n, splits, (unsigned)blocks, stream);
+    void *wsp = nullptr;
+    if (int rc = workspace(xo_bytes + scale_bytes + part_max, stream, &wsp)) return rc;
+    _Float16 *xo = (_Float16 *)wsp;
+    float *scale = (float *)((uint8_t *)wsp + xo_bytes), *inv = scale + rows;
+    float *part = (float *)((uint8_t *)wsp + xo_bytes + scale_bytes);
+    prefill_prepare_launch(x, scale, inv, xo, rows, k, mblocks, norm_w, eps, stream);
+    for (int i = 0; i < count; ++i) {
+        const jitnn_hip_weight *w = ws[i];
+        const Plan &p = plan[i];
+        float *out = p.splits > 1 ? part : ys[i];
+        const float *b1 = p.splits > 1 ? nullptr : bias;
+        const dim3 grid(p.ntiles, mtiles, p.splits);
+        if (p.kq) prefill_launch_k(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, k, p.split_steps);
+        else prefill_launch_q32(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, k, p.split_steps);
+        if (p.splits > 1) {  // (the stream orders the next weight's partial sums after this join)
+            const size_t count4 = (size_t)rows * w->n / 4;
+            size_t blocks = (count4 + 255) / 256;
+            if (blocks > (size_t)g.cus * 8) blocks = (size_t)g.cus * 8;
+            prefill_join_launch(part, bias, ys[i], count4, w->n, p.splits, (unsigned)blocks, stream);
+        }
     }
     HIP_TRY(hipGetLastError());
     return workspace_done(stream);
+}
+
+int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    return launch_prefill_group(&w, &y, 1, x, rows, bias, nullptr, 0.f, stream);
 }
 
 template <int FMT>
@@ -977,6 +1004,20 @@ int check_model(const jitnn_hip_llama *m) {
     return JITNN_HIP_OK;
 }
 
+// ys[i] = RMSNorm(x) ws[i]^T for `rows` rows.  With more rows than the GEMV kernels take (and formats the many-row
+// kernels know) the norm is part of the one activation preparation the weights share; otherwise it is a kernel of its
+// own into `xn` [rows, d] and the linears take their usual route.
+int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows,
+                        const float *nw, float *xn, hipStream_t st) {
+    bool group = rows > g.gemv_max_rows && prefill_prepare_fuses_norm(m->d);
+    for (int i = 0; i < count; ++i) group = group && !is_extra_format(ws[i]->fmt);
+    if (group) return launch_prefill_group(ws, ys, count, x, rows, nullptr, nw, m->eps, st);
+    hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(256), 0, st, x, nw, xn, m->d, m->eps);
+    for (int i = 0; i < count; ++i)
+        if (int rc = jitnn_hip_linear_dev(ws[i], xn, rows, nullptr, ys[i], (void *)st)) return rc;
+    return JITNN_HIP_OK;
+}
+
 // The many-token buffers of a model, for at least `tokens` rows.
 int ensure_prefill(jitnn_hip_llama *m, int tokens) {
     if (tokens <= m->pf_cap) return JITNN_HIP_OK;
@@ -1208,10 +1249,11 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         const jitnn_hip_weight *const *w = m->w + (size_t)l * 7;
         const float *nw = m->norms + (size_t)l * 2 * d;
         const size_t lo = (size_t)l * m->max_ctx * m->kv * m->hd;
-        hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(T), dim3(256), 0, st, x, nw, xn, d, m->eps);
-        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_Q], xn, T, nullptr, q, stream)) return rc;
-        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_K], xn, T, nullptr, k, stream)) return rc;
-        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_V], xn, T, nullptr, v, stream)) return rc;
+        {
+            const jitnn_hip_weight *ws[3] = {w[JITNN_HIP_W_ATTN_Q], w[JITNN_HIP_W_ATTN_K], w[JITNN_HIP_W_ATTN_V]};
+            float *ys[3] = {q, k, v};
+            if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st)) return rc;
+        }
         hipLaunchKernelGGL(rope_append_rows_kernel, dim3(T), dim3(256), 0, st, q, k, v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads, m->kv, m->hd,
                            pos0);
         int arc;
@@ -1226,9 +1268,11 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_O], att, T, nullptr, xn, stream)) return rc;
         hipLaunchKernelGGL(add_rows_kernel, dim3(add_blocks), dim3(256), 0, st, reinterpret_cast<const float4 *>(x), reinterpret_cast<const float4 *>(xn),
                            reinterpret_cast<float4 *>(xa), (size_t)T * d / 4);
-        hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(T), dim3(256), 0, st, xa, nw + d, xn, d, m->eps);
-        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_FFN_GATE], xn, T, nullptr, gate, stream)) return rc;
-        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_FFN_UP], xn, T, nullptr, up, stream)) return rc;
+        {
+            const jitnn_hip_weight *ws[2] = {w[JITNN_HIP_W_FFN_GATE], w[JITNN_HIP_W_FFN_UP]};
+            float *ys[2] = {gate, up};
+            if (int rc = normed_linears_rows(m, ws, ys, 2, xa, T, nw + d, xn, st)) return rc;
+        }
         {
             const long long count = (long long)T * m->ffn;
             const unsigned blocks = (unsigned)std::min<long long>((count + 1023) / 1024, (long long)g.cus * 16);

@@ -90,11 +90,14 @@ static __global__ void __launch_bounds__(256) x_to_operand_kernel(const float *_
 // different XCDs, each with its own L2: the workgroup -> token map keeps the eight writers of a line on one XCD, so
 // that the line leaves its L2 whole.  grid = padded tokens (a multiple of 64); padding tokens write zeros.
 // J = 8-value pieces per thread: a row holds at most 256 J of them.
+// NORM: the row is RMS-normalised first, x <- x * nw / sqrt(mean(x^2) + eps) (ops/RowNorm.java:286-306), for callers
+// whose linear follows a norm (the layers of a model): the normalised activations exist only as these operands.
 constexpr int XP_MAXJ = 8, XP_MAXK = XP_MAXJ * 256 * 8;
-template <int J>
+template <int J, bool NORM>
 __global__ void __launch_bounds__(256) x_prepare_kernel(const float *__restrict__ x, float *__restrict__ inv_scale, _Float16 *__restrict__ xo,
-                                                         int m, int k) {
+                                                         int m, int k, const float *__restrict__ nw, float eps) {
     __shared__ float red[4];
+    __shared__ float red2[4];
     const int b = blockIdx.x, tok = (b & ~63) | ((b & 7) << 3) | ((b >> 3) & 7), t = threadIdx.x;
     const int ksteps = pf_ksteps(k), npieces = 2 * ksteps;  // 8-value pieces of a row, zero padding included
     const float *xr = x + (size_t)min(tok, m - 1) * k;
@@ -107,15 +110,43 @@ __global__ void __launch_bounds__(256) x_prepare_kernel(const float *__restrict_
         v[j][0] = src[0];
         v[j][1] = src[1];
     }
+    float4 w[NORM ? J : 1][2];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const float4 *src = reinterpret_cast<const float4 *>(nw + min(8 * (t + 256 * j), k - 8));
+            w[j][0] = src[0];
+            w[j][1] = src[1];
+        }
+    }
 #pragma unroll
     for (int j = 0; j < J; ++j) {
         const bool in = tok < m && 8 * (t + 256 * j) < k;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < 2; ++h)
             if (!in) v[j][h] = make_float4(0.f, 0.f, 0.f, 0.f);
-            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j][h].x), fabsf(v[j][h].y)), fmaxf(fabsf(v[j][h].z), fabsf(v[j][h].w))));
-        }
     }
+    if constexpr (NORM) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) ss += (v[j][h].x * v[j][h].x + v[j][h].y * v[j][h].y) + (v[j][h].z * v[j][h].z + v[j][h].w * v[j][h].w);
+        ss = wave_sum(ss);
+        if ((t & 63) == 0) red2[t >> 6] = ss;
+        __syncthreads();
+        const float is = 1.f / sqrtf(((red2[0] + red2[1]) + (red2[2] + red2[3])) / (float)k + eps);
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                v[j][h] = make_float4(v[j][h].x * is * w[j][h].x, v[j][h].y * is * w[j][h].y, v[j][h].z * is * w[j][h].z, v[j][h].w * is * w[j][h].w);
+    }
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j][h].x), fabsf(v[j][h].y)), fmaxf(fabsf(v[j][h].z), fabsf(v[j][h].w))));
     amax = wave_max(amax);
     if ((t & 63) == 0) red[t >> 6] = amax;
     __syncthreads();
