@@ -451,8 +451,10 @@ int workspace_done(hipStream_t stream) {
 // `count` weights of one row length share the activations x [rows, k] (prepared once): ys[i] = x ws[i]^T (+ bias, one
 // weight only).  norm_w != nullptr: the RMSNorm in front of the linears is fused into the preparation (rows of at most
 // XP_MAXK values; the caller checks with prefill_prepare_fuses_norm).
+// residual != nullptr (one weight only): y = residual + x w^T, added by the join of the K slices, or, for a launch that
+// does not split K, by a pass of its own over the product left in `tmp` [rows, n].
 int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias,
-                         const float *norm_w, float eps, hipStream_t stream) {
+                         const float *norm_w, float eps, hipStream_t stream, const float *residual = nullptr, float *tmp = nullptr) {
     // (the kernels live in prefill_k.hip and prefill_q32.hip)
     struct Plan {
         bool kq;
@@ -460,6 +462,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
         size_t part_bytes;
     } plan[4];
     if (count < 1 || count > 4) return fail(JITNN_HIP_EINVAL, "%d weights on one activation", count);
+    if (residual && (count != 1 || !tmp || ws[0]->n % 4 != 0)) return fail(JITNN_HIP_EINVAL, "a residual needs one weight, rows of whole quads and a buffer");
     const int k = ws[0]->k;
     const int mtiles = (rows + PF_BM - 1) / PF_BM, mblocks = mtiles * (PF_BM / 32);  // operands padded to whole tiles of tokens
     const int nsteps = (k + PF_BK - 1) / PF_BK;
@@ -496,7 +499,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     for (int i = 0; i < count; ++i) {
         const jitnn_hip_weight *w = ws[i];
         const Plan &p = plan[i];
-        float *out = p.splits > 1 ? part : ys[i];
+        float *out = p.splits > 1 ? part : residual ? tmp : ys[i];
         const float *b1 = p.splits > 1 ? nullptr : bias;
         const dim3 grid(p.ntiles, mtiles, p.splits);
         if (p.kq) prefill_launch_k(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, k, p.split_steps);
@@ -505,7 +508,12 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
             const size_t count4 = (size_t)rows * w->n / 4;
             size_t blocks = (count4 + 255) / 256;
             if (blocks > (size_t)g.cus * 8) blocks = (size_t)g.cus * 8;
-            prefill_join_launch(part, bias, ys[i], count4, w->n, p.splits, (unsigned)blocks, stream);
+            prefill_join_launch(part, bias, residual, ys[i], count4, w->n, p.splits, (unsigned)blocks, stream);
+        } else if (residual) {
+            const size_t count4 = (size_t)rows * w->n / 4;
+            const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
+            hipLaunchKernelGGL(add_rows_kernel, dim3(blocks), dim3(256), 0, stream, reinterpret_cast<const float4 *>(tmp),
+                               reinterpret_cast<const float4 *>(residual), reinterpret_cast<float4 *>(ys[i]), count4);
         }
     }
     HIP_TRY(hipGetLastError());
@@ -1018,6 +1026,19 @@ int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const 
     return JITNN_HIP_OK;
 }
 
+// y = res + x w^T for `rows` rows (tmp [rows, n] is scratch)
+int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, const float *res, float *tmp, float *y, hipStream_t st) {
+    if (rows > g.gemv_max_rows && !is_extra_format(w->fmt) && w->n % 4 == 0) {
+        return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp);
+    }
+    if (int rc = jitnn_hip_linear_dev(w, x, rows, nullptr, tmp, (void *)st)) return rc;
+    const size_t count4 = (size_t)rows * w->n / 4;
+    const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
+    hipLaunchKernelGGL(add_rows_kernel, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const float4 *>(res), reinterpret_cast<const float4 *>(tmp),
+                       reinterpret_cast<float4 *>(y), count4);
+    return JITNN_HIP_OK;
+}
+
 // The many-token buffers of a model, for at least `tokens` rows.
 int ensure_prefill(jitnn_hip_llama *m, int tokens) {
     if (tokens <= m->pf_cap) return JITNN_HIP_OK;
@@ -1243,7 +1264,6 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
     const int d = m->d, T = tokens, qd = m->heads * m->hd;
     float *xn = m->pf[0], *q = m->pf[1], *k = m->pf[2], *v = m->pf[3], *att = m->pf[4], *xa = m->pf[5], *xb = m->pf[6], *gate = m->pf[7],
           *up = m->pf[8], *h = m->pf[9];
-    const unsigned add_blocks = (unsigned)std::min<size_t>(((size_t)T * d / 4 + 255) / 256, (size_t)g.cus * 8);
     const float *x = x_dev;
     for (int l = 0; l < m->layers; ++l) {
         const jitnn_hip_weight *const *w = m->w + (size_t)l * 7;
@@ -1265,9 +1285,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         }
         if (arc) return arc;
         // xa = x + Wo att, xb = xa + W2 (silu(W1 n) * (W3 n)), n = RMSNorm(xa)
-        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_ATTN_O], att, T, nullptr, xn, stream)) return rc;
-        hipLaunchKernelGGL(add_rows_kernel, dim3(add_blocks), dim3(256), 0, st, reinterpret_cast<const float4 *>(x), reinterpret_cast<const float4 *>(xn),
-                           reinterpret_cast<float4 *>(xa), (size_t)T * d / 4);
+        if (int rc = residual_linear_rows(w[JITNN_HIP_W_ATTN_O], att, T, x, xn, xa, st)) return rc;
         {
             const jitnn_hip_weight *ws[2] = {w[JITNN_HIP_W_FFN_GATE], w[JITNN_HIP_W_FFN_UP]};
             float *ys[2] = {gate, up};
@@ -1278,9 +1296,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
             const unsigned blocks = (unsigned)std::min<long long>((count + 1023) / 1024, (long long)g.cus * 16);
             hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, st, gate, up, h, (int)count);
         }
-        if (int rc = jitnn_hip_linear_dev(w[JITNN_HIP_W_FFN_DOWN], h, T, nullptr, xn, stream)) return rc;
-        hipLaunchKernelGGL(add_rows_kernel, dim3(add_blocks), dim3(256), 0, st, reinterpret_cast<const float4 *>(xa), reinterpret_cast<const float4 *>(xn),
-                           reinterpret_cast<float4 *>(xb), (size_t)T * d / 4);
+        if (int rc = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], h, T, xa, xn, xb, st)) return rc;
         x = xb;
     }
     (void)qd;

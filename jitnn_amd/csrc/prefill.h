@@ -666,10 +666,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
 }
 
-// y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]), slices in order: the second half of a
+// y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]) (+ res[tok, row]), slices in order: the second half of a
 // split-K launch.  count4 = m * n / 4 (n is a multiple of 4 whenever the launch splits).
-static __global__ void __launch_bounds__(256) prefill_join_kernel(const float *__restrict__ part, const float *__restrict__ bias, float *__restrict__ y,
-                                                            size_t count4, int n, int splits) {
+static __global__ void __launch_bounds__(256) prefill_join_kernel(const float *__restrict__ part, const float *__restrict__ bias,
+                                                                   const float *__restrict__ res, float *__restrict__ y, size_t count4, int n, int splits) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count4; i += (size_t)gridDim.x * 256) {
         float4 a = reinterpret_cast<const float4 *>(part)[i];
         for (int z = 1; z < splits; ++z) {
@@ -681,6 +681,13 @@ static __global__ void __launch_bounds__(256) prefill_join_kernel(const float *_
         }
         if (bias) {
             const float4 b = *reinterpret_cast<const float4 *>(bias + (i * 4) % (size_t)n);
+            a.x += b.x;
+            a.y += b.y;
+            a.z += b.z;
+            a.w += b.w;
+        }
+        if (res) {  // a residual [m, n] rides along (the layers of a model: y = x + W a)
+            const float4 b = reinterpret_cast<const float4 *>(res)[i];
             a.x += b.x;
             a.y += b.y;
             a.z += b.z;

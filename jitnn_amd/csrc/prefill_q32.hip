@@ -44,8 +44,9 @@ void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Flo
     }
 }
 
-void prefill_join_launch(const float *part, const float *bias, float *y, size_t count4, int n, int splits, unsigned blocks, hipStream_t s) {
-    hipLaunchKernelGGL(prefill_join_kernel, dim3(blocks), dim3(256), 0, s, part, bias, y, count4, n, splits);
+void prefill_join_launch(const float *part, const float *bias, const float *res, float *y, size_t count4, int n, int splits, unsigned blocks,
+                         hipStream_t s) {
+    hipLaunchKernelGGL(prefill_join_kernel, dim3(blocks), dim3(256), 0, s, part, bias, res, y, count4, n, splits);
 }
 
 }  // namespace jitnn

@@ -27,7 +27,8 @@ void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, con
 bool prefill_prepare_fuses_norm(int k);
 void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *norm_w, float eps,
                             hipStream_t s);
-void prefill_join_launch(const float *part, const float *bias, float *y, size_t count4, int n, int splits, unsigned blocks, hipStream_t s);
+void prefill_join_launch(const float *part, const float *bias, const float *res, float *y, size_t count4, int n, int splits, unsigned blocks,
+                         hipStream_t s);
 
 // ---- gemv_mfma.hip: gemv_mfma_kernel<fmt>
 KernelRef gemv_mfma_kernel_ref(int fmt);
