@@ -117,6 +117,22 @@ JITNN_HIP_API int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x
 JITNN_HIP_API int jitnn_hip_quantize_q8_0(const float *x_host, long long numel, void *blocks_host);
 JITNN_HIP_API int jitnn_hip_quantize_q8_0_dev(const float *x_dev, long long numel, void *blocks_dev, void *stream);
 
+/* ---- counters ------------------------------------------------------------------------------------ */
+
+/* Calls and tensor bytes per operator since the library was loaded (or since jitnn_hip_stats_reset), counted the way
+ * the reference's telemetry counts an operator's traffic (engine/Telemetry.java:222-240, tensorBytes): every input and
+ * output tensor once, block-quantised tensors at numel / blockValues * blockBytes - the same "algorithmic bytes" the
+ * benchmark divides by time.  Operators: "linear_gemv" (up to 64 rows), "linear_mfma" (more rows), "dequantize",
+ * "quantize_q8_0", "llama_decode", "llama_prefill" (the two model steps count their own linears under themselves, not
+ * under the linear operators).  Writes up to cap entries and returns the number of operators; thread-safe. */
+typedef struct jitnn_hip_stat {
+    char name[32];
+    long long calls;
+    long long tensor_bytes;
+} jitnn_hip_stat;
+JITNN_HIP_API int jitnn_hip_stats(jitnn_hip_stat *out, int cap);
+JITNN_HIP_API int jitnn_hip_stats_reset(void);
+
 /* ---- measurement aid ---------------------------------------------------------------------------- */
 
 /* Streams nbytes of device memory through 128-bit loads and nothing else (the result is discarded): what the

@@ -4,7 +4,7 @@ The arithmetic lives in libjitnn_hip.so (C ABI: include/jitnn_hip.h); this packa
 mirror of the reference's Tensor / Gguf / Quant / F interface for that path, used by the tests and the
 benchmark.  Importing it requires the built library.
 """
-from ._lib import JitnnError, device_info, init  # noqa: F401
+from ._lib import JitnnError, device_info, init, stats, stats_reset  # noqa: F401
 from .dtype import DType  # noqa: F401
 from .ops import F, Gguf, Quant  # noqa: F401
 from .tensor import Tensor  # noqa: F401

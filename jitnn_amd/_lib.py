@@ -32,6 +32,8 @@ def _bind() -> C.CDLL:
         "jitnn_hip_device_info": (i, [C.c_char_p, i, C.POINTER(i), C.POINTER(ll)]),
         "jitnn_hip_last_error": (C.c_char_p, []),
         "jitnn_hip_sync": (i, []),
+        "jitnn_hip_stats": (i, [vp, i]),
+        "jitnn_hip_stats_reset": (i, []),
         "jitnn_hip_block_values": (i, [i]),
         "jitnn_hip_block_bytes": (i, [i]),
         "jitnn_hip_weight_nbytes": (ll, [i, ll, ll]),
@@ -112,3 +114,20 @@ def device_info() -> dict:
     cus, hbm = C.c_int(), C.c_longlong()
     check(lib.jitnn_hip_device_info(name, 256, C.byref(cus), C.byref(hbm)), "jitnn_hip_device_info")
     return {"name": name.value.decode(), "compute_units": cus.value, "hbm_bytes": hbm.value}
+
+
+class _Stat(C.Structure):
+    _fields_ = [("name", C.c_char * 32), ("calls", C.c_longlong), ("tensor_bytes", C.c_longlong)]
+
+
+def stats() -> dict:
+    """Calls and tensor bytes per operator since the library was loaded or stats_reset(): {name: (calls, bytes)}, bytes
+    counted as the reference's telemetry counts them (engine/Telemetry.java:222-240)."""
+    n = lib.jitnn_hip_stats(None, 0)
+    buf = (_Stat * n)()
+    lib.jitnn_hip_stats(C.cast(buf, C.c_void_p), n)
+    return {e.name.decode(): (e.calls, e.tensor_bytes) for e in buf}
+
+
+def stats_reset() -> None:
+    check(lib.jitnn_hip_stats_reset(), "jitnn_hip_stats_reset")

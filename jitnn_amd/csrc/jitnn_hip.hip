@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -94,6 +95,21 @@ __global__ void __launch_bounds__(256) probe_read_kernel(const u32x4 *__restrict
     for (; i < n16; i += stride) acc ^= p[i];
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) *sink = acc.x;
 }
+
+// ---- counters (jitnn_hip_stats): calls and tensor bytes per operator, the reference's telemetry convention
+enum StatOp { ST_GEMV, ST_MFMA, ST_DEQUANT, ST_QUANT, ST_DECODE, ST_PREFILL, ST_COUNT };
+const char *const kStatNames[ST_COUNT] = {"linear_gemv", "linear_mfma", "dequantize", "quantize_q8_0", "llama_decode", "llama_prefill"};
+std::atomic<long long> g_stat_calls[ST_COUNT], g_stat_bytes[ST_COUNT];
+thread_local int g_stat_nested = 0;  // inside a model step: its linears are the step's own traffic
+void count_op(StatOp op, long long bytes) {
+    if (g_stat_nested) return;
+    g_stat_calls[op].fetch_add(1, std::memory_order_relaxed);
+    g_stat_bytes[op].fetch_add(bytes, std::memory_order_relaxed);
+}
+struct StatNest {
+    StatNest() { ++g_stat_nested; }
+    ~StatNest() { --g_stat_nested; }
+};
 
 bool known(int fmt) { return block_values(fmt) != 0; }
 
@@ -636,6 +652,24 @@ int jitnn_hip_sync(void) {
     return JITNN_HIP_OK;
 }
 
+int jitnn_hip_stats(jitnn_hip_stat *out, int cap) {
+    if (cap > 0 && !out) return fail(JITNN_HIP_EINVAL, "output is NULL");
+    for (int i = 0; i < ST_COUNT && i < cap; ++i) {
+        std::snprintf(out[i].name, sizeof(out[i].name), "%s", kStatNames[i]);
+        out[i].calls = g_stat_calls[i].load(std::memory_order_relaxed);
+        out[i].tensor_bytes = g_stat_bytes[i].load(std::memory_order_relaxed);
+    }
+    return ST_COUNT;
+}
+
+int jitnn_hip_stats_reset(void) {
+    for (int i = 0; i < ST_COUNT; ++i) {
+        g_stat_calls[i].store(0, std::memory_order_relaxed);
+        g_stat_bytes[i].store(0, std::memory_order_relaxed);
+    }
+    return JITNN_HIP_OK;
+}
+
 int jitnn_hip_weight_upload(int fmt, const void *blocks_host, long long nbytes, int n, int k, jitnn_hip_weight **out) {
     if (int rc = check_weight_args(fmt, nbytes, n, k, blocks_host, out)) return rc;
     if (int rc = check_ready()) return rc;
@@ -689,6 +723,7 @@ int jitnn_hip_dequantize_dev(const jitnn_hip_weight *w, float *y_dev, void *stre
     if (!w || !y_dev) return fail(JITNN_HIP_EINVAL, "weight or output is NULL");
     if (int rc = check_ready()) return rc;
     hipStream_t s = (hipStream_t)stream;
+    count_op(ST_DEQUANT, (long long)w->nbytes + 4ll * w->n * w->k);
     switch (w->fmt) {
     case F_Q4_0: launch_dequant<F_Q4_0>(w, y_dev, s); break;
     case F_Q4_1: launch_dequant<F_Q4_1>(w, y_dev, s); break;
@@ -726,7 +761,9 @@ int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows
     if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
     if (int rc = check_ready()) return rc;
     hipStream_t s = (hipStream_t)stream;
-    if (rows > g.gemv_max_rows && !is_extra_format(w->fmt)) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s);
+    const bool many = rows > g.gemv_max_rows && !is_extra_format(w->fmt);
+    count_op(many ? ST_MFMA : ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n) + (bias_dev ? 4ll * w->n : 0));
+    if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s);
     for (int r0 = 0; r0 < rows; r0 += 8) {
         const int nb = rows - r0 < 8 ? rows - r0 : 8;
         if (int rc = launch_gemv(w, x_dev + (size_t)r0 * w->k, nb, bias_dev, y_dev + (size_t)r0 * w->n, s)) return rc;
@@ -762,6 +799,7 @@ int jitnn_hip_quantize_q8_0_dev(const float *x_dev, long long numel, void *block
     if (numel < 0 || numel % 32 != 0) return fail(JITNN_HIP_EINVAL, "Q8_0 needs a multiple of 32 values, got %lld", numel);
     if (int rc = check_ready()) return rc;
     if (numel == 0) return JITNN_HIP_OK;
+    count_op(ST_QUANT, 4ll * numel + numel / 32 * 34);
     const size_t blocks = (size_t)numel / 32;
     size_t grid = (blocks + 255) / 256;
     if (grid > (size_t)g.cus * 16) grid = (size_t)g.cus * 16;
@@ -1012,6 +1050,13 @@ int check_model(const jitnn_hip_llama *m) {
     return JITNN_HIP_OK;
 }
 
+// bytes of every weight a step of the model reads (norm vectors included)
+long long model_weight_bytes(const jitnn_hip_llama *m) {
+    long long b = m->w_out->nbytes + 4ll * (2 * m->layers + 1) * m->d;
+    for (int i = 0; i < m->layers * 7; ++i) b += m->w[i]->nbytes;
+    return b;
+}
+
 // ys[i] = RMSNorm(x) ws[i]^T for `rows` rows.  With more rows than the GEMV kernels take (and formats the many-row
 // kernels know) the norm is part of the one activation preparation the weights share; otherwise it is a kernel of its
 // own into `xn` [rows, d] and the linears take their usual route.
@@ -1205,6 +1250,8 @@ int jitnn_hip_llama_decode_dev(jitnn_hip_llama *m, const float *x_dev, int pos, 
     if (pos < 0 || pos >= m->max_ctx) return fail(JITNN_HIP_EINVAL, "position %d of a cache of %d", pos, m->max_ctx);
     hipStream_t st = (hipStream_t)stream;
     const int d = m->d;
+    count_op(ST_DECODE, model_weight_bytes(m) + 4ll * m->layers * 2 * (pos + 1) * m->kv * m->hd + 4ll * (d + m->vocab));
+    StatNest nest;
     // residual stream: layer input x (the caller's buffer for layer 0, xb afterwards) -> xa after attention -> xb after the FFN
     const float *x = x_dev;
     for (int l = 0; l < m->layers; ++l) {
@@ -1261,6 +1308,8 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
     if (m->d % 4 != 0) return fail(JITNN_HIP_EUNSUPPORTED, "d_model %d is not a multiple of 4", m->d);
     if (int rc = ensure_prefill(m, tokens)) return rc;
     hipStream_t st = (hipStream_t)stream;
+    count_op(ST_PREFILL, model_weight_bytes(m) + 4ll * m->layers * 2 * (pos0 + tokens) * m->kv * m->hd + 4ll * ((long long)tokens * m->d + (logits_dev ? m->vocab : 0)));
+    StatNest nest;
     const int d = m->d, T = tokens, qd = m->heads * m->hd;
     float *xn = m->pf[0], *q = m->pf[1], *k = m->pf[2], *v = m->pf[3], *att = m->pf[4], *xa = m->pf[5], *xb = m->pf[6], *gate = m->pf[7],
           *up = m->pf[8], *h = m->pf[9];

@@ -106,3 +106,12 @@ def test_host_mirror_rejects_misuse_before_native_calls():
         Gguf.dequantize(x)
     with pytest.raises(ValueError):
         Quant.dequantize(x)
+
+
+def test_counters_list_the_operators():
+    """jitnn_hip_stats needs no device: six operators, nothing counted before a call succeeds."""
+    import jitnn_amd
+    jitnn_amd.stats_reset()
+    st = jitnn_amd.stats()
+    assert list(st) == ["linear_gemv", "linear_mfma", "dequantize", "quantize_q8_0", "llama_decode", "llama_prefill"]
+    assert all(v == (0, 0) for v in st.values())

@@ -290,3 +290,22 @@ def test_extra_format_dequant_and_linear_vs_oracle(jn, fmt):
         y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias) if rows % 2 else None).numpy()
         assert y.shape == (rows, n)
         assert norm_err(y, ref) <= GEMV_BAR, (fmt, rows, norm_err(y, ref))
+
+
+def test_counters_follow_the_reference_byte_convention(jn):
+    """Telemetry.tensorBytes (engine/Telemetry.java:222-240): every input and output tensor once, block tensors at
+    numel / blockValues * blockBytes."""
+    rng = np.random.default_rng(8)
+    n, k = 96, 512
+    raw = random_valid_blocks(rng, "Q4_K", n, k)
+    w = weight(jn, "Q4_K", raw, n, k)
+    jn.stats_reset()
+    jn.Gguf.linear(jn.Tensor.of(rng.standard_normal((3, k)).astype(np.float32)), w, jn.Tensor.of(np.zeros(n, dtype=np.float32)))
+    jn.Gguf.linear(jn.Tensor.of(rng.standard_normal((70, k)).astype(np.float32)), w, None)
+    jn.Gguf.dequantize(w)
+    st = jn.stats()
+    wb = n * k // 256 * 144
+    assert st["linear_gemv"] == (1, wb + 4 * 3 * (k + n) + 4 * n)
+    assert st["linear_mfma"] == (1, wb + 4 * 70 * (k + n))
+    assert st["dequantize"] == (1, wb + 4 * n * k)
+    assert st["llama_decode"] == (0, 0)
