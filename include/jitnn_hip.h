@@ -120,7 +120,7 @@ JITNN_HIP_API int jitnn_hip_quantize_q8_0_dev(const float *x_dev, long long nume
 /* ---- counters ------------------------------------------------------------------------------------ */
 
 /* Calls and tensor bytes per operator since the library was loaded (or since jitnn_hip_stats_reset), counted the way
- * the reference's telemetry counts an operator's traffic (engine/Telemetry.java:222-240, tensorBytes): every input and
+ * the reference's telemetry counts an operator's traffic (core/engine/Telemetry.java:222-240, tensorBytes): every input and
  * output tensor once, block-quantised tensors at numel / blockValues * blockBytes - the same "algorithmic bytes" the
  * benchmark divides by time.  Operators: "linear_gemv" (up to 64 rows), "linear_mfma" (more rows), "dequantize",
  * "quantize_q8_0", "llama_decode", "llama_prefill" (the two model steps count their own linears under themselves, not

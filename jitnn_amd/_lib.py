@@ -122,7 +122,7 @@ class _Stat(C.Structure):
 
 def stats() -> dict:
     """Calls and tensor bytes per operator since the library was loaded or stats_reset(): {name: (calls, bytes)}, bytes
-    counted as the reference's telemetry counts them (engine/Telemetry.java:222-240)."""
+    counted as the reference's telemetry counts them (jitnn-core/src/main/java/ai/beestream/jitnn/engine/Telemetry.java:222-240)."""
     n = lib.jitnn_hip_stats(None, 0)
     buf = (_Stat * n)()
     lib.jitnn_hip_stats(C.cast(buf, C.c_void_p), n)

@@ -293,7 +293,7 @@ def test_extra_format_dequant_and_linear_vs_oracle(jn, fmt):
 
 
 def test_counters_follow_the_reference_byte_convention(jn):
-    """Telemetry.tensorBytes (engine/Telemetry.java:222-240): every input and output tensor once, block tensors at
+    """Telemetry.tensorBytes (jitnn-core/src/main/java/ai/beestream/jitnn/engine/Telemetry.java:222-240): every input and output tensor once, block tensors at
     numel / blockValues * blockBytes."""
     rng = np.random.default_rng(8)
     n, k = 96, 512
