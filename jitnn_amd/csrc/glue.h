@@ -389,6 +389,150 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
     }
 }
 
+// The same attention with FP16 operands for prompts beyond the GEMV range, where the linears around it run on FP16
+// operands too: q, keys, values and probabilities go to LDS as binary16 (half the LDS traffic, twice the workgroups
+// per CU), products are v_dot2_f32_f16 - two multiply-adds per instruction, FP32 accumulation - and the softmax
+// statistics stay in FP32.  Values and probabilities are stored in pairs of consecutive keys so that a pair is one
+// dot2 operand.  Same grid, same tiles and same causal rule as attn_prefill_kernel.
+typedef _Float16 att_h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 att_h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 att_h8 __attribute__((ext_vector_type(8)));
+template <int D>
+constexpr size_t attn_prefill_h_lds_bytes() {
+    return sizeof(_Float16) * ((size_t)ATT_ROWS * D + (size_t)AttCfg<D>::CH * (D + 8) + (size_t)AttCfg<D>::CH * D + (size_t)AttCfg<D>::CH * ATT_ROWS);
+}
+template <int D>
+__global__ void __launch_bounds__(256) attn_prefill_h_kernel(const float *__restrict__ q, const float *__restrict__ kcache,
+                                                              const float *__restrict__ vcache, float *__restrict__ out, int heads, int kv_heads, int pos0,
+                                                              int T, float scale) {
+    constexpr int CH = AttCfg<D>::CH, DQ = D / 4, KN = CH / 16, DV = D / 16, KP = D + 8;
+    static_assert(D % 64 == 0 && CH % 16 == 0 && ATT_RT == 2, "tiles of 16 threads, two rows each");
+    extern __shared__ __align__(16) float att_smem[];
+    _Float16 *Qh = reinterpret_cast<_Float16 *>(att_smem);  // [ATT_ROWS][D]
+    _Float16 *Kh = Qh + ATT_ROWS * D;                       // [CH][D + 8]
+    _Float16 *Vh = Kh + CH * KP;                            // [CH / 2][D][2]: the values of two consecutive keys side by side
+    _Float16 *Ph = Vh + CH * D;                             // [CH / 2][ATT_ROWS][2]: probabilities, likewise
+    const int tid = threadIdx.x, rg = tid >> 4, kl = tid & 15;
+    const int group = heads / kv_heads, QT = ATT_ROWS / group, rows = QT * group;
+    const int g = blockIdx.y;
+    const int tb = 2 * (int)blockIdx.y < kv_heads ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;  // (as in attn_prefill_kernel)
+    const int t0 = tb * QT;
+    const int tl = min(t0 + QT, T) - 1;
+    const int nchunks = (pos0 + tl + CH) / CH;
+    for (int i = tid; i < ATT_ROWS * DQ; i += 256) {
+        const int r = i / DQ, e = (i - r * DQ) * 4, tq = r / group, h = r - tq * group;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (r < rows && t0 + tq < T) v = *reinterpret_cast<const float4 *>(q + ((size_t)(t0 + tq) * heads + g * group + h) * D + e);
+        *reinterpret_cast<att_h4 *>(&Qh[r * D + e]) = att_h4{(_Float16)v.x, (_Float16)v.y, (_Float16)v.z, (_Float16)v.w};
+    }
+    float mrun[ATT_RT], lrun[ATT_RT], acc[ATT_RT][DV];
+#pragma unroll
+    for (int i = 0; i < ATT_RT; ++i) {
+        mrun[i] = -INFINITY;
+        lrun[i] = 0.f;
+#pragma unroll
+        for (int e = 0; e < DV; ++e) acc[i][e] = 0.f;
+    }
+    for (int c = 0; c < nchunks; ++c) {
+        const int j0 = c * CH, nk = min(CH, pos0 + tl + 1 - j0);
+        __syncthreads();  // the chunk before has been read
+        for (int i = tid; i < (CH / 2) * DQ; i += 256) {  // a pair of keys, four values of each
+            const int jp = i / DQ, e = (i - jp * DQ) * 4;
+            float4 k0 = make_float4(0.f, 0.f, 0.f, 0.f), k1 = k0, v0 = k0, v1 = k0;
+            const size_t row = ((size_t)(j0 + 2 * jp) * kv_heads + g) * D + e;
+            if (2 * jp < nk) {
+                k0 = *reinterpret_cast<const float4 *>(kcache + row);
+                v0 = *reinterpret_cast<const float4 *>(vcache + row);
+            }
+            if (2 * jp + 1 < nk) {
+                k1 = *reinterpret_cast<const float4 *>(kcache + row + (size_t)kv_heads * D);
+                v1 = *reinterpret_cast<const float4 *>(vcache + row + (size_t)kv_heads * D);
+            }
+            *reinterpret_cast<att_h4 *>(&Kh[(2 * jp) * KP + e]) = att_h4{(_Float16)k0.x, (_Float16)k0.y, (_Float16)k0.z, (_Float16)k0.w};
+            *reinterpret_cast<att_h4 *>(&Kh[(2 * jp + 1) * KP + e]) = att_h4{(_Float16)k1.x, (_Float16)k1.y, (_Float16)k1.z, (_Float16)k1.w};
+            *reinterpret_cast<att_h8 *>(&Vh[(jp * D + e) * 2]) = att_h8{(_Float16)v0.x, (_Float16)v1.x, (_Float16)v0.y, (_Float16)v1.y,
+                                                                     (_Float16)v0.z, (_Float16)v1.z, (_Float16)v0.w, (_Float16)v1.w};
+        }
+        __syncthreads();
+        // ---- scores of rows 2 rg, 2 rg + 1 against keys kl + 16 n: eight values of d per LDS read, four dot2 each
+        float sc[ATT_RT][KN];
+#pragma unroll
+        for (int i = 0; i < ATT_RT; ++i)
+#pragma unroll
+            for (int n = 0; n < KN; ++n) sc[i][n] = 0.f;
+#pragma unroll 4
+        for (int d8 = 0; d8 < D / 8; ++d8) {
+            att_h8 qv[ATT_RT], kv[KN];
+#pragma unroll
+            for (int i = 0; i < ATT_RT; ++i) qv[i] = *reinterpret_cast<const att_h8 *>(&Qh[(ATT_RT * rg + i) * D + 8 * d8]);
+#pragma unroll
+            for (int n = 0; n < KN; ++n) kv[n] = *reinterpret_cast<const att_h8 *>(&Kh[(kl + 16 * n) * KP + 8 * d8]);
+#pragma unroll
+            for (int i = 0; i < ATT_RT; ++i)
+#pragma unroll
+                for (int n = 0; n < KN; ++n)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        sc[i][n] = __builtin_amdgcn_fdot2(att_h2{qv[i][2 * t], qv[i][2 * t + 1]}, att_h2{kv[n][2 * t], kv[n][2 * t + 1]}, sc[i][n], false);
+        }
+        // ---- running softmax of each row, in FP32
+#pragma unroll
+        for (int i = 0; i < ATT_RT; ++i) {
+            const int r = ATT_RT * rg + i, tq = r / group;
+            const bool live = r < rows && t0 + tq < T;
+            float mc = -INFINITY;
+#pragma unroll
+            for (int n = 0; n < KN; ++n) {
+                const bool seen = live && j0 + kl + 16 * n <= pos0 + t0 + tq;
+                sc[i][n] = seen ? sc[i][n] * scale : -INFINITY;
+                mc = fmaxf(mc, sc[i][n]);
+            }
+            const float mn = fmaxf(mrun[i], row_max(mc));
+            const float alpha = mrun[i] > -INFINITY ? __expf(mrun[i] - mn) : 0.f;
+            float ls = 0.f;
+#pragma unroll
+            for (int n = 0; n < KN; ++n) {
+                const float p = sc[i][n] > -INFINITY ? __expf(sc[i][n] - mn) : 0.f;
+                const int j = kl + 16 * n;
+                Ph[((j >> 1) * ATT_ROWS + r) * 2 + (j & 1)] = (_Float16)p;
+                ls += p;
+            }
+            lrun[i] = lrun[i] * alpha + row_sum(ls);
+            mrun[i] = mn;
+#pragma unroll
+            for (int e = 0; e < DV; ++e) acc[i][e] *= alpha;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // ---- weighted value sums: rows 2 rg, 2 rg + 1, values DV kl .. + DV - 1, two keys per dot2
+#pragma unroll 4
+        for (int jp = 0; jp < CH / 2; ++jp) {
+            const att_h4 pp = *reinterpret_cast<const att_h4 *>(&Ph[(jp * ATT_ROWS + ATT_RT * rg) * 2]);  // rows 2 rg and 2 rg + 1, keys 2 jp and 2 jp + 1
+            const att_h2 pr[ATT_RT] = {att_h2{pp[0], pp[1]}, att_h2{pp[2], pp[3]}};
+#pragma unroll
+            for (int e8 = 0; e8 < DV / 4; ++e8) {
+                const att_h8 v = *reinterpret_cast<const att_h8 *>(&Vh[(jp * D + DV * kl + 4 * e8) * 2]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+#pragma unroll
+                    for (int i = 0; i < ATT_RT; ++i) acc[i][4 * e8 + t] = __builtin_amdgcn_fdot2(pr[i], att_h2{v[2 * t], v[2 * t + 1]}, acc[i][4 * e8 + t], false);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < ATT_RT; ++i) {
+        const int r = ATT_RT * rg + i, tq = r / group, h = r - tq * group;
+        if (r < rows && t0 + tq < T) {
+            float *o = out + ((size_t)(t0 + tq) * heads + g * group + h) * D + DV * kl;
+            const float il = 1.f / lrun[i];
+#pragma unroll
+            for (int e = 0; e < DV / 4; ++e)
+                *reinterpret_cast<float4 *>(o + 4 * e) = make_float4(acc[i][4 * e] * il, acc[i][4 * e + 1] * il, acc[i][4 * e + 2] * il, acc[i][4 * e + 3] * il);
+        }
+    }
+}
+
 // y = a + b, four values per thread (the residual connections of many rows)
 __global__ void __launch_bounds__(256) add_rows_kernel(const float4 *__restrict__ a, const float4 *__restrict__ b, float4 *__restrict__ y, size_t count4) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count4; i += (size_t)gridDim.x * 256) {

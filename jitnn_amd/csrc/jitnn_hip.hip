@@ -71,6 +71,7 @@ struct State {
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
     bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
+    bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
 };
 State g;
 std::mutex g_mu;
@@ -630,6 +631,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
     g.device = device_ordinal;
     g.ready = true;
     return JITNN_HIP_OK;
@@ -1113,10 +1115,18 @@ template <int D>
 int launch_attention_rows(const jitnn_hip_llama *m, int layer, int pos0, int tokens, const float *q, float *att, hipStream_t st) {
     const int group = m->heads / m->kv, qt = ATT_ROWS / group;
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
-    constexpr size_t lds = attn_prefill_lds_bytes<D>();
-    if (int rc = allow_lds((const void *)attn_prefill_kernel<D>, lds)) return rc;
-    hipLaunchKernelGGL(attn_prefill_kernel<D>, dim3((tokens + qt - 1) / qt, m->kv), dim3(256), lds, st, q, m->kc + lo, m->vc + lo, att, m->heads, m->kv,
-                       pos0, tokens, 1.0f / sqrtf((float)D));
+    const dim3 grid((tokens + qt - 1) / qt, m->kv);
+    const float scale = 1.0f / sqrtf((float)D);
+    // prompts beyond the GEMV range have FP16-operand linears on both sides of the attention: FP16 operands here too
+    if (tokens > g.gemv_max_rows && g.prefill_attn_fp16) {
+        constexpr size_t lds = attn_prefill_h_lds_bytes<D>();
+        if (int rc = allow_lds((const void *)attn_prefill_h_kernel<D>, lds)) return rc;
+        hipLaunchKernelGGL(attn_prefill_h_kernel<D>, grid, dim3(256), lds, st, q, m->kc + lo, m->vc + lo, att, m->heads, m->kv, pos0, tokens, scale);
+    } else {
+        constexpr size_t lds = attn_prefill_lds_bytes<D>();
+        if (int rc = allow_lds((const void *)attn_prefill_kernel<D>, lds)) return rc;
+        hipLaunchKernelGGL(attn_prefill_kernel<D>, grid, dim3(256), lds, st, q, m->kc + lo, m->vc + lo, att, m->heads, m->kv, pos0, tokens, scale);
+    }
     return JITNN_HIP_OK;
 }
 

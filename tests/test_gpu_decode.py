@@ -139,15 +139,17 @@ def test_prefill_matches_token_by_token_reference(jn, pos0, tokens, bar):
     dec.close()
 
 
+@pytest.mark.parametrize("tokens,bar", [(40, 1e-4), (70, 5e-3)])
 @pytest.mark.parametrize("heads,kv_heads,head_dim", [(4, 2, 128), (6, 2, 64), (2, 2, 192), (2, 1, 256)])
-def test_prefill_head_shapes(jn, heads, kv_heads, head_dim):
+def test_prefill_head_shapes(jn, heads, kv_heads, head_dim, tokens, bar):
     """Every head size the attention kernels are built for, groups of 1, 2 and 3 query heads per key/value head; 40 tokens
-    after 7 cached positions (several key chunks, the last one partly filled)."""
-    cfg = dict(layers=1, d_model=512, heads=heads, kv_heads=kv_heads, head_dim=head_dim, ffn=512, vocab=300, max_ctx=64, rms_eps=1e-5,
+    (FP32 attention, GEMV linears) and 70 tokens (FP16-operand attention and linears) after 7 cached positions: several
+    key chunks, the last one partly filled."""
+    cfg = dict(layers=1, d_model=512, heads=heads, kv_heads=kv_heads, head_dim=head_dim, ffn=512, vocab=300, max_ctx=96, rms_eps=1e-5,
                rope_theta=5e5)
     dec, layers, out_norm, out_w = build(jn, cfg, 17, {s: "Q8_0" for s in SLOTS}, "Q8_0")
     rng = np.random.default_rng(4)
-    pos0, tokens = 7, 40
+    pos0 = 7
     kc = np.zeros((1, cfg["max_ctx"], kv_heads, head_dim), dtype=np.float32)
     vc = np.zeros_like(kc)
     kc[:, :pos0] = rng.standard_normal(kc[:, :pos0].shape)
@@ -157,9 +159,9 @@ def test_prefill_head_shapes(jn, heads, kv_heads, head_dim):
     for t in range(tokens):
         ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x[t], pos0 + t)
     y = dec.prefill(x, pos0)
-    assert norm_err(y, ref) <= 1e-4, norm_err(y, ref)
+    assert norm_err(y, ref) <= bar, norm_err(y, ref)
     k, v = dec.kv_read(0, pos0, tokens)
-    assert norm_err(k, kc[0, pos0:pos0 + tokens]) <= 1e-4 and norm_err(v, vc[0, pos0:pos0 + tokens]) <= 1e-4
+    assert norm_err(k, kc[0, pos0:pos0 + tokens]) <= bar and norm_err(v, vc[0, pos0:pos0 + tokens]) <= bar
     dec.close()
 
 
