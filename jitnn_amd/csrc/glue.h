@@ -433,27 +433,43 @@ __global__ void __launch_bounds__(256) attn_prefill_h_kernel(const float *__rest
 #pragma unroll
         for (int e = 0; e < DV; ++e) acc[i][e] = 0.f;
     }
-    for (int c = 0; c < nchunks; ++c) {
+    // The keys and values of a chunk are requested one chunk ahead, into registers, so that the trip to L2 / HBM runs
+    // under the arithmetic of the chunk before (with FP16 tiles the registers are there: 53 against 71 us per layer at
+    // 512 tokens; the FP32 kernel loses its second workgroup per CU to them).  A thread takes pairs of keys, four
+    // values of each; past the chunk's last key it re-reads that key, which the causal mask hides.
+    constexpr int NIH = ((CH / 2) * DQ + 255) / 256;
+    float4 rk0[NIH], rk1[NIH], rv0[NIH], rv1[NIH];
+    auto fetch = [&](int c) {
         const int j0 = c * CH, nk = min(CH, pos0 + tl + 1 - j0);
+#pragma unroll
+        for (int it = 0; it < NIH; ++it) {
+            const int i = min(tid + it * 256, (CH / 2) * DQ - 1), jp = i / DQ, e = (i - jp * DQ) * 4;
+            const size_t r0 = ((size_t)(j0 + min(2 * jp, nk - 1)) * kv_heads + g) * D + e;
+            const size_t r1 = ((size_t)(j0 + min(2 * jp + 1, nk - 1)) * kv_heads + g) * D + e;
+            rk0[it] = *reinterpret_cast<const float4 *>(kcache + r0);
+            rv0[it] = *reinterpret_cast<const float4 *>(vcache + r0);
+            rk1[it] = *reinterpret_cast<const float4 *>(kcache + r1);
+            rv1[it] = *reinterpret_cast<const float4 *>(vcache + r1);
+        }
+    };
+    fetch(0);
+    for (int c = 0; c < nchunks; ++c) {
+        const int j0 = c * CH;
         __syncthreads();  // the chunk before has been read
-        for (int i = tid; i < (CH / 2) * DQ; i += 256) {  // a pair of keys, four values of each
-            const int jp = i / DQ, e = (i - jp * DQ) * 4;
-            float4 k0 = make_float4(0.f, 0.f, 0.f, 0.f), k1 = k0, v0 = k0, v1 = k0;
-            const size_t row = ((size_t)(j0 + 2 * jp) * kv_heads + g) * D + e;
-            if (2 * jp < nk) {
-                k0 = *reinterpret_cast<const float4 *>(kcache + row);
-                v0 = *reinterpret_cast<const float4 *>(vcache + row);
+#pragma unroll
+        for (int it = 0; it < NIH; ++it) {
+            const int i = tid + it * 256;
+            if (i < (CH / 2) * DQ) {
+                const int jp = i / DQ, e = (i - jp * DQ) * 4;
+                const float4 k0 = rk0[it], k1 = rk1[it], v0 = rv0[it], v1 = rv1[it];
+                *reinterpret_cast<att_h4 *>(&Kh[(2 * jp) * KP + e]) = att_h4{(_Float16)k0.x, (_Float16)k0.y, (_Float16)k0.z, (_Float16)k0.w};
+                *reinterpret_cast<att_h4 *>(&Kh[(2 * jp + 1) * KP + e]) = att_h4{(_Float16)k1.x, (_Float16)k1.y, (_Float16)k1.z, (_Float16)k1.w};
+                *reinterpret_cast<att_h8 *>(&Vh[(jp * D + e) * 2]) = att_h8{(_Float16)v0.x, (_Float16)v1.x, (_Float16)v0.y, (_Float16)v1.y,
+                                                                         (_Float16)v0.z, (_Float16)v1.z, (_Float16)v0.w, (_Float16)v1.w};
             }
-            if (2 * jp + 1 < nk) {
-                k1 = *reinterpret_cast<const float4 *>(kcache + row + (size_t)kv_heads * D);
-                v1 = *reinterpret_cast<const float4 *>(vcache + row + (size_t)kv_heads * D);
-            }
-            *reinterpret_cast<att_h4 *>(&Kh[(2 * jp) * KP + e]) = att_h4{(_Float16)k0.x, (_Float16)k0.y, (_Float16)k0.z, (_Float16)k0.w};
-            *reinterpret_cast<att_h4 *>(&Kh[(2 * jp + 1) * KP + e]) = att_h4{(_Float16)k1.x, (_Float16)k1.y, (_Float16)k1.z, (_Float16)k1.w};
-            *reinterpret_cast<att_h8 *>(&Vh[(jp * D + e) * 2]) = att_h8{(_Float16)v0.x, (_Float16)v1.x, (_Float16)v0.y, (_Float16)v1.y,
-                                                                     (_Float16)v0.z, (_Float16)v1.z, (_Float16)v0.w, (_Float16)v1.w};
         }
         __syncthreads();
+        if (c + 1 < nchunks) fetch(c + 1);
         // ---- scores of rows 2 rg, 2 rg + 1 against keys kl + 16 n: eight values of d per LDS read, four dot2 each
         float sc[ATT_RT][KN];
 #pragma unroll
