@@ -397,15 +397,20 @@ __global__ void __launch_bounds__(256) attn_prefill_kernel(const float *__restri
 typedef _Float16 att_h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 att_h4 __attribute__((ext_vector_type(4)));
 typedef _Float16 att_h8 __attribute__((ext_vector_type(8)));
+// (chunks of twice the keys of the FP32 kernels: the FP16 tiles leave room, and a chunk costs two barriers)
+template <int D>
+struct AttCfgH {
+    static constexpr int CH = 2 * AttCfg<D>::CH;
+};
 template <int D>
 constexpr size_t attn_prefill_h_lds_bytes() {
-    return sizeof(_Float16) * ((size_t)ATT_ROWS * D + (size_t)AttCfg<D>::CH * (D + 8) + (size_t)AttCfg<D>::CH * D + (size_t)AttCfg<D>::CH * ATT_ROWS);
+    return sizeof(_Float16) * ((size_t)ATT_ROWS * D + (size_t)AttCfgH<D>::CH * (D + 8) + (size_t)AttCfgH<D>::CH * D + (size_t)AttCfgH<D>::CH * ATT_ROWS);
 }
 template <int D>
 __global__ void __launch_bounds__(256) attn_prefill_h_kernel(const float *__restrict__ q, const float *__restrict__ kcache,
                                                               const float *__restrict__ vcache, float *__restrict__ out, int heads, int kv_heads, int pos0,
                                                               int T, float scale) {
-    constexpr int CH = AttCfg<D>::CH, DQ = D / 4, KN = CH / 16, DV = D / 16, KP = D + 8;
+    constexpr int CH = AttCfgH<D>::CH, DQ = D / 4, KN = CH / 16, DV = D / 16, KP = D + 8;
     static_assert(D % 64 == 0 && CH % 16 == 0 && ATT_RT == 2, "tiles of 16 threads, two rows each");
     extern __shared__ __align__(16) float att_smem[];
     _Float16 *Qh = reinterpret_cast<_Float16 *>(att_smem);  // [ATT_ROWS][D]
