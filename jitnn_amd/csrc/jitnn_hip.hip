@@ -71,6 +71,7 @@ struct State {
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
     bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
+    int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
     bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
 };
 State g;
@@ -493,11 +494,11 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
         if (!kr.fn) return fail(JITNN_HIP_EUNSUPPORTED, "no many-row kernel for format %d", w->fmt);
         if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
         p.ntiles = (w->n + PF_BN - 1) / PF_BN;
-        // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 16 steps writes its
+        // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 8 steps writes its
         // own partial y, a second kernel adds the slices in order.
         p.splits = 1;
         if (w->n % 4 == 0) {
-            while (p.splits < 8 && p.ntiles * mtiles * p.splits * 2 <= g.cus && nsteps / (p.splits * 2) >= 16) p.splits *= 2;
+            while (p.splits < 8 && p.ntiles * mtiles * p.splits * 2 <= g.cus && nsteps / (p.splits * 2) >= g.prefill_min_slice) p.splits *= 2;
         }
         // slices of the 256-value formats start on whole blocks (four steps): the kernel stages their raw bytes by block
         p.split_steps = (nsteps + p.splits - 1) / p.splits;
@@ -632,6 +633,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
     g.ready = true;
     return JITNN_HIP_OK;
