@@ -72,6 +72,7 @@ struct State {
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
     bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
+    bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
     bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
 };
 State g;
@@ -472,7 +473,8 @@ int workspace_done(hipStream_t stream) {
 // residual != nullptr (one weight only): y = residual + x w^T, added by the join of the K slices, or, for a launch that
 // does not split K, by a pass of its own over the product left in `tmp` [rows, n].
 int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias,
-                         const float *norm_w, float eps, hipStream_t stream, const float *residual = nullptr, float *tmp = nullptr) {
+                         const float *norm_w, float eps, hipStream_t stream, const float *residual = nullptr, float *tmp = nullptr,
+                         const float *swiglu_up = nullptr) {
     // (the kernels live in prefill_k.hip and prefill_q32.hip)
     struct Plan {
         bool kq;
@@ -513,7 +515,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     _Float16 *xo = (_Float16 *)wsp;
     float *scale = (float *)((uint8_t *)wsp + xo_bytes), *inv = scale + rows;
     float *part = (float *)((uint8_t *)wsp + xo_bytes + scale_bytes);
-    prefill_prepare_launch(x, scale, inv, xo, rows, k, mblocks, norm_w, eps, stream);
+    prefill_prepare_launch(x, scale, inv, xo, rows, k, mblocks, norm_w, eps, swiglu_up, stream);
     for (int i = 0; i < count; ++i) {
         const jitnn_hip_weight *w = ws[i];
         const Plan &p = plan[i];
@@ -633,6 +635,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
     g.ready = true;
@@ -1075,10 +1078,21 @@ int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const 
     return JITNN_HIP_OK;
 }
 
-// y = res + x w^T for `rows` rows (tmp [rows, n] is scratch)
-int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, const float *res, float *tmp, float *y, hipStream_t st) {
-    if (rows > g.gemv_max_rows && !is_extra_format(w->fmt) && w->n % 4 == 0) {
-        return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp);
+// y = res + x w^T for `rows` rows (tmp [rows, n] is scratch).  up != nullptr: the activations are silu(x) * up (the FFN's
+// gate and up projections); on the many-row path they are formed inside the activation preparation, otherwise by
+// swiglu_kernel into `h` [rows, k].
+int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, const float *res, float *tmp, float *y, hipStream_t st,
+                         const float *up = nullptr, float *h = nullptr) {
+    const bool many = rows > g.gemv_max_rows && !is_extra_format(w->fmt) && w->n % 4 == 0;
+    if (many && (!up || (g.prefill_fuse_swiglu && prefill_prepare_fuses_norm(w->k)))) {
+        return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp, up);
+    }
+    if (up) {
+        const long long count = (long long)rows * w->k;
+        const unsigned blocks = (unsigned)std::min<long long>((count + 1023) / 1024, (long long)g.cus * 16);
+        hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, st, x, up, h, (int)count);
+        x = h;
+        if (many) return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp);
     }
     if (int rc = jitnn_hip_linear_dev(w, x, rows, nullptr, tmp, (void *)st)) return rc;
     const size_t count4 = (size_t)rows * w->n / 4;
@@ -1352,12 +1366,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
             float *ys[2] = {gate, up};
             if (int rc = normed_linears_rows(m, ws, ys, 2, xa, T, nw + d, xn, st)) return rc;
         }
-        {
-            const long long count = (long long)T * m->ffn;
-            const unsigned blocks = (unsigned)std::min<long long>((count + 1023) / 1024, (long long)g.cus * 16);
-            hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, st, gate, up, h, (int)count);
-        }
-        if (int rc = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], h, T, xa, xn, xb, st)) return rc;
+        if (int rc = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], gate, T, xa, xn, xb, st, up, h)) return rc;
         x = xb;
     }
     (void)qd;

@@ -90,12 +90,16 @@ static __global__ void __launch_bounds__(256) x_to_operand_kernel(const float *_
 // different XCDs, each with its own L2: the workgroup -> token map keeps the eight writers of a line on one XCD, so
 // that the line leaves its L2 whole.  grid = padded tokens (a multiple of 64); padding tokens write zeros.
 // J = 8-value pieces per thread: a row holds at most 256 J of them.
-// NORM: the row is RMS-normalised first, x <- x * nw / sqrt(mean(x^2) + eps) (ops/RowNorm.java:286-306), for callers
-// whose linear follows a norm (the layers of a model): the normalised activations exist only as these operands.
+// MODE XP_NORM: the row is RMS-normalised first, x <- x * nw / sqrt(mean(x^2) + eps) (ops/RowNorm.java:286-306), for
+// callers whose linear follows a norm (the layers of a model): the normalised activations exist only as these operands.
+// MODE XP_SWIGLU: the row is silu(x) * nw, nw being a second [m, k] array (F.swiglu, F.java:1159-1161, in front of the
+// down projection of an FFN): the gated activations exist only as these operands.
 constexpr int XP_MAXJ = 8, XP_MAXK = XP_MAXJ * 256 * 8;
-template <int J, bool NORM>
+constexpr int XP_PLAIN = 0, XP_NORM = 1, XP_SWIGLU = 2;
+template <int J, int MODE>
 __global__ void __launch_bounds__(256) x_prepare_kernel(const float *__restrict__ x, float *__restrict__ inv_scale, _Float16 *__restrict__ xo,
                                                          int m, int k, const float *__restrict__ nw, float eps) {
+    constexpr bool NORM = MODE == XP_NORM;
     __shared__ float red[4];
     __shared__ float red2[4];
     const int b = blockIdx.x, tok = (b & ~63) | ((b & 7) << 3) | ((b >> 3) & 7), t = threadIdx.x;
@@ -110,14 +114,23 @@ __global__ void __launch_bounds__(256) x_prepare_kernel(const float *__restrict_
         v[j][0] = src[0];
         v[j][1] = src[1];
     }
-    float4 w[NORM ? J : 1][2];
-    if constexpr (NORM) {
+    float4 w[MODE != XP_PLAIN ? J : 1][2];
+    if constexpr (MODE != XP_PLAIN) {
+        const float *wr = MODE == XP_SWIGLU ? nw + (size_t)min(tok, m - 1) * k : nw;
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-            const float4 *src = reinterpret_cast<const float4 *>(nw + min(8 * (t + 256 * j), k - 8));
+            const float4 *src = reinterpret_cast<const float4 *>(wr + min(8 * (t + 256 * j), k - 8));
             w[j][0] = src[0];
             w[j][1] = src[1];
         }
+    }
+    if constexpr (MODE == XP_SWIGLU) {
+        auto sw = [](float g, float u) { return (g / (1.f + __expf(-g))) * u; };
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                v[j][h] = make_float4(sw(v[j][h].x, w[j][h].x), sw(v[j][h].y, w[j][h].y), sw(v[j][h].z, w[j][h].z), sw(v[j][h].w, w[j][h].w));
     }
 #pragma unroll
     for (int j = 0; j < J; ++j) {

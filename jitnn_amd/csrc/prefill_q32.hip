@@ -23,22 +23,23 @@ void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, con
     }
 }
 
-template <bool NORM>
+template <int MODE>
 static void prepare_one_launch(const float *x, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *nw, float eps, hipStream_t s) {
     const int pieces = pf_ksteps(k) * 2;  // per row; 256 threads take J each
-    if (pieces <= 512) hipLaunchKernelGGL((x_prepare_kernel<2, NORM>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
-    else if (pieces <= 1024) hipLaunchKernelGGL((x_prepare_kernel<4, NORM>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
-    else hipLaunchKernelGGL((x_prepare_kernel<8, NORM>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
+    if (pieces <= 512) hipLaunchKernelGGL((x_prepare_kernel<2, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
+    else if (pieces <= 1024) hipLaunchKernelGGL((x_prepare_kernel<4, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
+    else hipLaunchKernelGGL((x_prepare_kernel<8, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
 }
 
 bool prefill_prepare_fuses_norm(int k) { return k <= XP_MAXK; }
 
 void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *norm_w, float eps,
-                            hipStream_t s) {
+                            const float *swiglu_up, hipStream_t s) {
     if (k <= XP_MAXK) {
-        if (norm_w) prepare_one_launch<true>(x, inv_scale, xo, rows, k, mblocks, norm_w, eps, s);
-        else prepare_one_launch<false>(x, inv_scale, xo, rows, k, mblocks, nullptr, 0.f, s);
-    } else {  // (callers ask prefill_prepare_fuses_norm first: rows this long take no norm here)
+        if (swiglu_up) prepare_one_launch<XP_SWIGLU>(x, inv_scale, xo, rows, k, mblocks, swiglu_up, 0.f, s);
+        else if (norm_w) prepare_one_launch<XP_NORM>(x, inv_scale, xo, rows, k, mblocks, norm_w, eps, s);
+        else prepare_one_launch<XP_PLAIN>(x, inv_scale, xo, rows, k, mblocks, nullptr, 0.f, s);
+    } else {  // (callers ask prefill_prepare_fuses_norm first: rows this long take no norm or gate here)
         hipLaunchKernelGGL(x_row_scale_kernel, dim3(rows), dim3(256), 0, s, x, scale, inv_scale, k);
         hipLaunchKernelGGL(x_to_operand_kernel, dim3(mblocks, pf_ksteps(k) / 4), dim3(256), 0, s, x, scale, xo, rows, k);
     }

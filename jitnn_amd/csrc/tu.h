@@ -23,10 +23,11 @@ void prefill_launch_k(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const
 void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const _Float16 *xo, const float *inv_scale, const float *bias, float *y,
                         int m, int n, int k, int split_steps);
 // activation preparation and the join of K slices (prefill_q32.hip)
-// (norm_w != nullptr: RMSNorm with that weight and eps fused into the preparation - only where prefill_prepare_fuses_norm(k))
+// (norm_w != nullptr: RMSNorm with that weight and eps fused into the preparation; swiglu_up != nullptr: the activations
+// are silu(x) * swiglu_up, both [rows, k] - either only where prefill_prepare_fuses_norm(k))
 bool prefill_prepare_fuses_norm(int k);
 void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *norm_w, float eps,
-                            hipStream_t s);
+                            const float *swiglu_up, hipStream_t s);
 void prefill_join_launch(const float *part, const float *bias, const float *res, float *y, size_t count4, int n, int splits, unsigned blocks,
                          hipStream_t s);
 
