@@ -629,6 +629,17 @@ struct UnitPair<F_Q8_0> {
 // loads are unconditional (rows past the end re-read the last row) so that the hardware's in-order load
 // counter can be waited on exactly; only the decode and the store are skipped for rows that do not exist.
 // The first rows' loads are issued before the staging barrier, so HBM latency overlaps the staging too.
+// Wave priority by the rows a wave still has to do.  The SIMD's arbiter serves its oldest wave first: of the waves
+// that share a SIMD one runs ahead, and the others are left to finish alone at the issue rate of a single wave (about
+// half of what two reach together).  With the priority stepping down as the last rows come up (more than 8, 4, 2 rows
+// left), whoever is behind at a step is served first until it has caught up, and the waves of a SIMD finish together.
+__device__ __forceinline__ void step_priority(int left) {
+    if (left > 8) __builtin_amdgcn_s_setprio(3);
+    else if (left > 4) __builtin_amdgcn_s_setprio(2);
+    else if (left > 2) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(0);
+}
+
 constexpr int XREG_THREADS = 256;  // workgroup size of gemv_xreg_kernel (compile-time: the staging is fully unrolled)
 
 // Arguments of gemv_xreg_kernel.  Up to three matrices of the same format and row length share one launch and
@@ -644,6 +655,7 @@ struct XregArgs {
     float eps;
     int k;
     float nib;
+    int rpw;  // rows the busiest wave sees (0: no priority steps)
 };
 
 // Extra template switches:
@@ -752,6 +764,8 @@ __device__ __forceinline__ void gemv_xreg_body(const XregArgs &a, const int bid,
         for (int i = 0; i < NS; ++i) xs[s].sm[i] = sums[(s * 64 + lane) * NS + i];
     }
 
+    int left = a.rpw;  // 0: the priority stays where it is
+    step_priority(left);
     float gate = 0.f;  // DUAL: the gate row's result, held until the up row of the same index is done
     for (int base = row0; base < n; base += RSTEP * stride) {
 #pragma unroll
@@ -765,6 +779,7 @@ __device__ __forceinline__ void gemv_xreg_body(const XregArgs &a, const int bid,
                     U::template dot<1, 1, CV>(w1, uc[s], xs[s], acc, a.nib);
                 }
                 const float t = wave_sum(acc[0][0]);
+                if (!DUAL || (b & 1)) step_priority(--left);
                 if (DUAL) {
                     if ((b & 1) == 0) gate = t;
                     else if (lane == 0) a.y[0][row] = (gate / (1.f + __expf(-gate))) * t;
@@ -874,6 +889,8 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_b2_kernel(const uint8_
             for (int i = 0; i < NS; ++i) xs[s].sm[b][i] = sums[b][(s * 64 + lane) * NS + i];
         }
 
+    int left = row0 < n ? (n - row0 + stride - 1) / stride : 0;  // rows of this wave
+    step_priority(left);
     for (int base = row0; base < n; base += NB * stride) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
@@ -886,6 +903,7 @@ __global__ void __launch_bounds__(XREG_THREADS) gemv_xreg_b2_kernel(const uint8_
                     U::template dot<2, 1, CV>(w1, uc[s], xs[s], acc, nib);
                 }
                 const float t0 = wave_sum(acc[0][0]), t1 = wave_sum(acc[0][1]);
+                step_priority(--left);
                 if (lane == 0) {
                     y[row] = BIAS ? t0 + bv[b] : t0;
                     y[(size_t)n + row] = BIAS ? t1 + bv[b] : t1;

@@ -64,6 +64,7 @@ struct State {
     size_t lds_per_cu = 0;   // LDS of a compute unit
     int xreg_blocks_per_cu = 0;  // JITNN_HIP_XREG_BLOCKS: override of the workgroups per CU (0 = built-in choice)
     int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1 or 2 (0 = built-in choice)
+    bool xreg_priority = true;   // JITNN_HIP_XREG_PRIORITY=0: no wave priority steps in the register-resident kernels (A/B measurements)
     // JITNN_HIP_GEMV_MAX_ROWS: up to this many rows run the FP32 GEMV kernels (in batches of 8), more rows the FP16
     // MFMA kernel - the counterpart of jitnn.gguf.tiledRows (core/JitnnConfig.java:423-424).  64 keeps every row
     // count the reference's own tests use (1, 5, 40) on the FP32 path, whose error meets their 2e-4 / 1e-3 bars.
@@ -251,6 +252,7 @@ int launch_xreg(const XregCall &c, hipStream_t stream) {
     if (blocks > cap) blocks = cap;
     const int rows_per_wave = (n + blocks * waves - 1) / (blocks * waves);
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
+    a.rpw = g.xreg_priority ? rows_per_wave : 0;
     const int mode = c.w2 ? 3 : c.norm_w ? 2 : c.bias ? 1 : 0;
     hipLaunchKernelGGL(pick_xreg(c.w[0]->fmt, a.k % 64 == 0, mode, pf), dim3(blocks), dim3(threads), 0, stream, a);
     HIP_TRY(hipGetLastError());
@@ -288,6 +290,8 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
     if (blocks_b > (nb + waves - 1) / waves) blocks_b = (nb + waves - 1) / waves;
     const int rpw_a = (na + blocks_a * waves - 1) / (blocks_a * waves), rpw_b = (nb + blocks_b * waves - 1) / (blocks_b * waves);
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : ((rpw_a > rpw_b ? rpw_a : rpw_b) >= 16 ? 1 : 2);
+    a.rpw = g.xreg_priority ? rpw_a : 0;
+    b.rpw = g.xreg_priority ? rpw_b : 0;
     xreg2_fn fn = pf == 1 ? pick_xreg2_pf<1>(ca.w[0]->fmt, cb.w[0]->fmt) : pick_xreg2_pf<2>(ca.w[0]->fmt, cb.w[0]->fmt);
     hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(XREG_THREADS), 0, stream, a, b, blocks_a);
     HIP_TRY(hipGetLastError());
@@ -627,6 +631,7 @@ int jitnn_hip_init(int device_ordinal) {
         int v = atoi(e);
         if (v >= 1 && v <= 2) g.xreg_pf = v;
     }
+    if (const char *e = getenv("JITNN_HIP_XREG_PRIORITY")) g.xreg_priority = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_GEMV_MAX_ROWS")) {
         int v = atoi(e);
         if (v >= 1) g.gemv_max_rows = v;
