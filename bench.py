@@ -31,8 +31,8 @@ sys.path.insert(0, str(ROOT / "tests"))
 
 PEAK_HBM_GBPS = 8000.0
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc (profiles/gemv_q4_k_14336x4096_b1_pmc_traffic.txt):
-# FETCH_SIZE 16234.9 KiB x 2.0 (a 256 MiB copy kernel reads 131087 on this counter) + WRITE_SIZE 112.0 KiB x 1.0
-HEADLINE_TRAFFIC_BYTES = int((16234.9 * 2.0 + 112.0) * 1024)
+# FETCH_SIZE 16245.9 KiB x 2.0 (a 256 MiB copy kernel reads 131087 on this counter) + WRITE_SIZE 112.0 KiB x 1.0
+HEADLINE_TRAFFIC_BYTES = int((16245.9 * 2.0 + 112.0) * 1024)
 BLOCK = {"Q8_0": (8, 32, 34), "Q4_0": (2, 32, 18), "Q4_1": (3, 32, 20), "Q4_K": (12, 256, 144), "Q5_K": (13, 256, 176),
          "Q6_K": (14, 256, 210)}
 
