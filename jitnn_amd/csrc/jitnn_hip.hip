@@ -64,6 +64,8 @@ struct State {
     size_t lds_per_cu = 0;   // LDS of a compute unit
     int xreg_blocks_per_cu = 0;  // JITNN_HIP_XREG_BLOCKS: override of the workgroups per CU (0 = built-in choice)
     int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1 or 2 (0 = built-in choice)
+    bool q6k_int = true;         // JITNN_HIP_Q6K_INT=0: the Q6_K output head through the FP32 variant (A/B measurements)
+    int q6k_int_min_rows = 16;   // JITNN_HIP_Q6K_INT_MIN_ROWS: rows per wave from which Q6_K takes the integer variant (tests: 1)
     bool xreg_priority = true;   // JITNN_HIP_XREG_PRIORITY=0: no wave priority steps in the register-resident kernels (A/B measurements)
     // JITNN_HIP_GEMV_MAX_ROWS: up to this many rows run the FP32 GEMV kernels (in batches of 8), more rows the FP16
     // MFMA kernel - the counterpart of jitnn.gguf.tiledRows (core/JitnnConfig.java:423-424).  64 keeps every row
@@ -254,7 +256,15 @@ int launch_xreg(const XregCall &c, hipStream_t stream) {
     const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
     a.rpw = g.xreg_priority ? rows_per_wave : 0;
     const int mode = c.w2 ? 3 : c.norm_w ? 2 : c.bias ? 1 : 0;
-    hipLaunchKernelGGL(pick_xreg(c.w[0]->fmt, a.k % 64 == 0, mode, pf), dim3(blocks), dim3(threads), 0, stream, a);
+    xreg_fn fn = pick_xreg(c.w[0]->fmt, a.k % 64 == 0, mode, pf);
+    // Q6_K with many rows per wave (the output head): the integer variant, whose one-off cost of turning the
+    // activations into byte planes is spread over the rows
+    if (c.w[0]->fmt == F_Q6_K && g.q6k_int && rows_per_wave >= g.q6k_int_min_rows && a.k % 256 == 0) {
+        if (mode == 0) fn = pf == 1 ? gemv_xreg_kernel<Unit<F_Q6_K>, 2, 1, false, false, false> : gemv_xreg_kernel<Unit<F_Q6_K>, 2, 2, false, false, false>;
+        else if (mode == 1) fn = pf == 1 ? gemv_xreg_kernel<Unit<F_Q6_K>, 2, 1, true, false, false> : gemv_xreg_kernel<Unit<F_Q6_K>, 2, 2, true, false, false>;
+        else if (mode == 2) fn = pf == 1 ? gemv_xreg_kernel<Unit<F_Q6_K>, 2, 1, false, true, false> : gemv_xreg_kernel<Unit<F_Q6_K>, 2, 2, false, true, false>;
+    }
+    hipLaunchKernelGGL(fn, dim3(blocks), dim3(threads), 0, stream, a);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
@@ -630,6 +640,11 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_XREG_PF")) {
         int v = atoi(e);
         if (v >= 1 && v <= 2) g.xreg_pf = v;
+    }
+    if (const char *e = getenv("JITNN_HIP_Q6K_INT")) g.q6k_int = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_Q6K_INT_MIN_ROWS")) {
+        int v = atoi(e);
+        if (v >= 1) g.q6k_int_min_rows = v;
     }
     if (const char *e = getenv("JITNN_HIP_XREG_PRIORITY")) g.xreg_priority = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_GEMV_MAX_ROWS")) {

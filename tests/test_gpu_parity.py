@@ -120,6 +120,43 @@ def test_gemv_vs_oracle(jn, fmt, n, k):
         assert norm_err(y, ref) <= GEMV_BAR, (fmt, n, k, rows, norm_err(y, ref))
 
 
+@pytest.mark.parametrize("k", [256, 1024, 4096])
+def test_q6k_many_rows_integer_variant(jn, k):
+    """A Q6_K matrix tall enough that every wave sees 16 rows or more takes the integer variant of the batch-1 kernel
+    (activations as 22-bit fixed point in byte planes, v_dot4): same bar, and in fact FP32-grade error, on ordinary,
+    outlier-ridden, tiny, partly zero and unit-vector activations, with and without bias."""
+    from oracle import oracle
+    rng = np.random.default_rng(4242 + k)
+    n = 16 * 2048 + 37
+    raw = random_valid_blocks(rng, "Q6_K", n, k)
+    w = weight(jn, "Q6_K", raw, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    xs = []
+    xs.append(rng.standard_normal(k).astype(np.float32))
+    x = rng.standard_normal(k).astype(np.float32)
+    x[rng.integers(0, k, size=max(1, k // 128))] *= np.float32(1e4)   # outliers share their 64-value unit with ordinary values
+    xs.append(x)
+    xs.append((rng.standard_normal(k) * 1e-30).astype(np.float32))    # near the bottom of the FP32 range
+    x = rng.standard_normal(k).astype(np.float32)
+    x[: k // 2] = 0.0                                                  # whole units of zeros
+    x[k // 2: k // 2 + 64] *= np.float32(1e-20)
+    xs.append(x)
+    x = np.zeros(k, dtype=np.float32)
+    x[k - 3] = 1.0                                                     # a column of the dequantised matrix
+    xs.append(x)
+    for i, x in enumerate(xs):
+        b = bias if i % 2 else None
+        ref = oracle.gguf_linear(14, x[None, :], raw, b, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x[None, :]), w, jn.Tensor.of(b) if b is not None else None).numpy()
+        assert y.shape == (1, n)
+        err = norm_err(y, ref) if b is None else norm_err(y - b, ref - b)
+        assert err <= GEMV_BAR, (k, i, err)
+        assert err <= 5e-6, (k, i, err)   # what the variant actually delivers
+    col = jn.Gguf.linear(jn.Tensor.of(xs[4][None, :]), w, None).numpy()[0]
+    deq = w.to_float_array().reshape(n, k)[:, k - 3]
+    assert np.allclose(col, deq, rtol=3e-7, atol=0.0)
+
+
 @pytest.mark.parametrize("fmt", HOT_FORMATS)
 @pytest.mark.parametrize("rows", [2, 5, 7, 8])
 def test_batch_rows_of_very_different_magnitude(jn, fmt, rows):
