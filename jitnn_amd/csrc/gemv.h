@@ -41,17 +41,6 @@ __device__ __forceinline__ float dot4(float a, float b, float c, float d, const 
     return acc;
 }
 
-// The same four multiply-adds into four separate partial sums: no instruction depends on the one before it, so a
-// wave that runs alone on its SIMD (its neighbour waiting for memory) still issues every cycle.  For the variants
-// with few (row, batch) pairs, where the extra accumulators fit.
-__device__ __forceinline__ void dot4w(float a, float b, float c, float d, const float4 &x, float (&acc)[4]) {
-    acc[0] = __builtin_fmaf(a, x.x, acc[0]);
-    acc[1] = __builtin_fmaf(b, x.y, acc[1]);
-    acc[2] = __builtin_fmaf(c, x.z, acc[2]);
-    acc[3] = __builtin_fmaf(d, x.w, acc[3]);
-}
-__device__ __forceinline__ float sum4(const float (&a)[4]) { return (a[0] + a[1]) + (a[2] + a[3]); }
-
 // Where a lane finds the activations of its unit: quad g (values 4g..4g+3 in unit order) and partial sum i of
 // batch row b.  XLds reads them from the staged LDS copy; XReg holds them in registers (batch 1).
 struct XLds {
@@ -114,16 +103,11 @@ struct Unit<F_Q4_K> {
 
     template <int B, int R, int CV, class X>
     __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
-        constexpr bool WIDE = R * B <= 2;  // eight independent partial sums per (row, batch) pair instead of two
-        float sl[R][B], sh[R][B], wl[R][B][4], wh[R][B][4];
+        float sl[R][B], sh[R][B];
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int b = 0; b < B; ++b) {
-                sl[r][b] = sh[r][b] = 0.f;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) wl[r][b][i] = wh[r][b][i] = 0.f;
-            }
+            for (int b = 0; b < B; ++b) sl[r][b] = sh[r][b] = 0.f;
 #pragma unroll
         for (int d = 0; d < 8; ++d) {
             // decode the step's nibbles of every row first, then walk the batch rows: one pair of activation quads
@@ -140,24 +124,10 @@ struct Unit<F_Q4_K> {
                 const float4 xa = xs.q(b, d), xb = xs.q(b, d + 8);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    if constexpr (WIDE) {
-                        dot4w(lo[r][0], lo[r][1], lo[r][2], lo[r][3], xa, wl[r][b]);
-                        dot4w(hi[r][0], hi[r][1], hi[r][2], hi[r][3], xb, wh[r][b]);
-                    } else {
-                        sl[r][b] = dot4(lo[r][0], lo[r][1], lo[r][2], lo[r][3], xa, sl[r][b]);
-                        sh[r][b] = dot4(hi[r][0], hi[r][1], hi[r][2], hi[r][3], xb, sh[r][b]);
-                    }
+                    sl[r][b] = dot4(lo[r][0], lo[r][1], lo[r][2], lo[r][3], xa, sl[r][b]);
+                    sh[r][b] = dot4(hi[r][0], hi[r][1], hi[r][2], hi[r][3], xb, sh[r][b]);
                 }
             }
-        }
-        if constexpr (WIDE) {
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int b = 0; b < B; ++b) {
-                    sl[r][b] = sum4(wl[r][b]);
-                    sh[r][b] = sum4(wh[r][b]);
-                }
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
@@ -281,18 +251,13 @@ struct Unit<F_Q6_K> {
     template <int B, int R, int CV, class X>
     __device__ static __forceinline__ void dot(const Raw (&w)[R], int u, const X &xs, float (&acc)[R][B], float nib) {
         (void)nib;
-        constexpr bool WIDE = R * B <= 1;  // sixteen independent partial sums instead of four
-        float s[R][B][4], ws[R][B][4][4];
+        float s[R][B][4];
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
             for (int b = 0; b < B; ++b)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    s[r][b][k] = 0.f;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) ws[r][b][k][i] = 0.f;
-                }
+                for (int k = 0; k < 4; ++k) s[r][b][k] = 0.f;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             uint32_t q0[R], q1[R], q2[R], q3[R];
@@ -309,27 +274,12 @@ struct Unit<F_Q6_K> {
                 const float4 x0 = xs.q(b, p), x1 = xs.q(b, 4 + p), x2 = xs.q(b, 8 + p), x3 = xs.q(b, 12 + p);
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
-                    if constexpr (WIDE) {
-                        dot4w(ub0(q0[r]), ub1(q0[r]), ub2(q0[r]), ub3(q0[r]), x0, ws[r][b][0]);
-                        dot4w(ub0(q1[r]), ub1(q1[r]), ub2(q1[r]), ub3(q1[r]), x1, ws[r][b][1]);
-                        dot4w(ub0(q2[r]), ub1(q2[r]), ub2(q2[r]), ub3(q2[r]), x2, ws[r][b][2]);
-                        dot4w(ub0(q3[r]), ub1(q3[r]), ub2(q3[r]), ub3(q3[r]), x3, ws[r][b][3]);
-                    } else {
-                        s[r][b][0] = dot4(ub0(q0[r]), ub1(q0[r]), ub2(q0[r]), ub3(q0[r]), x0, s[r][b][0]);
-                        s[r][b][1] = dot4(ub0(q1[r]), ub1(q1[r]), ub2(q1[r]), ub3(q1[r]), x1, s[r][b][1]);
-                        s[r][b][2] = dot4(ub0(q2[r]), ub1(q2[r]), ub2(q2[r]), ub3(q2[r]), x2, s[r][b][2]);
-                        s[r][b][3] = dot4(ub0(q3[r]), ub1(q3[r]), ub2(q3[r]), ub3(q3[r]), x3, s[r][b][3]);
-                    }
+                    s[r][b][0] = dot4(ub0(q0[r]), ub1(q0[r]), ub2(q0[r]), ub3(q0[r]), x0, s[r][b][0]);
+                    s[r][b][1] = dot4(ub0(q1[r]), ub1(q1[r]), ub2(q1[r]), ub3(q1[r]), x1, s[r][b][1]);
+                    s[r][b][2] = dot4(ub0(q2[r]), ub1(q2[r]), ub2(q2[r]), ub3(q2[r]), x2, s[r][b][2]);
+                    s[r][b][3] = dot4(ub0(q3[r]), ub1(q3[r]), ub2(q3[r]), ub3(q3[r]), x3, s[r][b][3]);
                 }
             }
-        }
-        if constexpr (WIDE) {
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int b = 0; b < B; ++b)
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) s[r][b][k] = sum4(ws[r][b][k]);
         }
         const int sh = (u & 1) * 8;
 #pragma unroll

@@ -208,13 +208,7 @@ xreg_fn pick_xreg(int fmt, bool pairs, int mode, int pf) {
     case 1: return pf == 1 ? pick_xreg_fmt<1, true, false, false>(fmt, pairs) : pick_xreg_fmt<2, true, false, false>(fmt, pairs);
     case 2: return pf == 1 ? pick_xreg_fmt<1, false, true, false>(fmt, pairs) : pick_xreg_fmt<2, false, true, false>(fmt, pairs);
     case 3: return pf == 1 ? pick_xreg_fmt<1, false, true, true>(fmt, pairs) : pick_xreg_fmt<3, false, true, true>(fmt, pairs);
-    default:
-        if (fmt == F_Q4_K && pf == 3) return gemv_xreg_kernel<Unit<F_Q4_K>, 1, 3, false, false, false>;
-        if (fmt == F_Q4_K && pf == 4) return gemv_xreg_kernel<Unit<F_Q4_K>, 1, 4, false, false, false>;
-        if (fmt == F_Q4_K && pf == 6) return gemv_xreg_kernel<Unit<F_Q4_K>, 1, 6, false, false, false>;
-        if (fmt == F_Q6_K && pf == 3) return gemv_xreg_kernel<Unit<F_Q6_K>, 0, 3, false, false, false>;
-        if (fmt == F_Q6_K && pf == 4) return gemv_xreg_kernel<Unit<F_Q6_K>, 0, 4, false, false, false>;
-        return pf == 1 ? pick_xreg_fmt<1, false, false, false>(fmt, pairs) : pick_xreg_fmt<2, false, false, false>(fmt, pairs);
+    default: return pf == 1 ? pick_xreg_fmt<1, false, false, false>(fmt, pairs) : pick_xreg_fmt<2, false, false, false>(fmt, pairs);
     }
 }
 
