@@ -18,7 +18,9 @@
  *    (core/Tensor.java:249-278); it stays in that layout in HBM.
  *  - Activations and outputs are FP32 row-major: x [rows, k], y [rows, n], bias [n].
  *  - "_dev" entry points take device pointers and a hipStream_t passed as void* (NULL = the null stream);
- *    they only enqueue work.  Entry points without "_dev" take host pointers and are synchronous.
+ *    they only enqueue work.  Entry points without "_dev" take host pointers and are synchronous: they copy
+ *    through pinned host memory and a device buffer that the library keeps per calling thread (no allocation
+ *    per call once the buffers have grown to the largest call) on a stream of that thread.
  *  - Thread safety: weights are immutable after upload and may be shared by any number of threads;
  *    each call uses only its arguments and per-call stream order; the last-error string is thread-local.
  */
@@ -62,6 +64,12 @@ JITNN_HIP_API int jitnn_hip_device_info(char *name, int cap, int *compute_units,
 JITNN_HIP_API const char *jitnn_hip_last_error(void);
 
 JITNN_HIP_API int jitnn_hip_sync(void);
+
+/* Frees what the library keeps for the calling thread: the staging buffers and the stream of the host-pointer entry
+ * points and the scratch of the many-row path (both grow on demand and are otherwise kept until the thread ends; the
+ * process's first thread keeps them until the process ends).  Waits for the device first.  The counterpart of dropping
+ * a thread's derived copies (core/cpu/Gemm.java:497-515). */
+JITNN_HIP_API int jitnn_hip_thread_release(void);
 
 /* ---- block formats (no device needed) ------------------------------------------------------------ */
 

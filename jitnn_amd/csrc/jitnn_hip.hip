@@ -17,6 +17,9 @@
 #include <utility>
 #include <vector>
 
+#include <sys/syscall.h>
+#include <unistd.h>
+
 #include "dequant.h"
 #include "gemv.h"
 #include "gemv_mfma.h"
@@ -118,6 +121,8 @@ struct StatNest {
 };
 
 bool known(int fmt) { return block_values(fmt) != 0; }
+
+bool calling_thread_is_main() { return (long)syscall(SYS_gettid) == (long)getpid(); }
 
 // Kernels that want more than 64 KiB of dynamic LDS must be told so once; remembered per kernel so that steady-state
 // launches (and launches under graph capture) make no attribute calls.
@@ -480,6 +485,69 @@ int workspace_done(hipStream_t stream) {
     return JITNN_HIP_OK;
 }
 
+// Per-thread staging of the host-pointer entry points (jitnn_hip_linear, _dequantize, _quantize_q8_0, the model steps
+// on host buffers): a pinned host buffer, a device buffer and a stream, all grow-only, so that a call costs copies and
+// launches but no allocation.  Buffers beyond STAGE_KEEP_MAX are not kept (a dequantised matrix goes through in pieces).
+constexpr size_t STAGE_KEEP_MAX = (size_t)128 << 20;
+struct HostStage {
+    uint8_t *pinned = nullptr, *dev = nullptr;
+    size_t pcap = 0, dcap = 0;
+    hipStream_t stream = nullptr;
+    void release() {
+        if (pinned) (void)hipHostFree(pinned);
+        if (dev) (void)hipFree(dev);
+        if (stream) (void)hipStreamDestroy(stream);
+        pinned = dev = nullptr;
+        pcap = dcap = 0;
+        stream = nullptr;
+    }
+};
+void release_workspace() {
+    Workspace &w = g_ws;
+    if (w.ptr) (void)hipFree(w.ptr);
+    if (w.ev) (void)hipEventDestroy(w.ev);
+    w = Workspace{};
+}
+struct ThreadState {
+    HostStage stage;
+    // A thread that ends gives its device memory back.  The process's first thread ends with the process, when the HIP
+    // runtime may already be gone: its buffers are left to the process teardown.
+    ~ThreadState() {
+        if (is_main) return;
+        stage.release();
+        release_workspace();
+    }
+    bool is_main = false;
+};
+thread_local ThreadState g_thread;
+bool calling_thread_is_main();
+
+int stage_reserve(size_t pinned_bytes, size_t dev_bytes) {
+    HostStage &st = g_thread.stage;
+    g_thread.is_main = calling_thread_is_main();
+    if (!st.stream) HIP_TRY(hipStreamCreateWithFlags(&st.stream, hipStreamNonBlocking));
+    auto round = [](size_t b) { return (b + ((size_t)1 << 16) - 1) & ~(((size_t)1 << 16) - 1); };
+    if (pinned_bytes > st.pcap) {
+        if (st.pinned) HIP_TRY(hipHostFree(st.pinned));
+        st.pinned = nullptr;
+        st.pcap = 0;
+        const size_t want = round(pinned_bytes);
+        hipError_t e = hipHostMalloc((void **)&st.pinned, want, hipHostMallocDefault);
+        if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipHostMalloc of %zu bytes of staging: %s", want, hipGetErrorString(e));
+        st.pcap = want;
+    }
+    if (dev_bytes > st.dcap) {
+        if (st.dev) HIP_TRY(hipFree(st.dev));
+        st.dev = nullptr;
+        st.dcap = 0;
+        const size_t want = round(dev_bytes);
+        hipError_t e = hipMalloc((void **)&st.dev, want);
+        if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc of %zu bytes of staging: %s", want, hipGetErrorString(e));
+        st.dcap = want;
+    }
+    return JITNN_HIP_OK;
+}
+
 // More rows than the GEMV kernels take: FP16 activations in operand order + dequantise-to-LDS MFMA kernel.
 // `count` weights of one row length share the activations x [rows, k] (prepared once): ys[i] = x ws[i]^T (+ bias, one
 // weight only).  norm_w != nullptr: the RMSNorm in front of the linears is fused into the preparation (rows of at most
@@ -770,17 +838,23 @@ int jitnn_hip_dequantize_dev(const jitnn_hip_weight *w, float *y_dev, void *stre
 int jitnn_hip_dequantize(const jitnn_hip_weight *w, float *y_host) {
     if (!w || !y_host) return fail(JITNN_HIP_EINVAL, "weight or output is NULL");
     if (int rc = check_ready()) return rc;
-    const size_t bytes = (size_t)w->n * w->k * sizeof(float);
-    float *y = nullptr;
-    hipError_t e = hipMalloc(&y, bytes);
-    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc of %zu bytes: %s", bytes, hipGetErrorString(e));
-    int rc = jitnn_hip_dequantize_dev(w, y, nullptr);
-    if (rc == JITNN_HIP_OK) {
-        e = hipMemcpy(y_host, y, bytes, hipMemcpyDeviceToHost);
-        if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    // in pieces of whole rows through the thread's device buffer: no allocation per call, bounded memory for any matrix
+    const size_t row_out = (size_t)w->k * sizeof(float), row_in = (size_t)w->nbytes / w->n;
+    size_t piece_rows = ((size_t)64 << 20) / row_out;
+    if (piece_rows < 1) piece_rows = 1;
+    if (piece_rows > (size_t)w->n) piece_rows = (size_t)w->n;
+    if (int rc = stage_reserve(0, piece_rows * row_out)) return rc;
+    HostStage &st = g_thread.stage;
+    count_op(ST_DEQUANT, (long long)w->nbytes + 4ll * w->n * w->k);
+    StatNest nest;
+    for (size_t r0 = 0; r0 < (size_t)w->n; r0 += piece_rows) {
+        const size_t nr = std::min(piece_rows, (size_t)w->n - r0);
+        const jitnn_hip_weight part{w->fmt, (int)nr, w->k, (long long)(nr * row_in), w->dev + r0 * row_in, false};
+        if (int rc = jitnn_hip_dequantize_dev(&part, (float *)st.dev, st.stream)) return rc;
+        HIP_TRY(hipMemcpyAsync((uint8_t *)y_host + r0 * row_out, st.dev, nr * row_out, hipMemcpyDeviceToHost, st.stream));
+        HIP_TRY(hipStreamSynchronize(st.stream));
     }
-    (void)hipFree(y);
-    return rc;
+    return JITNN_HIP_OK;
 }
 
 int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, void *stream) {
@@ -802,22 +876,32 @@ int jitnn_hip_linear(const jitnn_hip_weight *w, const float *x_host, int rows, c
     if (!w || !x_host || !y_host) return fail(JITNN_HIP_EINVAL, "weight, input or output is NULL");
     if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
     if (int rc = check_ready()) return rc;
+    // layout of both staging buffers: [x | bias | y], x and bias going up in one copy, y coming back in one
     const size_t xb = (size_t)rows * w->k * 4, yb = (size_t)rows * w->n * 4, bb = bias_host ? (size_t)w->n * 4 : 0;
-    uint8_t *buf = nullptr;
-    const size_t xo = 0, yo = (xb + 255) & ~(size_t)255, bo = yo + ((yb + 255) & ~(size_t)255);
-    hipError_t e = hipMalloc(&buf, bo + bb + 256);
-    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc: %s", hipGetErrorString(e));
-    int rc = JITNN_HIP_OK;
-    e = hipMemcpy(buf + xo, x_host, xb, hipMemcpyHostToDevice);
-    if (e == hipSuccess && bias_host) e = hipMemcpy(buf + bo, bias_host, bb, hipMemcpyHostToDevice);
-    if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
-    if (rc == JITNN_HIP_OK)
-        rc = jitnn_hip_linear_dev(w, (const float *)(buf + xo), rows, bias_host ? (const float *)(buf + bo) : nullptr, (float *)(buf + yo), nullptr);
-    if (rc == JITNN_HIP_OK) {
-        e = hipMemcpy(y_host, buf + yo, yb, hipMemcpyDeviceToHost);
-        if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    const size_t bo = (xb + 255) & ~(size_t)255, yo = bo + ((bb + 255) & ~(size_t)255), total = yo + yb;
+    const bool keep = total <= STAGE_KEEP_MAX;  // small calls go through pinned memory (one DMA each way, no page locking per call)
+    if (int rc = stage_reserve(keep ? total : 0, total)) return rc;
+    HostStage &st = g_thread.stage;
+    if (keep) {
+        memcpy(st.pinned, x_host, xb);
+        if (bias_host) memcpy(st.pinned + bo, bias_host, bb);
+        HIP_TRY(hipMemcpyAsync(st.dev, st.pinned, bias_host ? bo + bb : xb, hipMemcpyHostToDevice, st.stream));
+    } else {
+        HIP_TRY(hipMemcpyAsync(st.dev, x_host, xb, hipMemcpyHostToDevice, st.stream));
+        if (bias_host) HIP_TRY(hipMemcpyAsync(st.dev + bo, bias_host, bb, hipMemcpyHostToDevice, st.stream));
     }
-    (void)hipFree(buf);
+    int rc = jitnn_hip_linear_dev(w, (const float *)st.dev, rows, bias_host ? (const float *)(st.dev + bo) : nullptr, (float *)(st.dev + yo), st.stream);
+    if (rc == JITNN_HIP_OK) {
+        HIP_TRY(hipMemcpyAsync(keep ? (void *)(st.pinned + yo) : (void *)y_host, st.dev + yo, yb, hipMemcpyDeviceToHost, st.stream));
+        HIP_TRY(hipStreamSynchronize(st.stream));
+        if (keep) memcpy(y_host, st.pinned + yo, yb);
+    }
+    if (!keep) {  // a buffer this large is not held on to
+        (void)hipStreamSynchronize(st.stream);
+        (void)hipFree(st.dev);
+        st.dev = nullptr;
+        st.dcap = 0;
+    }
     return rc;
 }
 
@@ -840,20 +924,29 @@ int jitnn_hip_quantize_q8_0(const float *x_host, long long numel, void *blocks_h
     if (numel < 0 || numel % 32 != 0) return fail(JITNN_HIP_EINVAL, "Q8_0 needs a multiple of 32 values, got %lld", numel);
     if (int rc = check_ready()) return rc;
     if (numel == 0) return JITNN_HIP_OK;
-    const size_t xb = (size_t)numel * 4, qb = (size_t)numel / 32 * 34;
-    uint8_t *buf = nullptr;
-    hipError_t e = hipMalloc(&buf, xb + qb);
-    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc: %s", hipGetErrorString(e));
-    int rc = JITNN_HIP_OK;
-    e = hipMemcpy(buf, x_host, xb, hipMemcpyHostToDevice);
-    if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
-    if (rc == JITNN_HIP_OK) rc = jitnn_hip_quantize_q8_0_dev((const float *)buf, numel, buf + xb, nullptr);
-    if (rc == JITNN_HIP_OK) {
-        e = hipMemcpy(blocks_host, buf + xb, qb, hipMemcpyDeviceToHost);
-        if (e != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "hipMemcpy: %s", hipGetErrorString(e));
+    // in pieces of whole blocks through the thread's device buffer
+    const long long piece = (long long)16 << 20;  // values per piece: 64 MiB in, 17 MiB out
+    const size_t xmax = (size_t)std::min(numel, piece) * 4, qo = (xmax + 255) & ~(size_t)255;
+    if (int rc = stage_reserve(0, qo + (size_t)std::min(numel, piece) / 32 * 34)) return rc;
+    HostStage &st = g_thread.stage;
+    count_op(ST_QUANT, 4ll * numel + numel / 32 * 34);
+    StatNest nest;
+    for (long long v0 = 0; v0 < numel; v0 += piece) {
+        const long long nv = std::min(piece, numel - v0);
+        HIP_TRY(hipMemcpyAsync(st.dev, x_host + v0, (size_t)nv * 4, hipMemcpyHostToDevice, st.stream));
+        if (int rc = jitnn_hip_quantize_q8_0_dev((const float *)st.dev, nv, st.dev + qo, st.stream)) return rc;
+        HIP_TRY(hipMemcpyAsync((uint8_t *)blocks_host + v0 / 32 * 34, st.dev + qo, (size_t)nv / 32 * 34, hipMemcpyDeviceToHost, st.stream));
+        HIP_TRY(hipStreamSynchronize(st.stream));
     }
-    (void)hipFree(buf);
-    return rc;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_thread_release(void) {
+    if (!g.ready) return JITNN_HIP_OK;
+    (void)hipDeviceSynchronize();
+    g_thread.stage.release();
+    release_workspace();
+    return JITNN_HIP_OK;
 }
 
 int jitnn_hip_probe_read_dev(const void *dev, long long nbytes, void *stream) {
@@ -988,8 +1081,8 @@ int jitnn_hip_gguf_tensor_upload(const jitnn_hip_gguf *h, const char *name, jitn
     if (!t) return fail(JITNN_HIP_EINVAL, "%s: no tensor %s", h->f->path.c_str(), name);
     if (!known(t->type_id)) {
         const GgmlTypeInfo *ti = ggml_type(t->type_id);
-        return fail(JITNN_HIP_EUNSUPPORTED, "%s: ggml type %s%d has no block-quantised tensor type on this path", name, ti ? ti->name : "id ",
-                    ti ? 0 : t->type_id);
+        if (ti) return fail(JITNN_HIP_EUNSUPPORTED, "%s: ggml type %s has no block-quantised tensor type on this path", name, ti->name);
+        return fail(JITNN_HIP_EUNSUPPORTED, "%s: ggml type id %d has no block-quantised tensor type on this path", name, t->type_id);
     }
     if (t->shape.empty() || t->numel > 0x7fffffffLL)
         return fail(JITNN_HIP_EUNSUPPORTED, "%s: %lld values; tensors hold at most 2^31-1", name, t->numel);
@@ -1403,20 +1496,15 @@ int jitnn_hip_llama_prefill(jitnn_hip_llama *m, const float *x_host, int pos0, i
     if (int rc = check_model(m)) return rc;
     if (!x_host) return fail(JITNN_HIP_EINVAL, "input is NULL");
     if (tokens < 1) return fail(JITNN_HIP_EINVAL, "%d tokens", tokens);
-    float *x = nullptr;
     const size_t bytes = (size_t)tokens * m->d * 4;
-    if (hipMalloc(&x, bytes) != hipSuccess) {
-        (void)hipGetLastError();
-        return fail(JITNN_HIP_ENOMEM, "allocating %zu bytes of embeddings failed", bytes);
-    }
-    int rc = JITNN_HIP_OK;
-    if (hipMemcpy(x, x_host, bytes, hipMemcpyHostToDevice) != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "copying the embeddings failed");
-    if (!rc) rc = jitnn_hip_llama_prefill_dev(m, x, pos0, tokens, logits_host ? m->logits : nullptr, nullptr);
-    if (!rc && hipDeviceSynchronize() != hipSuccess) rc = fail(JITNN_HIP_EDEVICE, "the prefill step failed: %s", hipGetErrorString(hipGetLastError()));
-    if (!rc && logits_host && hipMemcpy(logits_host, m->logits, (size_t)m->vocab * 4, hipMemcpyDeviceToHost) != hipSuccess)
-        rc = fail(JITNN_HIP_EDEVICE, "copying the logits failed");
-    (void)hipFree(x);
-    return rc;
+    if (int rc = stage_reserve(0, bytes)) return rc;  // the embeddings go through the calling thread's device buffer
+    HostStage &st = g_thread.stage;
+    HIP_TRY(hipMemcpyAsync(st.dev, x_host, bytes, hipMemcpyHostToDevice, st.stream));
+    if (int rc = jitnn_hip_llama_prefill_dev(m, (const float *)st.dev, pos0, tokens, logits_host ? m->logits : nullptr, st.stream)) return rc;
+    if (logits_host) HIP_TRY(hipMemcpyAsync(logits_host, m->logits, (size_t)m->vocab * 4, hipMemcpyDeviceToHost, st.stream));
+    hipError_t e = hipStreamSynchronize(st.stream);
+    if (e != hipSuccess) return fail(JITNN_HIP_EDEVICE, "the prefill step failed: %s", hipGetErrorString(e));
+    return JITNN_HIP_OK;
 }
 
 int jitnn_hip_llama_decode(jitnn_hip_llama *m, const float *x_host, int pos, float *logits_host) {

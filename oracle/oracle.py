@@ -117,6 +117,30 @@ def gguf_linear(fmt: int, x, blocks, bias, n: int, k: int) -> np.ndarray:
     return y
 
 
+def gguf_linear_rows_parallel(fmt: int, x, blocks, bias, n: int, k: int, threads: int = 8) -> np.ndarray:
+    """gguf_linear with the output rows shared out over `threads` host threads.  Output rows are independent in the
+    reference's loop, so the result is bit-identical to the one-thread call; this only shortens the wait in tests of
+    whole models (the timed CPU baseline always runs the one-thread loop, which is what the reference does)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    x = _f32(x).reshape(-1, k)
+    w = _u8(blocks)
+    rb = nbytes(fmt, k)
+    assert w.size == rb * n, (w.size, rb, n)
+    b = None if bias is None else _f32(bias)
+    step = max(1, (n + threads - 1) // threads)
+    cuts = list(range(0, n, step))
+
+    def part(r0):
+        r1 = min(n, r0 + step)
+        return gguf_linear(fmt, x, w[r0 * rb:r1 * rb], None if b is None else b[r0:r1], r1 - r0, k)
+
+    if len(cuts) == 1:
+        return part(0)
+    with ThreadPoolExecutor(max_workers=threads) as pool:  # ctypes releases the GIL inside the C call
+        return np.concatenate(list(pool.map(part, cuts)), axis=1)
+
+
 def matmul_nt(a, b) -> np.ndarray:
     a, b = _f32(a), _f32(b)
     c = np.empty((a.shape[0], b.shape[0]), dtype=np.float32)

@@ -131,7 +131,10 @@ def test_prefill_matches_token_by_token_reference(jn, pos0, tokens, bar):
     assert norm_err(y, ref) <= bar, norm_err(y, ref)
     for li in range(cfg["layers"]):
         k, v = dec.kv_read(li, pos0, tokens)
-        assert norm_err(k, kc[li, pos0:pos0 + tokens]) <= bar and norm_err(v, vc[li, pos0:pos0 + tokens]) <= bar, li
+        # layer 0's keys and values are one linear of the normalised input each: the bar of that linear's path (2e-3 on
+        # FP16 operands); deeper layers sit behind attention and further linears
+        kv_bar = bar if tokens <= 64 or li > 0 else 2e-3
+        assert norm_err(k, kc[li, pos0:pos0 + tokens]) <= kv_bar and norm_err(v, vc[li, pos0:pos0 + tokens]) <= kv_bar, li
     # decoding goes on from the prefilled cache
     xn = rng.standard_normal(cfg["d_model"]).astype(np.float32)
     ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, xn, pos0 + tokens)
@@ -161,7 +164,14 @@ def test_prefill_head_shapes(jn, heads, kv_heads, head_dim, tokens, bar):
     y = dec.prefill(x, pos0)
     assert norm_err(y, ref) <= bar, norm_err(y, ref)
     k, v = dec.kv_read(0, pos0, tokens)
-    assert norm_err(k, kc[0, pos0:pos0 + tokens]) <= bar and norm_err(v, vc[0, pos0:pos0 + tokens]) <= bar
+    kv_bar = bar if tokens <= 64 else 2e-3  # one linear of the normalised input: the bar of the linear's own path
+    assert norm_err(k, kc[0, pos0:pos0 + tokens]) <= kv_bar and norm_err(v, vc[0, pos0:pos0 + tokens]) <= kv_bar
+    # one more token on the prefilled cache: the single-token attention kernel of this head size
+    xn = rng.standard_normal(cfg["d_model"]).astype(np.float32)
+    ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, xn, pos0 + tokens)
+    assert norm_err(dec.decode(xn, pos0 + tokens), ref) <= bar
+    kn, vn = dec.kv_read(0, pos0 + tokens, 1)
+    assert norm_err(kn[0], kc[0, pos0 + tokens]) <= kv_bar and norm_err(vn[0], vc[0, pos0 + tokens]) <= kv_bar
     dec.close()
 
 

@@ -31,11 +31,30 @@ def rows_of(raw, fmt, k, sel):
     return np.ascontiguousarray(raw.reshape(-1, rb)[sel]).reshape(-1)
 
 
+def baseline_weight(fmt, n, k, seed):
+    """The BASELINE configurations' weight: FP32 [n, k] drawn from N(0, 0.02) and quantised to fmt - Q8_0 with the
+    reference's own quantiser as the oracle restates it (Quant.java:102-118), the others with tests/quantizers.py; drawn
+    and quantised on the GPU by torch in row chunks (set-up only: the bytes then go to the oracle and the library)."""
+    import torch
+
+    import quantizers
+    from oracle import oracle
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    parts = []
+    for r0 in range(0, n, 8192):
+        w = torch.randn(min(8192, n - r0), k, generator=g, device="cuda") * 0.02
+        parts.append(oracle.quantize_q8_0(w.cpu().numpy()) if fmt == "Q8_0" else quantizers.quantize(fmt, w).cpu().numpy())
+        del w
+    torch.cuda.empty_cache()
+    return np.concatenate(parts)
+
+
+@pytest.mark.parametrize("source", ["random_blocks", "normal_0.02_quantised"])
 @pytest.mark.parametrize("fmt,n,k,batches", CONFIGS)
-def test_full_size_gemv(jn, fmt, n, k, batches):
+def test_full_size_gemv(jn, fmt, n, k, batches, source):
     from oracle import oracle
     rng = np.random.default_rng(GGML_ID[fmt] * 7 + n)
-    raw = random_valid_blocks(rng, fmt, n, k)
+    raw = random_valid_blocks(rng, fmt, n, k) if source == "random_blocks" else baseline_weight(fmt, n, k, 1000 + GGML_ID[fmt])
     w = jn.Tensor.quantized(jn.DType[fmt], raw, n, k)
     sel = np.unique(rng.integers(0, n, size=48))
     sub = rows_of(raw, fmt, k, sel)

@@ -202,6 +202,25 @@ def test_small_k_32_blocks_and_many_rows(jn, fmt):
         assert norm_err(y, ref) <= bar(rows), (fmt, rows, norm_err(y, ref))
 
 
+@pytest.mark.parametrize("fmt", ["Q4_0", "Q4_1", "Q8_0"])
+@pytest.mark.parametrize("k", [96, 160])
+def test_odd_block_counts_at_every_batch_size(jn, fmt, k):
+    """Rows of 3 and 5 blocks (no pairs of blocks, no whole 256-value columns) at 1..8 rows: the single-block variants of
+    the register kernels and of the kernel with the activations in LDS."""
+    from oracle import oracle
+    rng = np.random.default_rng(k + GGML_ID[fmt])
+    n = 45
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    for rows in range(1, 9):
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        b = bias if rows % 2 == 0 else None
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, b, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(b) if b is not None else None).numpy()
+        assert norm_err(y, ref) <= GEMV_BAR, (fmt, k, rows, norm_err(y, ref))
+
+
 PREFILL_SHAPES = [  # (n, k, rows): ragged tiles in every dimension, K past one step, K split into 8 and into 4 slices,
     # and (130 x 4352) into four slices of unequal length: 17 blocks of 256 over slices of whole blocks
     (256, 1024, 65), (131, 4096, 200), (64, 14336, 97), (130, 512, 129), (1, 256, 70), (384, 4096, 513), (130, 4352, 129),

@@ -63,3 +63,43 @@ def test_attention_decode_is_last_causal_row(goldens):
     vrep = np.repeat(vc, h // kv, axis=1).transpose(1, 0, 2)
     y2 = oracle.sdpa(q[:, None, :], krep, vrep, False)[:, 0, :]
     assert np.array_equal(y, y2)
+
+
+def test_prefill_ref_is_decode_ref_token_by_token():
+    """The many-token restatement used by the full-size prefill test is the decode oracle applied token by token: same
+    cache rows, same last-token logits, up to the summation order of the FP64 accumulator of the linears."""
+    import torch
+
+    import quantizers
+    from decode_oracle import SLOTS, decode_ref, prefill_ref
+    from helpers import GGML_ID
+    cfg = dict(layers=2, d_model=256, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=96, max_ctx=16, rms_eps=1e-5, rope_theta=5e5)
+    g = torch.Generator().manual_seed(3)
+    rng = np.random.default_rng(3)
+    d, qd, kd, ffn = 256, 256, 128, 512
+    shapes = {"attn_q": (qd, d), "attn_k": (kd, d), "attn_v": (kd, d), "attn_o": (d, qd), "ffn_gate": (ffn, d), "ffn_up": (ffn, d),
+              "ffn_down": (d, ffn)}
+    fmts = {"attn_q": "Q4_K", "attn_k": "Q4_K", "attn_v": "Q6_K", "attn_o": "Q4_0", "ffn_gate": "Q5_K", "ffn_up": "Q5_K", "ffn_down": "Q6_K"}
+    layers = []
+    for _ in range(2):
+        L = {}
+        for slot in SLOTS:
+            n, k = shapes[slot]
+            L[slot] = (GGML_ID[fmts[slot]], quantizers.quantize(fmts[slot], torch.randn(n, k, generator=g) * 0.05).numpy(), n, k)
+        L["attn_norm"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+        L["ffn_norm"] = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+        layers.append(L)
+    out_norm = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    out_w = (8, quantizers.quantize("Q8_0", torch.randn(96, d, generator=g) * 0.05).numpy(), 96, d)
+    pos0, T = 3, 9
+    k0 = np.zeros((2, 16, 2, 64), dtype=np.float32)
+    v0 = np.zeros_like(k0)
+    k0[:, :pos0] = rng.standard_normal(k0[:, :pos0].shape)
+    v0[:, :pos0] = rng.standard_normal(v0[:, :pos0].shape)
+    x = rng.standard_normal((T, d)).astype(np.float32)
+    ka, va, kb, vb = k0.copy(), v0.copy(), k0.copy(), v0.copy()
+    for t in range(T):
+        ref = decode_ref(cfg, layers, out_norm, out_w, ka, va, x[t], pos0 + t)
+    got = prefill_ref(cfg, layers, out_norm, out_w, kb, vb, x, pos0)
+    assert np.abs(got - ref).max() <= 1e-6 * np.abs(ref).max()
+    assert np.abs(ka - kb).max() <= 1e-6 * np.abs(ka).max() and np.abs(va - vb).max() <= 1e-6 * np.abs(va).max()
