@@ -34,6 +34,8 @@ def decode_ref(cfg, layers, out_norm, out_w, kcache, vcache, x, pos, threads: in
         x = oracle.add(x, lin(L["attn_o"], att.reshape(-1)))
         m = oracle.rms_norm(x, L["ffn_norm"], eps)
         x = oracle.add(x, lin(L["ffn_down"], oracle.swiglu(lin(L["ffn_gate"], m), lin(L["ffn_up"], m))))
+        if threads > 1 and li % 8 == 7:
+            print(f"  oracle: layer {li + 1} of {len(layers)}", flush=True)
     return lin(out_w, oracle.rms_norm(x, out_norm, eps))
 
 

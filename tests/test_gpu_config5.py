@@ -46,6 +46,8 @@ def build_8b(jn, layers, vocab, max_ctx, seed):
             L[name] = (1.0 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
             dec.set_norm(li, ni, L[name])
         stack.append(L)
+        if li % 8 == 7:
+            print(f"  built layer {li + 1} of {layers}", flush=True)
     out_norm = (1.0 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
     dec.set_norm(0, 2, out_norm)
     parts = [quantizers.quantize("Q6_K", torch.randn(min(8192, vocab - r0), 4096, generator=g, device="cuda") * 0.02) for r0 in range(0, vocab, 8192)]
