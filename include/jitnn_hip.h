@@ -118,6 +118,19 @@ JITNN_HIP_API int jitnn_hip_dequantize_dev(const jitnn_hip_weight *w, float *y_d
 JITNN_HIP_API int jitnn_hip_linear(const jitnn_hip_weight *w, const float *x_host, int rows, const float *bias_host, float *y_host);
 JITNN_HIP_API int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, void *stream);
 
+/* jitnn_hip_linear_dev for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments, same kernels, same results;
+ * where jitnn_hip_linear_dev takes the scratch of a many-row launch (FP16 activations in operand order, their row
+ * scales, the partial sums of K slices) from a buffer of the calling thread that it may have to allocate or grow, this
+ * entry point takes it from a fixed array of jitnn_hip_noalloc_scratch_bytes() (64 MiB) that the library holds on the
+ * GPU for the life of the process, and never calls hipMalloc or hipFree.  A call that needs more scratch (roughly
+ * rows * k * 2 bytes + up to 8 * rows * n * 4 bytes for launches that split K) fails with JITNN_HIP_EINVAL before
+ * anything is enqueued.  Every call on a GPU shares that one array: calls that overlap in time on one GPU (different
+ * streams or threads) race on it - keep them on one stream, or order them with events. */
+JITNN_HIP_API int jitnn_hip_linear_noalloc_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev,
+                                               void *stream);
+JITNN_HIP_API long long jitnn_hip_noalloc_scratch_bytes(void);
+
 /* ---- Q8_0 quantiser ----------------------------------------------------------------------------- */
 
 /* FP32 -> Q8_0 blocks (34 bytes per 32 values) with the reference quantiser's arithmetic: F.quantizeQ8 /

@@ -45,6 +45,8 @@ def _bind() -> C.CDLL:
         "jitnn_hip_dequantize_dev": (i, [vp, vp, vp]),
         "jitnn_hip_linear": (i, [vp, vp, i, vp, vp]),
         "jitnn_hip_linear_dev": (i, [vp, vp, i, vp, vp, vp]),
+        "jitnn_hip_linear_noalloc_dev": (i, [vp, vp, i, vp, vp, vp]),
+        "jitnn_hip_noalloc_scratch_bytes": (ll, []),
         "jitnn_hip_thread_release": (i, []),
         "jitnn_hip_quantize_q8_0": (i, [vp, ll, vp]),
         "jitnn_hip_quantize_q8_0_dev": (i, [vp, ll, vp, vp]),

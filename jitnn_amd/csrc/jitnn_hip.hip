@@ -38,6 +38,12 @@ struct jitnn_hip_weight {
     bool owned;
 };
 
+// Scratch of the entry point that allocates nothing (jitnn_hip_linear_noalloc_dev): FP16 activations in operand order,
+// their row scales and the partial sums of K slices of a many-row linear.  One copy per GPU, held until the process
+// ends.  In host code this name is only a handle for hipGetSymbolAddress; the device address is kept in State.
+#define JITNN_HIP_SCRATCH_BYTES (64ull << 20)
+static __device__ __align__(256) unsigned char scratch[JITNN_HIP_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -80,6 +86,7 @@ struct State {
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
     bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
+    void *scratch_ptr = nullptr;    // device address of `scratch` on g.device (hipGetSymbolAddress at init)
 };
 State g;
 std::mutex g_mu;
@@ -459,7 +466,18 @@ struct Workspace {
 };
 thread_local Workspace g_ws;
 
-int workspace(size_t bytes, hipStream_t stream, void **out) {
+// Where a many-row launch takes its scratch from: the calling thread's grow-only buffer (may allocate), or the
+// library's static array (never allocates; the caller keeps calls on one GPU from overlapping).
+enum ScratchSource { SCRATCH_THREAD, SCRATCH_STATIC };
+
+int workspace(size_t bytes, hipStream_t stream, void **out, ScratchSource src = SCRATCH_THREAD) {
+    if (src == SCRATCH_STATIC) {
+        if (bytes > JITNN_HIP_SCRATCH_BYTES)
+            return fail(JITNN_HIP_EINVAL, "this call needs %zu bytes of scratch; the entry point that allocates nothing has %llu", bytes,
+                        (unsigned long long)JITNN_HIP_SCRATCH_BYTES);
+        *out = g.scratch_ptr;
+        return JITNN_HIP_OK;
+    }
     Workspace &w = g_ws;
     if (!w.ev) HIP_TRY(hipEventCreateWithFlags(&w.ev, hipEventDisableTiming));
     if (bytes > w.cap) {
@@ -477,7 +495,8 @@ int workspace(size_t bytes, hipStream_t stream, void **out) {
     return JITNN_HIP_OK;
 }
 
-int workspace_done(hipStream_t stream) {
+int workspace_done(hipStream_t stream, ScratchSource src = SCRATCH_THREAD) {
+    if (src == SCRATCH_STATIC) return JITNN_HIP_OK;
     Workspace &w = g_ws;
     HIP_TRY(hipEventRecord(w.ev, stream));
     w.last = stream;
@@ -556,7 +575,7 @@ int stage_reserve(size_t pinned_bytes, size_t dev_bytes) {
 // does not split K, by a pass of its own over the product left in `tmp` [rows, n].
 int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias,
                          const float *norm_w, float eps, hipStream_t stream, const float *residual = nullptr, float *tmp = nullptr,
-                         const float *swiglu_up = nullptr) {
+                         const float *swiglu_up = nullptr, ScratchSource src = SCRATCH_THREAD) {
     // (the kernels live in prefill_k.hip and prefill_q32.hip)
     struct Plan {
         bool kq;
@@ -593,7 +612,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     const size_t xo_bytes = (size_t)mblocks * pf_ksteps(k) * 1024;
     const size_t scale_bytes = ((size_t)rows * 8 + 255) & ~(size_t)255;
     void *wsp = nullptr;
-    if (int rc = workspace(xo_bytes + scale_bytes + part_max, stream, &wsp)) return rc;
+    if (int rc = workspace(xo_bytes + scale_bytes + part_max, stream, &wsp, src)) return rc;
     _Float16 *xo = (_Float16 *)wsp;
     float *scale = (float *)((uint8_t *)wsp + xo_bytes), *inv = scale + rows;
     float *part = (float *)((uint8_t *)wsp + xo_bytes + scale_bytes);
@@ -619,11 +638,12 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
         }
     }
     HIP_TRY(hipGetLastError());
-    return workspace_done(stream);
+    return workspace_done(stream, src);
 }
 
-int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
-    return launch_prefill_group(&w, &y, 1, x, rows, bias, nullptr, 0.f, stream);
+int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream,
+                   ScratchSource src = SCRATCH_THREAD) {
+    return launch_prefill_group(&w, &y, 1, x, rows, bias, nullptr, 0.f, stream, nullptr, nullptr, nullptr, src);
 }
 
 template <int FMT>
@@ -701,6 +721,12 @@ int jitnn_hip_init(int device_ordinal) {
     if (!(h[0] > 0.f) || h[1] != 15.f * h[0])
         return fail(JITNN_HIP_EDEVICE, "fp8 probe: E4M3 bytes 0x01, 0x0f decode to %g, %g; expected q * 2^-9 or q * 2^-10", h[0], h[1]);
     g.nib = 1.f / h[0];
+    {   // the device address of the static scratch on this GPU (every GPU holds its own copy at its own address)
+        void *sp = nullptr;
+        hipError_t se = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));
+        if (se != hipSuccess || !sp) return fail(JITNN_HIP_EDEVICE, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(se));
+        g.scratch_ptr = sp;
+    }
     if (const char *e = getenv("JITNN_HIP_XREG_BLOCKS")) {
         int v = atoi(e);
         if (v >= 1 && v <= 32) g.xreg_blocks_per_cu = v;
@@ -857,20 +883,37 @@ int jitnn_hip_dequantize(const jitnn_hip_weight *w, float *y_host) {
     return JITNN_HIP_OK;
 }
 
-int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, void *stream) {
+}  // extern "C"
+
+namespace {
+
+int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, hipStream_t s, ScratchSource src) {
     if (!w || !x_dev || !y_dev) return fail(JITNN_HIP_EINVAL, "weight, input or output is NULL");
     if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
     if (int rc = check_ready()) return rc;
-    hipStream_t s = (hipStream_t)stream;
     const bool many = rows > g.gemv_max_rows && !is_extra_format(w->fmt);
     count_op(many ? ST_MFMA : ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n) + (bias_dev ? 4ll * w->n : 0));
-    if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s);
+    if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s, src);
     for (int r0 = 0; r0 < rows; r0 += 8) {
         const int nb = rows - r0 < 8 ? rows - r0 : 8;
         if (int rc = launch_gemv(w, x_dev + (size_t)r0 * w->k, nb, bias_dev, y_dev + (size_t)r0 * w->n, s)) return rc;
     }
     return JITNN_HIP_OK;
 }
+
+}  // namespace
+
+extern "C" {
+
+int jitnn_hip_linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, void *stream) {
+    return linear_dev(w, x_dev, rows, bias_dev, y_dev, (hipStream_t)stream, SCRATCH_THREAD);
+}
+
+int jitnn_hip_linear_noalloc_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, void *stream) {
+    return linear_dev(w, x_dev, rows, bias_dev, y_dev, (hipStream_t)stream, SCRATCH_STATIC);
+}
+
+long long jitnn_hip_noalloc_scratch_bytes(void) { return (long long)JITNN_HIP_SCRATCH_BYTES; }
 
 int jitnn_hip_linear(const jitnn_hip_weight *w, const float *x_host, int rows, const float *bias_host, float *y_host) {
     if (!w || !x_host || !y_host) return fail(JITNN_HIP_EINVAL, "weight, input or output is NULL");

@@ -1,0 +1,64 @@
+"""jitnn_hip_linear_noalloc_dev - the entry point that takes the scratch of a many-row launch from the library's fixed
+device array instead of a buffer it may have to allocate - against jitnn_hip_linear_dev on the same inputs: the same
+kernels on the same operands, so the same bits.  Two calls in a row, the second smaller (the array keeps the first
+call's contents), then the GEMV range (no scratch at all) and the size limit."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import random_valid_blocks
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def jn():
+    import jitnn_amd
+    jitnn_amd.init()
+    return jitnn_amd
+
+
+def vp(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def run(lib, name, w, x, bias, n):
+    y = torch.full((x.shape[0], n), float("nan"), device="cuda")
+    st = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = getattr(lib.lib, name)(w.handle, vp(x), x.shape[0], vp(bias) if bias is not None else None, vp(y), st)
+    lib.check(rc, name)
+    torch.cuda.synchronize()
+    return y
+
+
+def test_noalloc_linear_matches_linear_dev(jn):
+    from jitnn_amd import _lib as lib
+    assert lib.lib.jitnn_hip_noalloc_scratch_bytes() == 64 << 20
+    rng = np.random.default_rng(12)
+    g = torch.Generator(device="cuda").manual_seed(12)
+    # 4096 x 4096 at 512 rows splits K into slices (partial sums in the scratch); the second call is smaller in every way
+    calls = [("Q4_K", 4096, 4096, 512, True), ("Q6_K", 300, 1024, 97, False), ("Q8_0", 131, 32 * 9, 70, True), ("Q4_K", 192, 2048, 5, False)]
+    for fmt, n, k, rows, with_bias in calls:
+        w = jn.Tensor.quantized(jn.DType[fmt], random_valid_blocks(rng, fmt, n, k), n, k)
+        x = torch.randn(rows, k, device="cuda", generator=g)
+        bias = torch.randn(n, device="cuda", generator=g) if with_bias else None
+        ref = run(lib, "jitnn_hip_linear_dev", w, x, bias, n)
+        got = run(lib, "jitnn_hip_linear_noalloc_dev", w, x, bias, n)
+        assert torch.isfinite(ref).all()
+        assert torch.equal(got, ref), (fmt, n, k, rows)
+        again = run(lib, "jitnn_hip_linear_noalloc_dev", w, x, bias, n)
+        assert torch.equal(again, ref), (fmt, n, k, rows, "second call")
+
+
+def test_noalloc_linear_rejects_what_does_not_fit(jn):
+    from jitnn_amd import _lib as lib
+    rng = np.random.default_rng(13)
+    n, k, rows = 64, 16384, 4096  # 4096 x 16384 FP16 activations alone are 128 MiB
+    w = jn.Tensor.quantized(jn.DType.Q4_0, random_valid_blocks(rng, "Q4_0", n, k), n, k)
+    x = torch.zeros(rows, k, device="cuda")
+    y = torch.zeros(rows, n, device="cuda")
+    rc = lib.lib.jitnn_hip_linear_noalloc_dev(w.handle, vp(x), rows, None, vp(y), None)
+    assert rc == lib.EINVAL and "scratch" in lib.last_error()
+    torch.cuda.synchronize()
