@@ -27,12 +27,23 @@ from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
-sys.path.insert(0, str(ROOT / "tests"))
 
 PEAK_HBM_GBPS = 8000.0
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc (profiles/gemv_q4_k_14336x4096_b1_pmc_traffic.txt):
-# FETCH_SIZE 16245.9 KiB x 2.0 (a 256 MiB copy kernel reads 131087 on this counter) + WRITE_SIZE 112.0 KiB x 1.0
-HEADLINE_TRAFFIC_BYTES = int((16245.9 * 2.0 + 112.0) * 1024)
+TRAFFIC_PROFILE = ROOT / "profiles" / "gemv_q4_k_14336x4096_b1_pmc_traffic.txt"
+
+
+def headline_traffic_bytes():
+    """HBM bytes per launch of the headline kernel as the committed rocprofv3 --pmc summary states them (FETCH_SIZE and
+    WRITE_SIZE per dispatch, each scaled by what the same counter reads for a plain copy of known size); None when the
+    summary is missing or does not hold the line."""
+    import re
+    try:
+        m = re.search(r"HBM traffic per GEMV launch =.*=\s*([0-9 ]+) bytes", TRAFFIC_PROFILE.read_text())
+        return int(m.group(1).replace(" ", "")) if m else None
+    except OSError:
+        return None
+
+
 BLOCK = {"Q8_0": (8, 32, 34), "Q4_0": (2, 32, 18), "Q4_1": (3, 32, 20), "Q4_K": (12, 256, 144), "Q5_K": (13, 256, 176),
          "Q6_K": (14, 256, 210)}
 
@@ -46,7 +57,7 @@ class Workload:
     """One GEMV configuration: `copies` device-resident copies of a quantised weight, x and y on the device."""
 
     def __init__(self, torch, lib, fmt: str, n: int, k: int, b: int, copies: int, seed: int):
-        import quantizers
+        import quantizers  # quantizers.py beside this file: FP32 -> GGUF blocks for synthetic weights
         self.torch, self.lib, self.fmt, self.n, self.k, self.b = torch, lib, fmt, n, k, b
         fid = BLOCK[fmt][0]
         g = torch.Generator(device="cuda").manual_seed(seed)
@@ -151,26 +162,77 @@ def measure(torch, lib, fmt, n, k, b, copies, steps, warmup, seed, parity=True):
     return wl, out
 
 
-def cpu_baseline(wl: Workload, budget_s: float = 12.0):
-    """The oracle's restatement of Gguf.MatVec.reference (scalar, FP64 accumulation, one thread - what the reference's
-    CPU backend runs for quantised weights) on the same weight bytes and activations."""
+TILED_ROWS = 32  # jitnn.gguf.tiledRows (core/JitnnConfig.java:423-424)
+
+
+def cpu_route(fmt: str, rows: int) -> str:
+    """What the reference's Gguf.linear runs for this format and row count (core/ops/Gguf.java:76-98): the scalar
+    FP64 loop of gguf_matvec / linear_q8_0 on one thread, or dequantise (one thread) + the multithreaded FP32 GEMM."""
+    if fmt == "Q8_0":
+        return "scalar"
+    if (rows == 1 and fmt in ("Q4_0", "Q4_1", "Q4_K", "Q5_K", "Q6_K")) or (rows <= TILED_ROWS and fmt in ("Q4_0", "Q4_1", "Q5_K")):
+        return "scalar"
+    return "dequant_gemm"
+
+
+def cpu_baseline(wl: Workload, budget_s: float = 12.0, max_rows: int = 32768):
+    """The reference's CPU path for this workload, restated in C (oracle/), timed on this box's host cores on the same
+    weight bytes and activations: Gguf.MatVec.reference / Quant.LinearQ8.reference (scalar, FP64 accumulation, ONE thread -
+    what jitNN's CPU backend runs for quantised weights) where Gguf.linear takes that route, else Gguf.dequantize (one
+    thread) + the packed, K-blocked, 6 x 2-vector FMA GEMM on the physical cores of one socket.  Matrices of more than
+    `max_rows` weight rows are timed on their first `max_rows` rows and scaled (said in `sample`)."""
     import numpy as np
     from oracle import oracle
-    fid = BLOCK[wl.fmt][0]
-    raw = wl.weights[0].cpu().numpy()
+    fid, qk, nb = BLOCK[wl.fmt]
+    n = min(wl.n, max_rows)
+    rb = wl.k // qk * nb
+    raw = wl.weights[0][: n * rb].cpu().numpy()
     x = wl.x.cpu().numpy()
-    times = []
+    route = cpu_route(wl.fmt, wl.b)
+    threads = 1 if route == "scalar" else oracle.cpu_threads()
+    times, parts = [], []
     t_all = time.perf_counter()
     while True:
         t0 = time.perf_counter()
-        oracle.gguf_linear(fid, x, raw, None, wl.n, wl.k)
+        if route == "scalar":
+            oracle.gguf_linear(fid, x, raw, None, n, wl.k)
+        else:
+            _, t_deq, t_mm = oracle.dequant_gemm(fid, x, raw, None, n, wl.k, threads)
+            parts.append((t_deq, t_mm))
         times.append(time.perf_counter() - t0)
         if time.perf_counter() - t_all > budget_s or len(times) >= 9:
             break
-    med = float(np.median(times))
-    return {"value": wl.bytes / med / 1e9, "unit": "GB/s", "cores": 1, "kind": "port", "ms_per_step": med * 1e3,
-            "sample": f"the full {wl.fmt} {wl.n}x{wl.k} batch-{wl.b} GEMV, median of {len(times)} runs of the C restatement of the "
-                      "reference's scalar FP64 host loop (Gguf.MatVec.reference), same weight bytes and activations as the GPU"}
+    med = float(np.median(times)) * (wl.n / n)
+    what = (f"the full {wl.fmt} {wl.n}x{wl.k} batch-{wl.b} linear" if n == wl.n
+            else f"the first {n} of {wl.n} weight rows of the {wl.fmt} {wl.n}x{wl.k} batch-{wl.b} linear, time scaled by {wl.n / n:.3f}")
+    out = {"value": wl.bytes / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port", "ms_per_step": med * 1e3, "route": route,
+           "sample": f"{what}, median of {len(times)} runs of the C restatement of the reference's CPU path "
+                     + ("(scalar FP64 host loop, Gguf.MatVec.reference / Quant.LinearQ8.reference, one thread)" if route == "scalar" else
+                        f"(Gguf.dequantize on one thread + packed K-blocked FP32 GEMM of cpu/Gemm.java on {threads} threads, "
+                        f"{oracle.cpu_vector_lanes() * 32}-bit vectors)") + ", same weight bytes and activations as the GPU"}
+    if parts:
+        out["dequantize_ms"] = float(np.median([p[0] for p in parts])) * (wl.n / n) * 1e3
+        out["pack_and_gemm_ms"] = float(np.median([p[1] for p in parts])) * (wl.n / n) * 1e3
+    return out
+
+
+def host_path(torch, lib, wl: Workload, steps: int = 300):
+    """The same linear through the host-pointer entry point (jitnn_hip_linear: x from host memory, y back to host memory,
+    synchronous) - what a caller on the reference's Op.cpu seam gets - beside the device-resident launch."""
+    import numpy as np
+    x = np.ascontiguousarray(wl.x.cpu().numpy())
+    y = np.empty((wl.b, wl.n), dtype=np.float32)
+    xp, yp = x.ctypes.data_as(C.c_void_p), y.ctypes.data_as(C.c_void_p)
+    f = lib.lib.jitnn_hip_linear
+    for i in range(20):
+        lib.check(f(wl.handles[i % len(wl.handles)], xp, wl.b, None, yp), "jitnn_hip_linear")
+    t0 = time.perf_counter()
+    for i in range(steps):
+        f(wl.handles[i % len(wl.handles)], xp, wl.b, None, yp)
+    us = (time.perf_counter() - t0) / steps * 1e6
+    ok = bool(np.array_equal(y, wl.y.cpu().numpy())) if steps % len(wl.handles) == 1 % len(wl.handles) else None
+    return {"workload": f"{wl.fmt} {wl.n}x{wl.k} batch {wl.b} through jitnn_hip_linear (host pointers, synchronous, PCIe-inclusive)",
+            "us_per_call": us, "GBps": wl.bytes / us / 1e3, "steps": steps, "same_bits_as_device_path": ok}
 
 
 def quantized_device_weight(torch, lib, fmt, n, k, seed):
@@ -400,7 +462,8 @@ def main() -> int:
     # ---- headline: Q4_K 14336x4096 batch 1, rotating over 16 copies
     wl, head = measure(torch, lib, "Q4_K", 14336, 4096, 1, 16, a.steps, a.warmup, seed=1030)
     hot_wall, hot_ev = wl.time(min(a.steps, 2000), 50, rotate=False)
-    cpu = None if a.no_cpu else cpu_baseline(wl, 3.0 if a.quick else 12.0)
+    cpu = None if a.no_cpu else cpu_baseline(wl, 3.0 if a.quick else 8.0)
+    host = host_path(torch, lib, wl)
     head_bytes = wl.bytes
     wl.close()
 
@@ -413,6 +476,9 @@ def main() -> int:
             ("q4_0_11008x4096_b4", "Q4_0", 11008, 4096, 4, 16, 1020),
             ("q4_k_14336x4096_b2", "Q4_K", 14336, 4096, 2, 16, 1030),
             ("q4_k_14336x4096_b8", "Q4_K", 14336, 4096, 8, 16, 1030),
+            ("q4_k_14336x4096_b16", "Q4_K", 14336, 4096, 16, 16, 1030),
+            ("q4_k_14336x4096_b40", "Q4_K", 14336, 4096, 40, 16, 1030),
+            ("q4_k_14336x4096_b64", "Q4_K", 14336, 4096, 64, 16, 1030),
             ("q6_k_128256x4096_b1", "Q6_K", 128256, 4096, 1, 2, 1040),
         ]
         for name, fmt, n, k, b, copies, seed in extra:
@@ -420,6 +486,8 @@ def main() -> int:
                 continue
             steps = max(50, min(a.steps, 1000 if n < 100000 else 200))
             w2, out = measure(torch, lib, fmt, n, k, b, copies, steps, 20, seed)
+            if not a.no_cpu:
+                out["cpu_baseline"] = cpu_baseline(w2, 3.0)
             w2.close()
             configs[name] = out
 
@@ -451,9 +519,10 @@ def main() -> int:
                    "cache_resident_GBps": head_bytes * min(a.steps, 2000) / hot_ev / 1e9, "parity_norm_err": head["parity_norm_err"],
                    "pure_read_GBps": head["pure_read_GBps"], "pure_read_us_per_launch": head["pure_read_us_per_launch"]},
         "roofline": {"bound": "hbm", "achieved": head["GBps_events"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                     "frac": head["GBps_events"] / PEAK_HBM_GBPS, "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "frac": head["GBps_events"] / PEAK_HBM_GBPS, "traffic": headline_traffic_bytes(),
                      "kernel": "gemv Q4_K batch 1", "us_per_launch": head["us_per_step_events"]},
         "cpu_baseline": cpu,
+        "host_path": host,
         "configs": configs,
         "decode": decode,
         "prefill": prefill,

@@ -46,6 +46,9 @@ def _load() -> C.CDLL:
     lib.jo_matmul_nt_ref.restype = None
     lib.jo_gguf_linear.argtypes = [C.c_int, _f32p, _u8p, C.c_void_p, _f32p, C.c_int, C.c_int, C.c_int]
     lib.jo_quantize_q8_0_ref.argtypes = [_f32p, C.c_long, _u8p]
+    lib.jo_cpu_vector_lanes.argtypes = []
+    lib.jo_cpu_gemm_nt.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]
+    lib.jo_dequant_gemm.argtypes = [C.c_int, _f32p, _u8p, C.c_void_p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
     lib.jo_rms_norm.argtypes = [_f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_double]
     lib.jo_rms_norm.restype = None
     lib.jo_rope_tables.argtypes = [C.c_int, C.c_int, C.c_float, _f32p, _f32p]
@@ -139,6 +142,42 @@ def gguf_linear_rows_parallel(fmt: int, x, blocks, bias, n: int, k: int, threads
         return part(0)
     with ThreadPoolExecutor(max_workers=threads) as pool:  # ctypes releases the GIL inside the C call
         return np.concatenate(list(pool.map(part, cuts)), axis=1)
+
+
+def cpu_threads() -> int:
+    """The reference's default thread count (cpu/Cpu.java:221-225): physical cores among the processors this process may
+    use, at most the cores of one socket; the usable processors when the topology cannot be read."""
+    import os
+    try:
+        usable = sorted(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = list(range(os.cpu_count() or 1))
+    cores, per_socket = set(), {}
+    try:
+        for c in usable:
+            base = f"/sys/devices/system/cpu/cpu{c}/topology/"
+            core, pkg = open(base + "core_id").read().strip(), open(base + "physical_package_id").read().strip()
+            cores.add((pkg, core))
+            per_socket.setdefault(pkg, set()).add(core)
+    except OSError:
+        return max(1, len(usable))
+    return max(1, min(len(cores), max(len(v) for v in per_socket.values())))
+
+
+def cpu_vector_lanes() -> int:
+    return lib.jo_cpu_vector_lanes()
+
+
+def dequant_gemm(fmt: int, x, blocks, bias, n: int, k: int, threads: int):
+    """Gguf.linear's dequantise + FP32 GEMM branch as the reference's CPU backend runs it (oracle/jitnn_cpu_gemm.c);
+    returns (y [rows, n], seconds in the one-thread dequantiser, seconds in packing + GEMM)."""
+    x = _f32(x).reshape(-1, k)
+    b = None if bias is None else _f32(bias)
+    y = np.empty((x.shape[0], n), dtype=np.float32)
+    sec = (C.c_double * 2)()
+    rc = lib.jo_dequant_gemm(fmt, x, _u8(blocks), _opt(b), y, x.shape[0], n, k, threads, sec)
+    assert rc == 0, rc
+    return y, sec[0], sec[1]
 
 
 def matmul_nt(a, b) -> np.ndarray:

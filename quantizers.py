@@ -1,6 +1,7 @@
 """FP32 -> GGUF block quantisers for synthetic test and benchmark weights (torch ops: CPU or GPU tensors).
 
-Test tooling, not part of the path: the reference has no quantiser for these formats besides Q8_0
+Test and benchmark tooling (it sits beside bench.py, which draws its weights with it; tests/ imports it too), not part of
+the path: the reference has no quantiser for these formats besides Q8_0
 (core/ops/Quant.java:86-119), and parity is defined on the bytes both sides consume.  The layouts are ggml's
 block_q4_0 ... block_q6_K; the rounding choices are simple min/max fits, not ggml's error-minimising
 searches.  Every function returns a flat uint8 tensor of n*k/qk*nb bytes for w [n, k].

@@ -1,6 +1,6 @@
 """BASELINE config 5 at its full size: the 32-layer, d_model 4096, 32 / 8 heads of 128, FFN 14336, vocabulary 128256
 Q4_K_M decode step at context 512 against the composed CPU oracle, and a 512-token prompt through layers of that shape
-against the oracle applied token by token.  Weights are N(0, 0.02) through tests/quantizers.py (drawn and quantised on
+against the oracle applied token by token.  Weights are N(0, 0.02) through quantizers.py (drawn and quantised on
 the GPU with torch to keep the set-up short; the bytes then go to the oracle and, through the C ABI, to the library)."""
 import os
 

@@ -33,7 +33,7 @@ def rows_of(raw, fmt, k, sel):
 
 def baseline_weight(fmt, n, k, seed):
     """The BASELINE configurations' weight: FP32 [n, k] drawn from N(0, 0.02) and quantised to fmt - Q8_0 with the
-    reference's own quantiser as the oracle restates it (Quant.java:102-118), the others with tests/quantizers.py; drawn
+    reference's own quantiser as the oracle restates it (Quant.java:102-118), the others with quantizers.py; drawn
     and quantised on the GPU by torch in row chunks (set-up only: the bytes then go to the oracle and the library)."""
     import torch
 

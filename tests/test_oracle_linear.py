@@ -138,3 +138,21 @@ def test_quantize_q8_0_invariants():
     assert np.all(np.abs(dq - x.reshape(-1, 32)) <= (step * (0.5 + 127 * 2.0 ** -11) + 1e-12)[:, None])
     scale = np.abs(x).max()
     assert np.abs(dq.reshape(-1) - x).max() <= scale * (1 / 127.0) + 1e-6
+
+
+def test_cpu_dequant_gemm_baseline_agrees_with_the_oracle():
+    """The C restatement of the reference's dequantise + GEMM branch (the CPU baseline of the many-row configurations)
+    against the FP64 oracle on the same blocks: equal within FP32 rounding of a K-blocked FMA sum, at ragged sizes (edge
+    panels in both directions, K past one block of 256), for one thread and for several."""
+    from oracle import oracle
+    rng = np.random.default_rng(77)
+    for fmt, n, k, rows in (("Q4_K", 70, 768, 13), ("Q6_K", 33, 512, 40), ("Q4_0", 129, 96, 7), ("Q8_0", 16, 32, 1)):
+        raw = random_valid_blocks(rng, fmt, n, k)
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32)
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, bias, n, k)
+        for threads in (1, 3):
+            y, t_deq, t_mm = oracle.dequant_gemm(GGML_ID[fmt], x, raw, bias, n, k, threads)
+            assert norm_err(y, ref) <= 2e-6, (fmt, threads, norm_err(y, ref))
+            assert t_deq >= 0 and t_mm >= 0
+    assert oracle.cpu_vector_lanes() in (4, 8, 16) and oracle.cpu_threads() >= 1

@@ -1,4 +1,4 @@
-"""The synthetic-weight quantisers (tests/quantizers.py) produce valid blocks whose dequantisation (by the
+"""The synthetic-weight quantisers (quantizers.py at the repository root) produce valid blocks whose dequantisation (by the
 oracle) is close to the input: checks layout packing against the pinned dequantisers."""
 import numpy as np
 import pytest
