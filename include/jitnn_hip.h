@@ -257,6 +257,35 @@ JITNN_HIP_API int jitnn_hip_llama_decode_dev(jitnn_hip_llama *m, const float *x_
 JITNN_HIP_API int jitnn_hip_llama_prefill(jitnn_hip_llama *m, const float *x_host, int pos0, int tokens, float *logits_host);
 JITNN_HIP_API int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0, int tokens, float *logits_dev, void *stream);
 
+/* ---- generation loop ------------------------------------------------------------------------------------------------ */
+
+/* Text generation from a GGUF model is jitnn-llm's Llm.generate (jitnn-llm/src/main/java/ai/beestream/jitnn/llm/Llm.java:64-93),
+ * which hands the work to the third-party jitllm engine: tokenizer, embedding lookup, the layers over a KV cache, greedy
+ * choice of the next token (temperature 0, Llm.java:74-76).  Here the model side of that loop runs on the quantised decode
+ * step above; the tokenizer stays with the host (jitnn_amd/llm.py reads it from the file's metadata). */
+
+/* Pairing of the rotary embedding: 0 (default) rotates pairs (i, i + head_dim / 2), 1 pairs (2i, 2i + 1) - the two forms of
+ * Rope (core/ops/Rope.java:126-150, `interleaved`).  GGUF files of the "llama" architecture hold q and k weights permuted
+ * for the interleaved form. */
+JITNN_HIP_API int jitnn_hip_llama_set_rope_interleaved(jitnn_hip_llama *m, int interleaved);
+
+/* The token embedding table [vocab, d_model] (token_embd.weight) in ggml type F32 (0), F16 (1) or a block format, copied
+ * to HBM as it is; a token's embedding is its row, dequantised bit-exactly (F.embedding on the dequantised table). */
+JITNN_HIP_API int jitnn_hip_llama_set_embedding(jitnn_hip_llama *m, int ggml_type, const void *table_host, long long nbytes);
+
+/* x [count, d_model] = embedding rows of `count` token ids in device memory. */
+JITNN_HIP_API int jitnn_hip_llama_embed_dev(jitnn_hip_llama *m, const int *tokens_dev, int count, float *x_dev, void *stream);
+
+/* *token_dev = index of the largest of the model's `vocab` logits (the lowest index among equal ones). */
+JITNN_HIP_API int jitnn_hip_llama_argmax_dev(jitnn_hip_llama *m, const float *logits_dev, int *token_dev, void *stream);
+
+/* Greedy continuation of a prompt: the prompt's tokens run through the layers at positions pos0 .. (one call, as
+ * jitnn_hip_llama_prefill), then tokens are chosen and fed back one at a time until max_new_tokens were produced or
+ * eos_token (-1: none) was chosen.  Each new token is written to out_tokens and, when on_token is not NULL, passed to it
+ * as soon as it exists.  Returns the number of tokens produced (>= 0) or a negative error code.  Synchronous. */
+JITNN_HIP_API int jitnn_hip_llama_generate(jitnn_hip_llama *m, const int *prompt, int prompt_tokens, int pos0, int max_new_tokens, int eos_token,
+                                           int *out_tokens, void (*on_token)(int token, void *user), void *user);
+
 #ifdef __cplusplus
 }
 #endif

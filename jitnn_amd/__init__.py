@@ -11,3 +11,5 @@ from .tensor import Tensor  # noqa: F401
 from .llama import LlamaDecoder  # noqa: F401
 from .gguf_file import GgufFile, GgufTensorInfo  # noqa: F401
 from ._lib import UnsupportedTypeError  # noqa: F401
+from .tokenizer import Tokenizer  # noqa: F401
+from .llm import Llm, ModelInfo  # noqa: F401

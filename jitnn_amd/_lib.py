@@ -72,6 +72,11 @@ def _bind() -> C.CDLL:
         "jitnn_hip_llama_decode": (i, [vp, vp, i, vp]),
         "jitnn_hip_llama_decode_dev": (i, [vp, vp, i, vp, vp]),
         "jitnn_hip_llama_prefill": (i, [vp, vp, i, i, vp]),
+        "jitnn_hip_llama_set_rope_interleaved": (i, [vp, i]),
+        "jitnn_hip_llama_set_embedding": (i, [vp, i, vp, ll]),
+        "jitnn_hip_llama_embed_dev": (i, [vp, vp, i, vp, vp]),
+        "jitnn_hip_llama_argmax_dev": (i, [vp, vp, vp, vp]),
+        "jitnn_hip_llama_generate": (i, [vp, vp, i, i, i, i, vp, vp, vp]),
         "jitnn_hip_llama_prefill_dev": (i, [vp, vp, i, i, vp, vp]),
     }
     for name, (res, args) in sig.items():

@@ -136,6 +136,16 @@ __global__ void __launch_bounds__(256) dequant_kernel(const uint8_t *__restrict_
     }
 }
 
+// Rows token[t] of a block-quantised table [vocab, k], dequantised bit-exactly into x [tokens, k] (the embedding lookup of
+// a model whose token table is quantised).  grid = tokens.
+template <int FMT>
+__global__ void __launch_bounds__(256) dequant_rows_kernel(const uint8_t *__restrict__ w, const int *__restrict__ tokens, float *__restrict__ x, int k) {
+    const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
+    const uint8_t *wr = w + (size_t)tokens[blockIdx.x] * rowbytes;
+    float4 *xr = reinterpret_cast<float4 *>(x + (size_t)blockIdx.x * k);
+    for (int f = threadIdx.x; f < (k >> 2); f += 256) xr[f] = dequant4<FMT>(wr, (size_t)f * 4);
+}
+
 // Plain GEMV for the formats without a tuned kernel: one wave per weight row, every lane dequantises quads of the row
 // with the bit-exact decoder and multiplies them with up to eight activation rows; a fixed DPP tree adds the lanes.
 //   y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]), b < rows <= 8.  grid: any; waves take rows round-robin.

@@ -24,8 +24,8 @@ __global__ void __launch_bounds__(256) rms_norm_kernel(const float *__restrict__
     for (int i = threadIdx.x; i < n; i += 256) y[i] = x[i] * is * w[i];
 }
 
-// One token's attention: rotary embedding of the new query and key heads in the rotate-half
-// form (pairs (i, i + D/2), interleaved = false; ops/Rope.java:126-150, F.ropeHeads), append of the rotated key and
+// One token's attention: rotary embedding of the new query and key heads - pairs (i, i + D/2), the reference's default
+// rotate-half form, or pairs (2i, 2i + 1) when `interleaved` (ops/Rope.java:126-150, F.ropeHeads) -, append of the rotated key and
 // the value to the cache, grouped-query attention over the s = pos + 1 cached positions
 // (F.scaledDotProductAttentionBTHD with F.repeatHeads, F.java:588-624; ops/FlashAttention.java:538-626: query head
 // h reads key/value head h / group).
@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
                                                            const float *__restrict__ v_raw, float *__restrict__ kcache,
                                                            float *__restrict__ vcache, const float *__restrict__ cosv,
                                                            const float *__restrict__ sinv, float *__restrict__ part, int heads, int kv_heads,
-                                                           int pos, float scale) {
+                                                           int pos, float scale, int interleaved) {
     constexpr int CH = AttCfg<D>::CH, HALF = D / 2, DQ = D / 4;
     __shared__ float Ks[CH][D + 1];
     __shared__ float Vs[CH][D];
@@ -61,9 +61,10 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
     for (int i = tid; i < group * HALF; i += 256) {
         const int h = i / HALF, p = i - h * HALF;
         const float *r = q_raw + (size_t)(g * group + h) * D;
-        const float a = r[p], b = r[p + HALF], cs = cp[p], sn = sp[p];
-        Qs[h][p] = a * cs - b * sn;
-        Qs[h][p + HALF] = a * sn + b * cs;
+        const int i0 = interleaved ? 2 * p : p, i1 = interleaved ? 2 * p + 1 : p + HALF;  // the pair rotated by angle p
+        const float a = r[i0], b = r[i1], cs = cp[p], sn = sp[p];
+        Qs[h][i0] = a * cs - b * sn;
+        Qs[h][i1] = a * sn + b * cs;
     }
     // ---- keys and values of the chunk: every load is issued before the first LDS write (one round trip to HBM);
     // the new token's row comes from k_raw / v_raw, rotated, and is appended to the cache on the way
@@ -87,11 +88,17 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
         if (j < nk && j0 + j == pos) {
             const size_t row = ((size_t)pos * kv_heads + g) * D;
             const float *r = k_raw + (size_t)g * D;
-            const int p = e < HALF ? e : e - HALF;
-            const float4 a = *reinterpret_cast<const float4 *>(r + p), b = *reinterpret_cast<const float4 *>(r + p + HALF);
-            const float4 cs = *reinterpret_cast<const float4 *>(cp + p), sn = *reinterpret_cast<const float4 *>(sp + p);
-            if (e < HALF) kreg[it] = make_float4(a.x * cs.x - b.x * sn.x, a.y * cs.y - b.y * sn.y, a.z * cs.z - b.z * sn.z, a.w * cs.w - b.w * sn.w);
-            else kreg[it] = make_float4(a.x * sn.x + b.x * cs.x, a.y * sn.y + b.y * cs.y, a.z * sn.z + b.z * cs.z, a.w * sn.w + b.w * cs.w);
+            if (interleaved) {  // pairs (2i, 2i + 1): values e, e + 1 turn by angle e / 2, values e + 2, e + 3 by angle e / 2 + 1
+                const float4 x = *reinterpret_cast<const float4 *>(r + e);
+                const float c0 = cp[e >> 1], s0 = sp[e >> 1], c1 = cp[(e >> 1) + 1], s1 = sp[(e >> 1) + 1];
+                kreg[it] = make_float4(x.x * c0 - x.y * s0, x.x * s0 + x.y * c0, x.z * c1 - x.w * s1, x.z * s1 + x.w * c1);
+            } else {
+                const int p = e < HALF ? e : e - HALF;
+                const float4 a = *reinterpret_cast<const float4 *>(r + p), b = *reinterpret_cast<const float4 *>(r + p + HALF);
+                const float4 cs = *reinterpret_cast<const float4 *>(cp + p), sn = *reinterpret_cast<const float4 *>(sp + p);
+                if (e < HALF) kreg[it] = make_float4(a.x * cs.x - b.x * sn.x, a.y * cs.y - b.y * sn.y, a.z * cs.z - b.z * sn.z, a.w * cs.w - b.w * sn.w);
+                else kreg[it] = make_float4(a.x * sn.x + b.x * cs.x, a.y * sn.y + b.y * cs.y, a.z * sn.z + b.z * cs.z, a.w * sn.w + b.w * cs.w);
+            }
             vreg[it] = *reinterpret_cast<const float4 *>(v_raw + (size_t)g * D + e);
             *reinterpret_cast<float4 *>(kcache + row + e) = kreg[it];
             *reinterpret_cast<float4 *>(vcache + row + e) = vreg[it];
@@ -216,23 +223,25 @@ __global__ void __launch_bounds__(256) rms_norm_rows_kernel(const float *__restr
 __global__ void __launch_bounds__(256) rope_append_rows_kernel(float *__restrict__ q, const float *__restrict__ k, const float *__restrict__ v,
                                                                 float *__restrict__ kcache, float *__restrict__ vcache,
                                                                 const float *__restrict__ cosv, const float *__restrict__ sinv, int heads, int kv_heads,
-                                                                int D, int pos0) {
+                                                                int D, int pos0, int interleaved) {
     const int t = blockIdx.x, pos = pos0 + t, half = D / 2;
     const float *cp = cosv + (size_t)pos * half, *sp = sinv + (size_t)pos * half;
     float *qt = q + (size_t)t * heads * D;
     for (int i = threadIdx.x; i < heads * half; i += 256) {
         const int h = i / half, p = i - h * half;
-        const float a = qt[h * D + p], b = qt[h * D + p + half], cs = cp[p], sn = sp[p];
-        qt[h * D + p] = a * cs - b * sn;
-        qt[h * D + p + half] = a * sn + b * cs;
+        const int i0 = h * D + (interleaved ? 2 * p : p), i1 = h * D + (interleaved ? 2 * p + 1 : p + half);
+        const float a = qt[i0], b = qt[i1], cs = cp[p], sn = sp[p];
+        qt[i0] = a * cs - b * sn;
+        qt[i1] = a * sn + b * cs;
     }
     const float *kt = k + (size_t)t * kv_heads * D, *vt = v + (size_t)t * kv_heads * D;
     float *kc = kcache + (size_t)pos * kv_heads * D, *vc = vcache + (size_t)pos * kv_heads * D;
     for (int i = threadIdx.x; i < kv_heads * half; i += 256) {
         const int h = i / half, p = i - h * half;
-        const float a = kt[h * D + p], b = kt[h * D + p + half], cs = cp[p], sn = sp[p];
-        kc[h * D + p] = a * cs - b * sn;
-        kc[h * D + p + half] = a * sn + b * cs;
+        const int i0 = h * D + (interleaved ? 2 * p : p), i1 = h * D + (interleaved ? 2 * p + 1 : p + half);
+        const float a = kt[i0], b = kt[i1], cs = cp[p], sn = sp[p];
+        kc[i0] = a * cs - b * sn;
+        kc[i1] = a * sn + b * cs;
     }
     for (int i = threadIdx.x; i < kv_heads * D; i += 256) vc[i] = vt[i];
 }
@@ -568,6 +577,54 @@ __global__ void __launch_bounds__(256) swiglu_kernel(const float *__restrict__ g
         const float v = gate[i];
         y[i] = (v / (1.f + __expf(-v))) * up[i];
     }
+}
+
+// Greedy choice of the next token: index of the largest logit, the lowest index among equals (NaN never wins).  One
+// workgroup of 1024 threads: a strided scan per thread, then wave and workgroup reductions on (value, index) pairs.
+__global__ void __launch_bounds__(1024) argmax_kernel(const float *__restrict__ x, int n, int *__restrict__ out) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const float v = x[i];
+        if (v > best || (v == best && i < idx)) {
+            best = v;
+            idx = i;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off);
+        const int oi = __shfl_xor(idx, off);
+        if (ov > best || (ov == best && oi < idx)) {
+            best = ov;
+            idx = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        bv[threadIdx.x >> 6] = best;
+        bi[threadIdx.x >> 6] = idx;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) {
+                best = bv[w];
+                idx = bi[w];
+            }
+        *out = idx == 0x7fffffff ? 0 : idx;
+    }
+}
+
+// x[t, :] = row token[t] of an unquantised embedding table [vocab, d] (F32: fmt 0, F16: fmt 1); block-quantised tables go
+// through dequant_rows_kernel.  grid = tokens.
+__global__ void __launch_bounds__(256) embed_plain_rows_kernel(const void *__restrict__ table, int fmt, const int *__restrict__ tokens, float *__restrict__ x,
+                                                                int d) {
+    const int t = blockIdx.x;
+    const size_t row = (size_t)tokens[t] * d;
+    for (int i = threadIdx.x; i < d; i += 256)
+        x[(size_t)t * d + i] = fmt == 0 ? reinterpret_cast<const float *>(table)[row + i]
+                                        : __half2float(reinterpret_cast<const __half *>(table)[row + i]);
 }
 
 }  // namespace jitnn

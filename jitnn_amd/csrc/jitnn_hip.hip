@@ -1150,6 +1150,12 @@ struct jitnn_hip_llama {
     // many-token (prefill) buffers, [pf_cap, ...] each, allocated by the first prefill call and grown when a longer one comes
     int pf_cap;
     float *pf[10];  // xn, q, k, v, att, xa, xb, gate, up, h
+    int rope_interleaved;  // 0: rotate-half pairs (i, i + D/2); 1: pairs (2i, 2i + 1)
+    // token embedding table [vocab, d] in ggml type embd_fmt (F32 = 0, F16 = 1 or a block format), owned
+    uint8_t *embd;
+    int embd_fmt;
+    int *tok_dev;   // [max_ctx] token ids of the generation loop (device)
+    int *tok_pin;   // one token id in pinned host memory
 };
 
 namespace {
@@ -1159,7 +1165,7 @@ void launch_attention(const jitnn_hip_llama *m, int layer, int pos, hipStream_t 
     const int chunks = (pos + 1 + AttCfg<D>::CH - 1) / AttCfg<D>::CH;
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
     hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->k, m->v, m->kc + lo, m->vc + lo, m->cosv, m->sinv,
-                       m->part, m->heads, m->kv, pos, 1.0f / sqrtf((float)D));
+                       m->part, m->heads, m->kv, pos, 1.0f / sqrtf((float)D), m->rope_interleaved);
     hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(m->heads), dim3(2 * D), 0, st, m->part, m->att, chunks);
 }
 
@@ -1369,6 +1375,9 @@ int jitnn_hip_llama_free(jitnn_hip_llama *m) {
         if (b) (void)hipFree(b);
     for (float *b : m->pf)
         if (b) (void)hipFree(b);
+    if (m->embd) (void)hipFree(m->embd);
+    if (m->tok_dev) (void)hipFree(m->tok_dev);
+    if (m->tok_pin) (void)hipHostFree(m->tok_pin);
     delete[] m->w;
     delete m;
     return JITNN_HIP_OK;
@@ -1506,7 +1515,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
             if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st)) return rc;
         }
         hipLaunchKernelGGL(rope_append_rows_kernel, dim3(T), dim3(256), 0, st, q, k, v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads, m->kv, m->hd,
-                           pos0);
+                           pos0, m->rope_interleaved);
         int arc;
         switch (m->hd) {
         case 64: arc = launch_attention_rows<64>(m, l, pos0, T, q, att, st); break;
@@ -1533,6 +1542,109 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
     }
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
+}
+
+// ---- generation loop: embedding lookup, greedy choice, prompt + token-by-token decode --------------------------------
+
+int jitnn_hip_llama_set_rope_interleaved(jitnn_hip_llama *m, int interleaved) {
+    if (!m) return fail(JITNN_HIP_EINVAL, "model is NULL");
+    m->rope_interleaved = interleaved != 0;
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_set_embedding(jitnn_hip_llama *m, int ggml_type, const void *table_host, long long nbytes) {
+    if (!m || !table_host) return fail(JITNN_HIP_EINVAL, "model or table is NULL");
+    long long need;
+    if (ggml_type == 0 || ggml_type == 1) {
+        need = (long long)m->vocab * m->d * (ggml_type == 0 ? 4 : 2);
+    } else {
+        need = jitnn_hip_weight_nbytes(ggml_type, m->vocab, m->d);
+        if (need < 0) return (int)need;
+    }
+    if (nbytes != need) return fail(JITNN_HIP_EINVAL, "an embedding table [%d, %d] of ggml type %d holds %lld bytes, got %lld", m->vocab, m->d, ggml_type, need, nbytes);
+    if (m->d % 4 != 0) return fail(JITNN_HIP_EUNSUPPORTED, "d_model %d is not a multiple of 4", m->d);
+    if (int rc = check_ready()) return rc;
+    if (m->embd) HIP_TRY(hipFree(m->embd));
+    m->embd = nullptr;
+    hipError_t e = hipMalloc(&m->embd, (size_t)nbytes);
+    if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipMalloc of %lld bytes: %s", nbytes, hipGetErrorString(e));
+    HIP_TRY(hipMemcpy(m->embd, table_host, (size_t)nbytes, hipMemcpyHostToDevice));
+    m->embd_fmt = ggml_type;
+    if (!m->tok_dev) HIP_TRY(hipMalloc(&m->tok_dev, (size_t)m->max_ctx * sizeof(int)));
+    if (!m->tok_pin) HIP_TRY(hipHostMalloc((void **)&m->tok_pin, sizeof(int), hipHostMallocDefault));
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_embed_dev(jitnn_hip_llama *m, const int *tokens_dev, int count, float *x_dev, void *stream) {
+    if (!m || !tokens_dev || !x_dev) return fail(JITNN_HIP_EINVAL, "NULL argument");
+    if (!m->embd) return fail(JITNN_HIP_EINVAL, "the model has no embedding table");
+    if (count < 1) return fail(JITNN_HIP_EINVAL, "%d tokens", count);
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)count), block(256);
+    switch (m->embd_fmt) {
+    case 0:
+    case 1: hipLaunchKernelGGL(embed_plain_rows_kernel, grid, block, 0, st, (const void *)m->embd, m->embd_fmt, tokens_dev, x_dev, m->d); break;
+    case F_Q4_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q4_1: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_1>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q5_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q5_1: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_1>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q8_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q8_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q2_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q2_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q3_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q3_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q4_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case F_Q5_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    default: hipLaunchKernelGGL(dequant_rows_kernel<F_Q6_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    }
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_argmax_dev(jitnn_hip_llama *m, const float *logits_dev, int *token_dev, void *stream) {
+    if (!m || !logits_dev || !token_dev) return fail(JITNN_HIP_EINVAL, "NULL argument");
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits_dev, m->vocab, token_dev);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+int jitnn_hip_llama_generate(jitnn_hip_llama *m, const int *prompt, int prompt_tokens, int pos0, int max_new_tokens, int eos_token, int *out_tokens,
+                             void (*on_token)(int token, void *user), void *user) {
+    if (int rc = check_model(m)) return rc;
+    if (!prompt || (!out_tokens && max_new_tokens > 0)) return fail(JITNN_HIP_EINVAL, "prompt or output is NULL");
+    if (!m->embd) return fail(JITNN_HIP_EINVAL, "the model has no embedding table");
+    if (prompt_tokens < 1 || max_new_tokens < 0 || pos0 < 0) return fail(JITNN_HIP_EINVAL, "%d prompt tokens from position %d, %d new tokens", prompt_tokens, pos0, max_new_tokens);
+    if ((long long)pos0 + prompt_tokens + max_new_tokens > (long long)m->max_ctx + 1)
+        return fail(JITNN_HIP_EINVAL, "positions %d .. %d do not fit a cache of %d", pos0, pos0 + prompt_tokens + max_new_tokens - 2, m->max_ctx);
+    for (int i = 0; i < prompt_tokens; ++i)
+        if (prompt[i] < 0 || prompt[i] >= m->vocab) return fail(JITNN_HIP_EINVAL, "token %d of a vocabulary of %d", prompt[i], m->vocab);
+    if (max_new_tokens == 0) return 0;
+    if (int rc = stage_reserve(0, (size_t)prompt_tokens * m->d * 4)) return rc;
+    HostStage &hs = g_thread.stage;
+    hipStream_t st = hs.stream;
+    // the prompt: embeddings of all tokens, one pass through the layers, logits of the last token
+    HIP_TRY(hipMemcpyAsync(m->tok_dev, prompt, (size_t)prompt_tokens * sizeof(int), hipMemcpyHostToDevice, st));
+    float *x = (float *)hs.dev;
+    if (int rc = jitnn_hip_llama_embed_dev(m, m->tok_dev, prompt_tokens, x, st)) return rc;
+    if (prompt_tokens == 1) {
+        if (int rc = jitnn_hip_llama_decode_dev(m, x, pos0, m->logits, st)) return rc;
+    } else {
+        if (int rc = jitnn_hip_llama_prefill_dev(m, x, pos0, prompt_tokens, m->logits, st)) return rc;
+    }
+    int produced = 0;
+    for (int pos = pos0 + prompt_tokens;; ++pos) {
+        // greedy: the largest logit (Llm.generate runs at temperature 0, jitnn-llm/.../llm/Llm.java:74-76)
+        if (int rc = jitnn_hip_llama_argmax_dev(m, m->logits, m->tok_dev, st)) return rc;
+        HIP_TRY(hipMemcpyAsync(m->tok_pin, m->tok_dev, sizeof(int), hipMemcpyDeviceToHost, st));
+        HIP_TRY(hipStreamSynchronize(st));
+        const int tok = *m->tok_pin;
+        if (tok == eos_token) break;
+        out_tokens[produced++] = tok;
+        if (on_token) on_token(tok, user);
+        if (produced == max_new_tokens) break;
+        if (int rc = jitnn_hip_llama_embed_dev(m, m->tok_dev, 1, m->xin, st)) return rc;
+        if (int rc = jitnn_hip_llama_decode_dev(m, m->xin, pos, m->logits, st)) return rc;
+    }
+    HIP_TRY(hipStreamSynchronize(st));
+    return produced;
 }
 
 int jitnn_hip_llama_prefill(jitnn_hip_llama *m, const float *x_host, int pos0, int tokens, float *logits_host) {

@@ -83,6 +83,63 @@ class LlamaDecoder:
         _lib.check(_lib.lib.jitnn_hip_llama_decode_dev(self._h, C.c_void_p(x_ptr), pos, C.c_void_p(logits_ptr), C.c_void_p(stream_ptr)),
                    "jitnn_hip_llama_decode_dev")
 
+    def set_rope_interleaved(self, on: bool) -> None:
+        """Rotary pairs (2i, 2i + 1) instead of the default (i, i + head_dim / 2): the two forms of Rope (core/ops/Rope.java:126-150)."""
+        _lib.check(_lib.lib.jitnn_hip_llama_set_rope_interleaved(self._h, 1 if on else 0), "jitnn_hip_llama_set_rope_interleaved")
+
+    def set_embedding(self, ggml_type: int, table) -> None:
+        """The token embedding table [vocab, d_model] as raw bytes of ggml type F32 (0), F16 (1) or a block format."""
+        raw = np.ascontiguousarray(table).view(np.uint8).reshape(-1)
+        _lib.check(_lib.lib.jitnn_hip_llama_set_embedding(self._h, ggml_type, _p(raw), raw.size), "jitnn_hip_llama_set_embedding")
+
+    def embed(self, tokens) -> np.ndarray:
+        """Embedding rows [count, d_model] of token ids (through device memory; for tests)."""
+        ids = np.ascontiguousarray(tokens, dtype=np.int32).reshape(-1)
+        n, d = ids.size, self.cfg["d_model"]
+        dev_ids, dev_x = C.c_void_p(), C.c_void_p()
+        _lib.check(_lib.lib.jitnn_hip_malloc(ids.nbytes, C.byref(dev_ids)), "jitnn_hip_malloc")
+        _lib.check(_lib.lib.jitnn_hip_malloc(n * d * 4, C.byref(dev_x)), "jitnn_hip_malloc")
+        try:
+            _lib.check(_lib.lib.jitnn_hip_memcpy_h2d(dev_ids, _p(ids), ids.nbytes), "jitnn_hip_memcpy_h2d")
+            _lib.check(_lib.lib.jitnn_hip_llama_embed_dev(self._h, dev_ids, n, dev_x, None), "jitnn_hip_llama_embed_dev")
+            x = np.empty((n, d), dtype=np.float32)
+            _lib.check(_lib.lib.jitnn_hip_memcpy_d2h(_p(x), dev_x, x.nbytes), "jitnn_hip_memcpy_d2h")
+            return x
+        finally:
+            _lib.lib.jitnn_hip_free(dev_ids)
+            _lib.lib.jitnn_hip_free(dev_x)
+
+    def argmax(self, logits) -> int:
+        """Index of the largest logit as the device kernel of the generation loop picks it (for tests)."""
+        a = np.ascontiguousarray(logits, dtype=np.float32).reshape(-1)
+        if a.size != self.cfg["vocab"]:
+            raise ValueError(f"{a.size} logits for a vocabulary of {self.cfg['vocab']}")
+        dev_l, dev_t = C.c_void_p(), C.c_void_p()
+        _lib.check(_lib.lib.jitnn_hip_malloc(a.nbytes, C.byref(dev_l)), "jitnn_hip_malloc")
+        _lib.check(_lib.lib.jitnn_hip_malloc(4, C.byref(dev_t)), "jitnn_hip_malloc")
+        try:
+            _lib.check(_lib.lib.jitnn_hip_memcpy_h2d(dev_l, _p(a), a.nbytes), "jitnn_hip_memcpy_h2d")
+            _lib.check(_lib.lib.jitnn_hip_llama_argmax_dev(self._h, dev_l, dev_t, None), "jitnn_hip_llama_argmax_dev")
+            t = np.empty(1, dtype=np.int32)
+            _lib.check(_lib.lib.jitnn_hip_memcpy_d2h(_p(t), dev_t, 4), "jitnn_hip_memcpy_d2h")
+            return int(t[0])
+        finally:
+            _lib.lib.jitnn_hip_free(dev_l)
+            _lib.lib.jitnn_hip_free(dev_t)
+
+    def generate(self, prompt_ids, max_new_tokens: int, eos_token: int = -1, on_token=None, pos0: int = 0) -> list:
+        """Greedy continuation of the prompt's token ids (jitnn_hip_llama_generate); on_token(token, None) is called for every
+        new token as soon as it exists."""
+        ids = np.ascontiguousarray(prompt_ids, dtype=np.int32).reshape(-1)
+        out = np.empty(max(max_new_tokens, 1), dtype=np.int32)
+        cb_type = C.CFUNCTYPE(None, C.c_int, C.c_void_p)
+        cb = cb_type(on_token) if on_token is not None else None
+        n = _lib.lib.jitnn_hip_llama_generate(self._h, _p(ids), ids.size, pos0, max_new_tokens, eos_token, _p(out),
+                                              C.cast(cb, C.c_void_p) if cb is not None else None, None)
+        if n < 0:
+            _lib.check(n, "jitnn_hip_llama_generate")
+        return [int(t) for t in out[:n]]
+
     def prefill(self, x, pos0: int = 0, logits: bool = True):
         """Runs the tokens whose embeddings are the rows of x [tokens, d_model] through the stack at positions
         pos0 .. pos0 + tokens - 1 (causal attention over the cache and one another), appends their keys and values,

@@ -10,10 +10,11 @@ from oracle import oracle
 SLOTS = ["attn_q", "attn_k", "attn_v", "attn_o", "ffn_gate", "ffn_up", "ffn_down"]
 
 
-def decode_ref(cfg, layers, out_norm, out_w, kcache, vcache, x, pos, threads: int = 1):
+def decode_ref(cfg, layers, out_norm, out_w, kcache, vcache, x, pos, threads: int = 1, rope_interleaved: bool = False):
     """layers: list of dicts {slot: (ggml id, raw, n, k)} + 'attn_norm', 'ffn_norm'; out_w = (id, raw, n, k);
     kcache/vcache [L, ctx, kv, hd] are updated in place at pos.  Returns logits [vocab].
-    threads > 1 shares the output rows of every linear out over host threads (bit-identical results)."""
+    threads > 1 shares the output rows of every linear out over host threads (bit-identical results); rope_interleaved
+    selects Rope's pairs (2i, 2i + 1) instead of (i, i + D/2) (ops/Rope.java:126-150)."""
     heads, kv, hd = cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
     eps, theta = cfg["rms_eps"], np.float32(cfg["rope_theta"])
 
@@ -26,8 +27,8 @@ def decode_ref(cfg, layers, out_norm, out_w, kcache, vcache, x, pos, threads: in
     x = np.asarray(x, dtype=np.float32)
     for li, L in enumerate(layers):
         n = oracle.rms_norm(x, L["attn_norm"], eps)
-        q = oracle.rope(lin(L["attn_q"], n).reshape(1, heads, hd), theta, pos, False, True)[0]
-        k = oracle.rope(lin(L["attn_k"], n).reshape(1, kv, hd), theta, pos, False, True)[0]
+        q = oracle.rope(lin(L["attn_q"], n).reshape(1, heads, hd), theta, pos, rope_interleaved, True)[0]
+        k = oracle.rope(lin(L["attn_k"], n).reshape(1, kv, hd), theta, pos, rope_interleaved, True)[0]
         v = lin(L["attn_v"], n).reshape(kv, hd)
         kcache[li, pos], vcache[li, pos] = k, v
         att = oracle.attention_decode(q, kcache[li, :pos + 1], vcache[li, :pos + 1])

@@ -1,0 +1,225 @@
+"""The generation loop (jitnn_amd.Llm over jitnn_hip_llama_generate) - the reference's jitnn-llm Llm.generate, whose
+arithmetic lives in the third-party jitllm engine, so parity here is behavioural, as in the reference's own test
+(jitnn-llm/src/test/java/ai/beestream/jitnn/llm/LlmAccelTest.java:44-60: the answer is not blank, greedy generation is
+deterministic, the streamed pieces add up to the text) - plus what the CPU oracle can pin on a model file the test writes
+itself: every embedding row bit for bit, and at every step the chosen token is the arg-max of the oracle's logits."""
+import numpy as np
+import pytest
+import torch
+
+import quantizers
+from decode_oracle import SLOTS, decode_ref
+from gguf_writer import write_gguf
+from helpers import GGML_ID
+
+WORDS = ["the", "cat", "sat", "on", "mat", "dog", "ran", "to", "park", "and", "a", "bird", "sang", "in", "tree", "hello", "world"]
+
+
+def spm_vocab():
+    """<unk>, <s>, </s>, the 256 byte tokens, single characters, then word pieces whose scores grow with their length."""
+    toks = ["<unk>", "<s>", "</s>"] + [f"<0x{b:02X}>" for b in range(256)]
+    types = [2, 3, 3] + [6] * 256
+    scores = [0.0] * len(toks)
+    pieces = ["▁"] + [chr(c) for c in range(ord("a"), ord("z") + 1)]
+    for w in WORDS:
+        for n in range(2, len(w) + 1):
+            pieces.append(w[:n])
+        pieces.append("▁" + w)
+        for n in range(1, len(w)):
+            pieces.append("▁" + w[:n])
+    seen = set(toks)
+    for p in pieces:
+        if p not in seen:
+            seen.add(p)
+            toks.append(p)
+            types.append(1)
+            scores.append(float(len(p)) - 10.0)
+    return toks, scores, types
+
+
+def bpe_vocab():
+    from jitnn_amd.tokenizer import _byte_to_unicode
+    b2u = _byte_to_unicode()
+    toks = [b2u[b] for b in range(256)]
+    merges = []
+    sp = b2u[ord(" ")]
+    for w in WORDS:
+        for lead in (sp, ""):  # the merges that start at the space come first, so that " word" wins over "word"
+            cur = (lead + w[0]) if lead else w[0]
+            if lead and cur not in toks:
+                merges.append(f"{lead} {w[0]}")
+                toks.append(cur)
+            for ch in w[1:]:
+                if cur + ch not in toks:
+                    merges.append(f"{cur} {ch}")
+                    toks.append(cur + ch)
+                cur += ch
+    toks += ["<|begin|>", "<|end|>"]
+    types = [1] * (len(toks) - 2) + [3, 3]
+    return toks, merges, types
+
+
+def test_spm_tokenizer_round_trip_and_byte_fallback():
+    from jitnn_amd.tokenizer import StreamDecoder, Tokenizer
+    toks, scores, types = spm_vocab()
+    tk = Tokenizer("llama", toks, scores, types, None, bos=1, eos=2, add_bos=True)
+    ids = tk.encode("the cat sat on the mat")
+    assert ids[0] == 1 and [toks[i] for i in ids[1:]] == ["▁the", "▁cat", "▁sat", "▁on", "▁the", "▁mat"]
+    assert tk.decode(ids, strip_leading_space=True) == "the cat sat on the mat"
+    text = "a bird sang: ¡olé! 東京 42"
+    ids = tk.encode(text, add_bos=False)
+    assert any(types[i] == 6 for i in ids)          # characters outside the vocabulary went to byte tokens
+    assert tk.decode(ids, strip_leading_space=True) == text
+    sd = StreamDecoder(tk)
+    pieces = [sd.push(i) for i in ids] + [sd.flush()]
+    assert "".join(pieces) == tk.decode(ids)         # a character split over byte tokens is held back until whole
+    assert tk.encode("", add_bos=False) == []
+
+
+def test_bpe_tokenizer_round_trip():
+    from jitnn_amd.tokenizer import Tokenizer
+    toks, merges, types = bpe_vocab()
+    tk = Tokenizer("gpt2", toks, None, types, merges, bos=len(toks) - 2, eos=len(toks) - 1, add_bos=False)
+    ids = tk.encode("hello world and a bird")
+    assert [tk.decode([i]) for i in ids] == ["hello", " world", " and", " a", " bird"]
+    text = "the dog ran to the park, 3 times! ¿sí?"
+    assert tk.decode(tk.encode(text)) == text
+    assert tk.decode([len(toks) - 1]) == ""          # control tokens print nothing
+
+
+# ------------------------------------------------------------------------------------------------ on the GPU
+
+CFG = dict(layers=2, d_model=256, heads=4, kv_heads=2, head_dim=64, ffn=512, max_ctx=64, rms_eps=1e-5, rope_theta=10000.0)
+MIX = {"attn_q": "Q4_K", "attn_k": "Q4_K", "attn_v": "Q6_K", "attn_o": "Q4_K", "ffn_gate": "Q4_K", "ffn_up": "Q4_K", "ffn_down": "Q6_K"}
+GGUF_NAME = {"attn_q": "attn_q", "attn_k": "attn_k", "attn_v": "attn_v", "attn_o": "attn_output", "ffn_gate": "ffn_gate", "ffn_up": "ffn_up",
+             "ffn_down": "ffn_down"}
+
+
+def write_model(path, arch, seed, embd_fmt="Q8_0", tied=False):
+    """A random Llama-style model with an SPM vocabulary; returns what the oracle needs."""
+    toks, scores, types = spm_vocab()
+    vocab = len(toks)
+    g = torch.Generator().manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    d, qd, kd, ffn = CFG["d_model"], CFG["heads"] * CFG["head_dim"], CFG["kv_heads"] * CFG["head_dim"], CFG["ffn"]
+    shapes = {"attn_q": (qd, d), "attn_k": (kd, d), "attn_v": (kd, d), "attn_o": (d, qd), "ffn_gate": (ffn, d), "ffn_up": (ffn, d), "ffn_down": (d, ffn)}
+    tensors, layers = [], []
+    emb_w = torch.randn(vocab, d, generator=g)
+    if embd_fmt == "F32":
+        emb_raw = emb_w.numpy().astype(np.float32)
+    elif embd_fmt == "F16":
+        emb_raw = emb_w.numpy().astype(np.float16)
+    else:
+        emb_raw = quantizers.quantize(embd_fmt, emb_w).numpy()
+    emb_id = {"F32": 0, "F16": 1}.get(embd_fmt, GGML_ID.get(embd_fmt))
+    tensors.append(("token_embd.weight", (vocab, d), emb_id, emb_raw))
+    for l in range(CFG["layers"]):
+        L = {}
+        for slot in SLOTS:
+            n, k = shapes[slot]
+            raw = quantizers.quantize(MIX[slot], torch.randn(n, k, generator=g) * 0.08).numpy()
+            L[slot] = (GGML_ID[MIX[slot]], raw, n, k)
+            tensors.append((f"blk.{l}.{GGUF_NAME[slot]}.weight", (n, k), GGML_ID[MIX[slot]], raw))
+        for nm in ("attn_norm", "ffn_norm"):
+            L[nm] = (1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+            tensors.append((f"blk.{l}.{nm}.weight", (d,), 0, L[nm]))
+        layers.append(L)
+    out_norm = (1.0 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    tensors.append(("output_norm.weight", (d,), 0, out_norm))
+    if tied:
+        out_w = (emb_id, emb_raw, vocab, d)
+    else:
+        raw = quantizers.quantize("Q6_K", torch.randn(vocab, d, generator=g) * 0.08).numpy()
+        out_w = (GGML_ID["Q6_K"], raw, vocab, d)
+        tensors.append(("output.weight", (vocab, d), GGML_ID["Q6_K"], raw))
+    meta = {"general.architecture": arch, "general.name": "tiny test model", f"{arch}.block_count": CFG["layers"], f"{arch}.embedding_length": d,
+            f"{arch}.attention.head_count": CFG["heads"], f"{arch}.attention.head_count_kv": CFG["kv_heads"], f"{arch}.feed_forward_length": ffn,
+            f"{arch}.attention.layer_norm_rms_epsilon": float(CFG["rms_eps"]), f"{arch}.rope.freq_base": float(CFG["rope_theta"]),
+            f"{arch}.context_length": CFG["max_ctx"], "tokenizer.ggml.model": "llama", "tokenizer.ggml.tokens": toks,
+            "tokenizer.ggml.scores": [float(s) for s in scores], "tokenizer.ggml.token_type": [int(t) for t in types],
+            "tokenizer.ggml.bos_token_id": 1, "tokenizer.ggml.eos_token_id": 2, "tokenizer.ggml.add_bos_token": True}
+    write_gguf(path, meta, tensors)
+    return dict(layers=layers, out_norm=out_norm, out_w=out_w, emb=(emb_id, emb_raw), vocab=vocab)
+
+
+def embedding_rows(emb, vocab, d):
+    from oracle import oracle
+    tid, raw = emb
+    if tid == 0:
+        return np.asarray(raw, dtype=np.float32).reshape(vocab, d)
+    if tid == 1:
+        return np.asarray(raw).view(np.float16).reshape(vocab, d).astype(np.float32)
+    return oracle.dequantize(tid, raw, vocab * d).reshape(vocab, d)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("arch,embd_fmt,tied", [("llama", "Q8_0", False), ("testarch", "Q4_K", False), ("llama", "F16", False), ("llama", "Q6_K", True)])
+def test_generate_from_a_gguf_file(tmp_path, arch, embd_fmt, tied):
+    import jitnn_amd
+    path = tmp_path / "tiny.gguf"
+    ref = write_model(path, arch, 7, embd_fmt, tied)
+    cfg = dict(CFG, vocab=ref["vocab"])
+    with jitnn_amd.Llm.load(path) as llm:
+        info = llm.info()
+        assert (info.architecture, info.layers, info.d_model, info.heads, info.kv_heads, info.vocab) == (arch, 2, 256, 4, 2, ref["vocab"])
+        # LlmAccelTest.weightsAreJitnnTensorsToo: the file's weights are tensors of this library too
+        wq = llm.gguf().tensor("blk.0.attn_q.weight")
+        assert wq.dim(1) == llm.gguf().integer(f"{arch}.embedding_length") and np.isfinite(wq.to_float_array()[0])
+        # embedding lookup: every row, bit for bit
+        table = embedding_rows(ref["emb"], ref["vocab"], 256)
+        got = llm.model().embed(np.arange(ref["vocab"]))
+        assert np.array_equal(got.view(np.uint32), table.view(np.uint32))
+        # LlmAccelTest.generatesGreedily: not blank, deterministic, streamed pieces add up
+        streamed = []
+        prompt = "the cat sat on the"
+        a = llm.generate(prompt, 12, streamed.append)
+        b = llm.generate(prompt, 12)
+        assert a.strip() != "" and a == b and a == "".join(streamed)
+        # token level against the oracle: the prompt token by token, then every chosen token is the arg-max of the oracle's logits
+        ids = llm.tokenizer().encode(prompt)
+        out = llm.generate_tokens(ids, 12)
+        assert llm.tokenizer().decode(out) == a or llm.tokenizer().decode(out).startswith(a)
+        kc = np.zeros((2, CFG["max_ctx"], 2, 64), dtype=np.float32)
+        vc = np.zeros_like(kc)
+        inter = arch == "llama"
+        logits = None
+        for pos, t in enumerate(ids):
+            logits = decode_ref(cfg, ref["layers"], ref["out_norm"], ref["out_w"], kc, vc, table[t], pos, rope_interleaved=inter)
+        pos = len(ids)
+        for step, t in enumerate(out):
+            best = int(np.argmax(logits))
+            margin = float(logits[best] - logits[t]) / max(float(np.abs(logits).max()), 1e-6)
+            assert t == best or margin <= 1e-4, (step, t, best, margin)  # (a different token only on a tie within the GEMV bar)
+            if step + 1 < len(out):
+                logits = decode_ref(cfg, ref["layers"], ref["out_norm"], ref["out_w"], kc, vc, table[t], pos, rope_interleaved=inter)
+                pos += 1
+        # stops at the end-of-sequence token: make it the most likely continuation by asking for it as the eos id
+        first = out[0]
+        assert llm.model().generate(ids, 5, eos_token=first) == []
+
+
+@pytest.mark.gpu
+def test_argmax_kernel_ties_and_nan():
+    import jitnn_amd
+    dec = jitnn_amd.LlamaDecoder(1, 256, 4, 2, 64, 512, 5000, 8)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal(5000).astype(np.float32)
+    assert dec.argmax(x) == int(np.argmax(x))
+    x[[77, 4091, 1300]] = 9.0          # equal maxima: the lowest index wins, as a sequential scan would choose
+    assert dec.argmax(x) == 77
+    x[5] = np.nan                       # NaN never wins
+    assert dec.argmax(x) == 77
+    x[:] = -np.inf
+    x[4999] = -1e30
+    assert dec.argmax(x) == 4999
+    dec.close()
+
+
+def test_generate_argument_checks():
+    pytest.importorskip("torch")
+    import jitnn_amd
+    from jitnn_amd import _lib
+    assert _lib.lib.jitnn_hip_llama_generate(None, None, 1, 0, 1, -1, None, None, None) == _lib.EINVAL
+    assert _lib.lib.jitnn_hip_llama_set_embedding(None, 0, None, 0) == _lib.EINVAL
+    with pytest.raises(ValueError):
+        jitnn_amd.Tokenizer("wordpiece", ["a"])
