@@ -1,0 +1,263 @@
+// 2..64 activation rows against raw GGUF blocks in ONE pass over the weights, on the matrix cores, at FP32-grade accuracy.
+//
+// gemv_mfma_kernel (gemv_mfma.h) takes at most eight rows per pass and spends most of its instructions on things that
+// do not depend on the weights' bytes: it rebuilds the activation operands in every workgroup and applies the block
+// scales to every 4 x 16 block sum in FP32.  This kernel family moves both out of the way:
+//   * rows_prepare_kernel builds the activation operands once per call: per group of eight rows and 256-value column of
+//     K, the rows scaled by a power of two (from the column's largest magnitude per row) and split into two FP16 parts,
+//     x 2^e = hi + lo, written in matrix-core operand order (hi and lo of a row in neighbouring operand rows, so that
+//     their block sums meet in one lane) together with the column's eight block sums of x and the inverse scales.  The
+//     main kernel streams them from L2: one 16-byte load per lane and operand.
+//   * the block scales are folded into the weight operand where that is exact: a Q4_K / Q5_K quant times its 6-bit
+//     scale is an integer below 2048, so sc * q is an FP16 value without rounding, and the matrix core accumulates the
+//     eight sub-blocks of a super-block in one FP32 chain; only the super-block's d and dmin (and the activation scale)
+//     meet the sums in FP32, once per 16 x 256 tile instead of once per block.  The conversion costs what the plain one
+//     did: (1024 + q) * sc - 1024 * sc is one packed FMA on the pattern 0x6400 | q.
+// A workgroup of eight waves owns tiles of 16 weight rows; wave w walks the 256-value columns w, w + 8, ... of K for the
+// workgroup's tiles, T tiles at a time: every lane fetches the bytes of its own weight row straight from global memory
+// (the four 8-byte pieces of a row's 128 quant bytes share a cache line, so the line is used whole), turns them into
+// operands once, and runs them against every group of eight activation rows.  Partial sums live in LDS per lane (the
+// group index is a run-time value) and are added across the eight waves in wave order at the end of a tile batch: a
+// fixed summation order, no atomics.
+#pragma once
+#include "common.h"
+#include "gemv_mfma.h"
+
+namespace jitnn {
+
+constexpr int GR_WAVES = 8, GR_THREADS = GR_WAVES * 64;
+constexpr int GR_MAX_GROUPS = 8;            // groups of eight activation rows: up to 64 rows
+constexpr int GR_OP_HALVES = 9 * 512;       // per (group, column): eight sub-block operands and the block-sum operand, 64 lanes x 8 halves each
+constexpr int GR_T = 2;                 // weight tiles a wave holds as operands at a time
+
+__host__ __device__ constexpr size_t gemv_rows_ops_bytes(int groups, int k) { return (size_t)groups * (k / 256) * GR_OP_HALVES * 2; }
+__host__ __device__ constexpr size_t gemv_rows_inv_bytes(int groups, int k) { return (size_t)groups * (k / 256) * 8 * sizeof(float); }
+__host__ __device__ constexpr size_t gemv_rows_lds_bytes() { return (size_t)GR_T * GR_MAX_GROUPS * GR_THREADS * sizeof(float2); }
+
+// One wave per (group g = blockIdx.y, column c = blockIdx.x): x [rows, k] -> operands.
+// Operand s < 8 (sub-block s of the column): lane m + 16 kq holds, for operand row m = 2 b + part (b = activation row of
+// the group, part 0 = hi, 1 = lo), the eight values 8 kq .. 8 kq + 7 of the sub-block in the order 0 2 1 3 4 6 5 7 - the
+// order in which the weight decoders emit the bytes of a dword.  Operand 8: rows as above, slot j of the lanes kq = 0 =
+// sum of sub-block j of the scaled row / 64, the other lanes zero.
+__global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restrict__ x, _Float16 *__restrict__ ops, float *__restrict__ inv, int rows,
+                                                           int k) {
+    const int lane = threadIdx.x, b = lane >> 3, part = lane & 7;
+    const int c = blockIdx.x, g = blockIdx.y, ncol = k >> 8;
+    const int row = g * 8 + b;
+    const bool have = row < rows;
+    const float *xp = x + (size_t)(have ? row : 0) * k + (size_t)c * 256 + 4 * part;
+    float4 v[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) v[t] = *reinterpret_cast<const float4 *>(xp + 32 * t);
+    float amax = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[t].x), fabsf(v[t].y)), fmaxf(fabsf(v[t].z), fabsf(v[t].w))));
+    amax = group_max8(amax);
+    float scale = 1.f;
+    if (amax > 0.f && amax < 3.0e38f) {
+        int e;
+        frexpf(amax, &e);             // amax = f * 2^e, f in [0.5, 1)
+        scale = ldexpf(1.f, 14 - e);  // largest scaled magnitude in [2^13, 2^14)
+    }
+    const float myinv = 1.f / scale;
+    if (!have) scale = 0.f;
+    uint8_t *base = reinterpret_cast<uint8_t *>(ops + ((size_t)g * ncol + c) * GR_OP_HALVES);
+    const int kq = part >> 1, h = part & 1;  // the quad `part` of a sub-block: lane group and half of its eight slots
+    float sm = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const float a0 = v[t].x * scale, a1 = v[t].z * scale, a2 = v[t].y * scale, a3 = v[t].w * scale;
+        const float bs = group_sum<8>((a0 + a1) + (a2 + a3));  // sub-block t of row b: its eight quads sit in the eight lanes of b
+        sm = part == t ? bs : sm;
+        const h2raw h01 = __builtin_amdgcn_cvt_pkrtz(a0, a1), h23 = __builtin_amdgcn_cvt_pkrtz(a2, a3);
+        const h2raw l01 = __builtin_amdgcn_cvt_pkrtz(a0 - (float)h01.x, a1 - (float)h01.y);
+        const h2raw l23 = __builtin_amdgcn_cvt_pkrtz(a2 - (float)h23.x, a3 - (float)h23.y);
+        *reinterpret_cast<u32x2 *>(base + t * 1024 + (2 * b + 16 * kq) * 16 + 8 * h) = u32x2{__builtin_bit_cast(uint32_t, h01), __builtin_bit_cast(uint32_t, h23)};
+        *reinterpret_cast<u32x2 *>(base + t * 1024 + (2 * b + 1 + 16 * kq) * 16 + 8 * h) = u32x2{__builtin_bit_cast(uint32_t, l01), __builtin_bit_cast(uint32_t, l23)};
+    }
+    // the block sums: scaled by 1/64 (a sum of 32 values below 2^14 stays below 2^13), hi / lo like the values
+    sm *= 0.015625f;
+    const _Float16 shi = (_Float16)sm, slo = (_Float16)(sm - (float)shi);
+    _Float16 *sop = reinterpret_cast<_Float16 *>(base + 8 * 1024);
+    if (lane >= 16) *reinterpret_cast<u32x4 *>(base + 8 * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
+    sop[(2 * b) * 8 + part] = shi;
+    sop[(2 * b + 1) * 8 + part] = slo;
+    if (part == 0) inv[((size_t)g * ncol + c) * 8 + b] = myinv;
+}
+
+// Per format: the bytes a lane (weight row n = lane & 15 of the tile, lane group kq = lane >> 4) fetches of a 256-value
+// column of its row, and their operands with the block scales folded in.
+template <int FMT>
+struct RTile;
+
+__device__ __forceinline__ f16x2 h2fma(uint32_t bits, f16x2 mul, f16x2 add) { return __builtin_elementwise_fma(as_h2(bits), mul, add); }
+
+template <>
+struct RTile<F_Q4_K> {
+    static constexpr int BYTES = 144;
+    struct Raw {
+        u32x4 h;
+        u32x2 q[4];
+    };
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *p, int kq) {
+        r.h = ld128<16>(p);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) r.q[c] = *reinterpret_cast<const u32x2 *>(p + 16 + 32 * c + 8 * kq);
+    }
+    // B[s]: sc_s * q of sub-block s; Bm: the eight mins in the first eight K slots; d, dmin of the super-block
+    __device__ static __forceinline__ void decode(const Raw &r, f16x8 (&B)[8], f16x8 &Bm, float &d, float &dmin) {
+        const K4Scales k = k4_scales(r.h);
+        d = k.d;
+        dmin = k.dmin;
+        const uint32_t mg = magic1024();
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const f16x2 ml = splat2(k.sc[2 * c]), al = splat2(-1024.f * k.sc[2 * c]);
+            const f16x2 mh = splat2(0.0625f * k.sc[2 * c + 1]), ah = splat2(-64.f * k.sc[2 * c + 1]);
+            const uint32_t w0 = r.q[c].x, w1 = r.q[c].y, s0 = w0 >> 8, s1 = w1 >> 8;
+            B[2 * c] = cat8(h2fma((w0 & 0x000f000fu) | mg, ml, al), h2fma((s0 & 0x000f000fu) | mg, ml, al), h2fma((w1 & 0x000f000fu) | mg, ml, al),
+                            h2fma((s1 & 0x000f000fu) | mg, ml, al));
+            B[2 * c + 1] = cat8(h2fma((w0 & 0x00f000f0u) | mg, mh, ah), h2fma((s0 & 0x00f000f0u) | mg, mh, ah), h2fma((w1 & 0x00f000f0u) | mg, mh, ah),
+                                h2fma((s1 & 0x00f000f0u) | mg, mh, ah));
+        }
+        Bm = cat8(bytes2(k.mnA, 0), bytes2(k.mnA, 16), bytes2(k.mnB, 0), bytes2(k.mnB, 16));
+    }
+};
+
+template <>
+struct RTile<F_Q5_K> {
+    static constexpr int BYTES = 176;
+    struct Raw {
+        u32x4 h;
+        u32x2 qh;
+        u32x2 q[4];
+    };
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *p, int kq) {
+        r.h = ld128<16>(p);
+        r.qh = *reinterpret_cast<const u32x2 *>(p + 16 + 8 * kq);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) r.q[c] = *reinterpret_cast<const u32x2 *>(p + 48 + 32 * c + 8 * kq);
+    }
+    __device__ static __forceinline__ void decode(const Raw &r, f16x8 (&B)[8], f16x8 &Bm, float &d, float &dmin) {
+        const K4Scales k = k4_scales(r.h);
+        d = k.d;
+        dmin = k.dmin;
+        const uint32_t mg = magic1024();
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const f16x2 ml = splat2(k.sc[2 * c]), al = splat2(-1024.f * k.sc[2 * c]);
+            const f16x2 mh = splat2(0.0625f * k.sc[2 * c + 1]), ah = splat2(-64.f * k.sc[2 * c + 1]);
+            f16x2 lo[4], hi[4];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const uint32_t w = t ? r.q[c].y : r.q[c].x, qh = t ? r.qh.y : r.qh.x, s = w >> 8, qs = qh >> 8;
+                // fifth bit of sub-block 2c (2c + 1): bit 2c (2c + 1) of the qh byte at the same position
+                lo[2 * t] = h2fma((w & 0x000f000fu) | (((qh >> (2 * c)) & 0x00010001u) << 4) | mg, ml, al);
+                lo[2 * t + 1] = h2fma((s & 0x000f000fu) | (((qs >> (2 * c)) & 0x00010001u) << 4) | mg, ml, al);
+                hi[2 * t] = h2fma((w & 0x00f000f0u) | (((qh >> (2 * c + 1)) & 0x00010001u) << 8) | mg, mh, ah);
+                hi[2 * t + 1] = h2fma((s & 0x00f000f0u) | (((qs >> (2 * c + 1)) & 0x00010001u) << 8) | mg, mh, ah);
+            }
+            B[2 * c] = cat8(lo[0], lo[1], lo[2], lo[3]);
+            B[2 * c + 1] = cat8(hi[0], hi[1], hi[2], hi[3]);
+        }
+        Bm = cat8(bytes2(k.mnA, 0), bytes2(k.mnA, 16), bytes2(k.mnB, 0), bytes2(k.mnB, 16));
+    }
+};
+
+// y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) for b < rows <= 8 * groups; k a multiple of 256, n >= 16.
+//   ops / inv: the output of rows_prepare_kernel for the same x.  grid: up to one workgroup per batch of GR_T tiles of 16
+//   weight rows (the host caps it at one per compute unit); GR_THREADS threads; gemv_rows_lds_bytes() of dynamic LDS.
+template <int FMT>
+__global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ ops,
+                                                                const float *__restrict__ inv, const float *__restrict__ bias, float *__restrict__ y,
+                                                                int n, int k, int rows, int groups) {
+    typedef RTile<FMT> R;
+    constexpr int T = GR_T;
+    extern __shared__ __attribute__((aligned(16))) uint8_t gr_smem[];
+    float2 *accl = reinterpret_cast<float2 *>(gr_smem);  // [tile t][group g][thread]
+    const int tid = threadIdx.x, lane = tid & 63, nq = lane & 15, kq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ncol = k >> 8, ntiles = (n + 15) >> 4, nbatch = (ntiles + T - 1) / T;
+    const size_t rowbytes = (size_t)ncol * R::BYTES;
+
+    for (int tb = blockIdx.x; tb < nbatch; tb += gridDim.x) {
+        // this lane's row of each tile of the batch (the last tile of a ragged matrix is the last 16 rows: in bounds, its
+        // first rows computed twice, stored once)
+        const uint8_t *rp[T];
+        bool live[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) {
+            const int tile = tb * T + t;
+            live[t] = tile < ntiles;  // workgroup-uniform
+            rp[t] = W + (size_t)(min((live[t] ? tile : ntiles - 1) * 16, n - 16) + nq) * rowbytes;
+        }
+        for (int i = tid; i < T * groups * GR_THREADS; i += GR_THREADS) accl[i] = make_float2(0.f, 0.f);
+        // (each thread only ever touches its own slots of accl until the final reduction: no barrier needed here)
+
+        typename R::Raw raw[T];
+        int c = wave;
+        if (c < ncol) {
+#pragma unroll
+            for (int t = 0; t < T; ++t) R::load(raw[t], rp[t] + (size_t)c * R::BYTES, kq);
+        }
+        for (; c < ncol; c += GR_WAVES) {
+            f16x8 B[T][8], Bm[T];
+            float d[T], dmin64[T];
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                float dm;
+                R::decode(raw[t], B[t], Bm[t], d[t], dm);
+                dmin64[t] = dm * 64.f;
+            }
+            if (c + GR_WAVES < ncol) {  // the next column's bytes are on their way while this one meets the activations
+#pragma unroll
+                for (int t = 0; t < T; ++t) R::load(raw[t], rp[t] + (size_t)(c + GR_WAVES) * R::BYTES, kq);
+            }
+            for (int g = 0; g < groups; ++g) {
+                const _Float16 *op = ops + ((size_t)g * ncol + c) * GR_OP_HALVES + lane * 8;
+                f16x8 A[9];
+#pragma unroll
+                for (int s = 0; s < 9; ++s) A[s] = *reinterpret_cast<const f16x8 *>(op + s * 512);
+                const float2 iv = *reinterpret_cast<const float2 *>(inv + ((size_t)g * ncol + c) * 8 + 2 * kq);
+#pragma unroll
+                for (int t = 0; t < T; ++t) {
+                    if (!live[t]) continue;
+                    f32x4 cs = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int s = 0; s < 8; ++s) cs = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[s], B[t][s], cs, 0, 0, 0);
+                    const f32x4 cm = mfma16(A[8], Bm[t]);
+                    // operand rows 4 kq + i: activation rows 2 kq (hi, lo) and 2 kq + 1 (hi, lo) of the group
+                    const float s0 = cs[0] + cs[1], s1 = cs[2] + cs[3], m0 = cm[0] + cm[1], m1 = cm[2] + cm[3];
+                    float2 a = accl[(t * groups + g) * GR_THREADS + tid];
+                    a.x = __builtin_fmaf(iv.x, __builtin_fmaf(d[t], s0, -dmin64[t] * m0), a.x);
+                    a.y = __builtin_fmaf(iv.y, __builtin_fmaf(d[t], s1, -dmin64[t] * m1), a.y);
+                    accl[(t * groups + g) * GR_THREADS + tid] = a;
+                }
+            }
+        }
+        __syncthreads();
+        // the eight waves' partial sums, in wave order: item (t, g, lane position) -> two outputs
+        for (int i = tid; i < T * groups * 64; i += GR_THREADS) {
+            const int tg = i >> 6, l = i & 63, t = tg / groups, g = tg - t * groups;
+            const int tile = tb * T + t;
+            if (tile < ntiles) {
+                float2 sum = make_float2(0.f, 0.f);
+#pragma unroll
+                for (int w = 0; w < GR_WAVES; ++w) {
+                    const float2 p = accl[tg * GR_THREADS + w * 64 + l];
+                    sum.x += p.x;
+                    sum.y += p.y;
+                }
+                const int r = l & 15, row = min(tile * 16, n - 16) + r, b0 = g * 8 + 2 * (l >> 4);
+                if (row >= tile * 16) {  // rows of a ragged last tile that an earlier tile already wrote are skipped
+                    const float bv = bias ? bias[row] : 0.f;
+                    if (b0 < rows) y[(size_t)b0 * n + row] = sum.x + bv;
+                    if (b0 + 1 < rows) y[(size_t)(b0 + 1) * n + row] = sum.y + bv;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace jitnn

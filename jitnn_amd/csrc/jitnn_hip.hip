@@ -83,6 +83,7 @@ struct State {
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
     bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
+    int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
     bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
@@ -748,6 +749,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_ROWS_MIN")) g.rows_kernel_min = atoi(e);
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
@@ -894,6 +896,16 @@ int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const fl
     const bool many = rows > g.gemv_max_rows && !is_extra_format(w->fmt);
     count_op(many ? ST_MFMA : ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n) + (bias_dev ? 4ll * w->n : 0));
     if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s, src);
+    // several rows, rows of whole 256-value columns: every row meets the weights in one pass over them (gemv_rows.h)
+    if (g.rows_kernel_min > 0 && rows >= g.rows_kernel_min && rows <= 64 && gemv_rows_supported(w->fmt) && w->k % 256 == 0 && w->n >= 16 && !g.force_lds) {
+        const KernelRef kr = gemv_rows_kernel_ref(w->fmt);
+        if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
+        void *scratch = nullptr;
+        if (int rc = workspace(gemv_rows_scratch_bytes(rows, w->k), s, &scratch, src)) return rc;
+        gemv_rows_launch(w->fmt, (unsigned)g.cus, s, w->dev, x_dev, scratch, bias_dev, y_dev, w->n, w->k, rows);
+        HIP_TRY(hipGetLastError());
+        return workspace_done(s, src);
+    }
     for (int r0 = 0; r0 < rows; r0 += 8) {
         const int nb = rows - r0 < 8 ? rows - r0 : 8;
         if (int rc = launch_gemv(w, x_dev + (size_t)r0 * w->k, nb, bias_dev, y_dev + (size_t)r0 * w->n, s)) return rc;

@@ -35,4 +35,11 @@ void prefill_join_launch(const float *part, const float *bias, const float *res,
 KernelRef gemv_mfma_kernel_ref(int fmt);
 void gemv_mfma_launch(int fmt, unsigned blocks, hipStream_t s, const uint8_t *W, const float *x, const float *bias, float *y, int n, int k, int rows);
 
+// ---- gemv_rows.hip: rows_prepare_kernel + gemv_rows_kernel<fmt>: 2..64 rows in one pass over the weights
+bool gemv_rows_supported(int fmt);
+size_t gemv_rows_scratch_bytes(int rows, int k);   // operands + scales of `rows` activation rows of k values
+KernelRef gemv_rows_kernel_ref(int fmt);
+void gemv_rows_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const float *x, void *scratch, const float *bias, float *y, int n,
+                      int k, int rows);
+
 }  // namespace jitnn
