@@ -509,15 +509,23 @@ int workspace_done(hipStream_t stream, ScratchSource src = SCRATCH_THREAD) {
 // on host buffers): a pinned host buffer, a device buffer and a stream, all grow-only, so that a call costs copies and
 // launches but no allocation.  Buffers beyond STAGE_KEEP_MAX are not kept (a dequantised matrix goes through in pieces).
 constexpr size_t STAGE_KEEP_MAX = (size_t)128 << 20;
+// 16-byte pieces from one buffer to another; one side is pinned host memory as the device sees it.  For the few KB of a
+// GEMV call a launch costs less than a DMA transfer's set-up, and the bytes cross the bus in whole lines.
+__global__ void __launch_bounds__(256) stage_copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t count16) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+constexpr size_t STAGE_KERNEL_COPY_MAX = (size_t)1 << 20;  // above this a DMA transfer is as fast and leaves the compute units alone
+
 struct HostStage {
     uint8_t *pinned = nullptr, *dev = nullptr;
+    uint8_t *pinned_dev = nullptr;  // the pinned buffer's address on the device
     size_t pcap = 0, dcap = 0;
     hipStream_t stream = nullptr;
     void release() {
         if (pinned) (void)hipHostFree(pinned);
         if (dev) (void)hipFree(dev);
         if (stream) (void)hipStreamDestroy(stream);
-        pinned = dev = nullptr;
+        pinned = dev = pinned_dev = nullptr;
         pcap = dcap = 0;
         stream = nullptr;
     }
@@ -549,12 +557,16 @@ int stage_reserve(size_t pinned_bytes, size_t dev_bytes) {
     auto round = [](size_t b) { return (b + ((size_t)1 << 16) - 1) & ~(((size_t)1 << 16) - 1); };
     if (pinned_bytes > st.pcap) {
         if (st.pinned) HIP_TRY(hipHostFree(st.pinned));
-        st.pinned = nullptr;
+        st.pinned = st.pinned_dev = nullptr;
         st.pcap = 0;
         const size_t want = round(pinned_bytes);
         hipError_t e = hipHostMalloc((void **)&st.pinned, want, hipHostMallocDefault);
         if (e != hipSuccess) return fail(JITNN_HIP_ENOMEM, "hipHostMalloc of %zu bytes of staging: %s", want, hipGetErrorString(e));
         st.pcap = want;
+        if (hipHostGetDevicePointer((void **)&st.pinned_dev, st.pinned, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            st.pinned_dev = nullptr;  // not mapped: the DMA path is used
+        }
     }
     if (dev_bytes > st.dcap) {
         if (st.dev) HIP_TRY(hipFree(st.dev));
@@ -937,17 +949,31 @@ int jitnn_hip_linear(const jitnn_hip_weight *w, const float *x_host, int rows, c
     const bool keep = total <= STAGE_KEEP_MAX;  // small calls go through pinned memory (one DMA each way, no page locking per call)
     if (int rc = stage_reserve(keep ? total : 0, total)) return rc;
     HostStage &st = g_thread.stage;
+    // small calls: the device itself fetches the input from the pinned buffer and writes the result back into it
+    const bool by_kernel = keep && st.pinned_dev && total <= STAGE_KERNEL_COPY_MAX;
+    auto copy16 = [&](uint8_t *dst, const uint8_t *src, size_t bytes) {
+        const size_t count16 = (bytes + 15) / 16;  // the sections of the layout are 256-byte aligned: rounding up stays inside
+        const unsigned blocks = (unsigned)std::min<size_t>((count16 + 255) / 256, 64);
+        hipLaunchKernelGGL(stage_copy_kernel, dim3(blocks), dim3(256), 0, st.stream, (uint4 *)dst, (const uint4 *)src, count16);
+    };
     if (keep) {
         memcpy(st.pinned, x_host, xb);
         if (bias_host) memcpy(st.pinned + bo, bias_host, bb);
-        HIP_TRY(hipMemcpyAsync(st.dev, st.pinned, bias_host ? bo + bb : xb, hipMemcpyHostToDevice, st.stream));
+        const size_t up = bias_host ? bo + bb : xb;
+        if (by_kernel) copy16(st.dev, st.pinned_dev, up);
+        else HIP_TRY(hipMemcpyAsync(st.dev, st.pinned, up, hipMemcpyHostToDevice, st.stream));
     } else {
         HIP_TRY(hipMemcpyAsync(st.dev, x_host, xb, hipMemcpyHostToDevice, st.stream));
         if (bias_host) HIP_TRY(hipMemcpyAsync(st.dev + bo, bias_host, bb, hipMemcpyHostToDevice, st.stream));
     }
     int rc = jitnn_hip_linear_dev(w, (const float *)st.dev, rows, bias_host ? (const float *)(st.dev + bo) : nullptr, (float *)(st.dev + yo), st.stream);
     if (rc == JITNN_HIP_OK) {
-        HIP_TRY(hipMemcpyAsync(keep ? (void *)(st.pinned + yo) : (void *)y_host, st.dev + yo, yb, hipMemcpyDeviceToHost, st.stream));
+        if (by_kernel) {
+            copy16(st.pinned_dev + yo, st.dev + yo, yb);
+            HIP_TRY(hipGetLastError());
+        } else {
+            HIP_TRY(hipMemcpyAsync(keep ? (void *)(st.pinned + yo) : (void *)y_host, st.dev + yo, yb, hipMemcpyDeviceToHost, st.stream));
+        }
         HIP_TRY(hipStreamSynchronize(st.stream));
         if (keep) memcpy(y_host, st.pinned + yo, yb);
     }
