@@ -83,6 +83,7 @@ struct State {
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
     bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
+    bool prefill_group = true;   // JITNN_HIP_PREFILL_GROUP=0: every weight of a group of linears in a launch of its own
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
@@ -589,39 +590,65 @@ int stage_reserve(size_t pinned_bytes, size_t dev_bytes) {
 int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias,
                          const float *norm_w, float eps, hipStream_t stream, const float *residual = nullptr, float *tmp = nullptr,
                          const float *swiglu_up = nullptr, ScratchSource src = SCRATCH_THREAD) {
-    // (the kernels live in prefill_k.hip and prefill_q32.hip)
-    struct Plan {
-        bool kq;
-        int ntiles, splits, split_steps;
+    // (the kernels live in prefill_k.hip, prefill_q32.hip and prefill_mixed.hip)
+    // Weights of one format - and a run of one K-quant format followed by a run of another for which a two-format kernel
+    // exists - share a launch: their row tiles are numbered one after the other, so that the 1024-row k and v projections
+    // fill the device together with q instead of splitting K eight ways each.
+    struct Launch {
+        int first, count, first_b;  // weights [first, first + count); first_b: where the second format starts (count: one format)
+        int tiles, splits, split_steps;
         size_t part_bytes;
-    } plan[4];
+    } launch[4];
+    int nlaunch = 0;
     if (count < 1 || count > 4) return fail(JITNN_HIP_EINVAL, "%d weights on one activation", count);
     if (residual && (count != 1 || !tmp || ws[0]->n % 4 != 0)) return fail(JITNN_HIP_EINVAL, "a residual needs one weight, rows of whole quads and a buffer");
     const int k = ws[0]->k;
     const int mtiles = (rows + PF_BM - 1) / PF_BM, mblocks = mtiles * (PF_BM / 32);  // operands padded to whole tiles of tokens
     const int nsteps = (k + PF_BK - 1) / PF_BK;
-    size_t part_max = 0;
+    auto kq = [](const jitnn_hip_weight *w) { return block_values(w->fmt) == 256; };
     for (int i = 0; i < count; ++i) {
         const jitnn_hip_weight *w = ws[i];
         if (w->k != k) return fail(JITNN_HIP_EINVAL, "weights of %d and %d values per row on one activation", k, w->k);
-        Plan &p = plan[i];
-        p.kq = block_values(w->fmt) == 256;
-        const KernelRef kr = p.kq ? prefill_kernel_k(w->fmt) : prefill_kernel_q32(w->fmt);
+        const KernelRef kr = kq(w) ? prefill_kernel_k(w->fmt) : prefill_kernel_q32(w->fmt);
         if (!kr.fn) return fail(JITNN_HIP_EUNSUPPORTED, "no many-row kernel for format %d", w->fmt);
         if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
-        p.ntiles = (w->n + PF_BN - 1) / PF_BN;
+    }
+    for (int i = 0; i < count;) {
+        Launch &l = launch[nlaunch++];
+        l.first = i;
+        int j = i + 1;
+        const bool joinable = !bias && !residual && g.prefill_group;  // (several weights: partial sums of all of them are joined by one kernel)
+        while (joinable && j < count && j - i < 3 && ws[j]->fmt == ws[i]->fmt && ws[j]->n % 4 == 0 && ws[i]->n % 4 == 0) ++j;
+        l.first_b = j - i;
+        if (joinable && j < count && j - i < 3 && ws[j]->fmt != ws[i]->fmt && ws[i]->n % 4 == 0) {
+            const KernelRef kr = prefill_kernel_mixed(ws[i]->fmt, ws[j]->fmt);
+            if (kr.fn) {
+                if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
+                const int fb = ws[j]->fmt;
+                while (j < count && j - i < 3 && ws[j]->fmt == fb && ws[j]->n % 4 == 0) ++j;
+            }
+        }
+        l.count = j - i;
+        l.tiles = 0;
+        size_t nsum = 0;
+        for (int q = i; q < j; ++q) {
+            l.tiles += (ws[q]->n + PF_BN - 1) / PF_BN;
+            nsum += (size_t)ws[q]->n;
+        }
         // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 8 steps writes its
         // own partial y, a second kernel adds the slices in order.
-        p.splits = 1;
-        if (w->n % 4 == 0) {
-            while (p.splits < 8 && p.ntiles * mtiles * p.splits * 2 <= g.cus && nsteps / (p.splits * 2) >= g.prefill_min_slice) p.splits *= 2;
+        l.splits = 1;
+        if (nsum % 4 == 0 && (l.count == 1 ? ws[i]->n % 4 == 0 : true)) {
+            while (l.splits < 8 && l.tiles * mtiles * l.splits * 2 <= g.cus && nsteps / (l.splits * 2) >= g.prefill_min_slice) l.splits *= 2;
         }
         // slices of the 256-value formats start on whole blocks (four steps): the kernel stages their raw bytes by block
-        p.split_steps = (nsteps + p.splits - 1) / p.splits;
-        if (p.kq) p.split_steps = (p.split_steps + 3) & ~3;
-        p.part_bytes = p.splits > 1 ? (size_t)p.splits * rows * w->n * 4 : 0;
-        if (p.part_bytes > part_max) part_max = p.part_bytes;
+        l.split_steps = (nsteps + l.splits - 1) / l.splits;
+        if (kq(ws[i])) l.split_steps = (l.split_steps + 3) & ~3;
+        l.part_bytes = l.splits > 1 ? (size_t)l.splits * rows * nsum * 4 : 0;
+        i = j;
     }
+    size_t part_max = 0;
+    for (int i = 0; i < nlaunch; ++i) part_max = std::max(part_max, launch[i].part_bytes);
     const size_t xo_bytes = (size_t)mblocks * pf_ksteps(k) * 1024;
     const size_t scale_bytes = ((size_t)rows * 8 + 255) & ~(size_t)255;
     void *wsp = nullptr;
@@ -630,24 +657,40 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     float *scale = (float *)((uint8_t *)wsp + xo_bytes), *inv = scale + rows;
     float *part = (float *)((uint8_t *)wsp + xo_bytes + scale_bytes);
     prefill_prepare_launch(x, scale, inv, xo, rows, k, mblocks, norm_w, eps, swiglu_up, stream);
-    for (int i = 0; i < count; ++i) {
-        const jitnn_hip_weight *w = ws[i];
-        const Plan &p = plan[i];
-        float *out = p.splits > 1 ? part : residual ? tmp : ys[i];
-        const float *b1 = p.splits > 1 ? nullptr : bias;
-        const dim3 grid(p.ntiles, mtiles, p.splits);
-        if (p.kq) prefill_launch_k(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, k, p.split_steps);
-        else prefill_launch_q32(w->fmt, grid, stream, w->dev, xo, inv, b1, out, rows, w->n, k, p.split_steps);
-        if (p.splits > 1) {  // (the stream orders the next weight's partial sums after this join)
+    for (int li = 0; li < nlaunch; ++li) {
+        const Launch &l = launch[li];
+        const jitnn_hip_weight *w = ws[l.first];
+        PfSegments sg{}, out{};
+        size_t before = 0;  // floats of partial sums of the segments before this one
+        for (int q = 0; q < l.count; ++q) {
+            const jitnn_hip_weight *wq = ws[l.first + q];
+            sg.W[q] = wq->dev;
+            sg.n[q] = wq->n;
+            sg.tiles[q] = (wq->n + PF_BN - 1) / PF_BN;
+            sg.y[q] = l.splits > 1 ? part + before : (residual ? tmp : ys[l.first + q]);
+            before += (size_t)l.splits * rows * wq->n;
+            out.y[q] = ys[l.first + q];
+            out.n[q] = wq->n;
+        }
+        const float *b1 = l.splits > 1 ? nullptr : bias;
+        const dim3 grid(l.tiles, mtiles, l.splits);
+        if (l.first_b < l.count) prefill_launch_mixed(w->fmt, ws[l.first + l.first_b]->fmt, l.first_b, grid, stream, sg, xo, inv, rows, k, l.split_steps);
+        else if (kq(w)) prefill_launch_k(w->fmt, grid, stream, sg, xo, inv, b1, rows, k, l.split_steps);
+        else prefill_launch_q32(w->fmt, grid, stream, sg, xo, inv, b1, rows, k, l.split_steps);
+        if (l.splits > 1 && l.count > 1) {  // (the stream orders the next launch's partial sums after this join)
+            size_t count4 = 0;
+            for (int q = 0; q < l.count; ++q) count4 += (size_t)rows * sg.n[q] / 4;
+            const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
+            prefill_join_group_launch(part, out, rows, l.splits, blocks, stream);
+        } else if (l.splits > 1) {
             const size_t count4 = (size_t)rows * w->n / 4;
-            size_t blocks = (count4 + 255) / 256;
-            if (blocks > (size_t)g.cus * 8) blocks = (size_t)g.cus * 8;
-            prefill_join_launch(part, bias, residual, ys[i], count4, w->n, p.splits, (unsigned)blocks, stream);
+            const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
+            prefill_join_launch(part, bias, residual, ys[l.first], count4, w->n, l.splits, blocks, stream);
         } else if (residual) {
             const size_t count4 = (size_t)rows * w->n / 4;
             const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
             hipLaunchKernelGGL(add_rows_kernel, dim3(blocks), dim3(256), 0, stream, reinterpret_cast<const float4 *>(tmp),
-                               reinterpret_cast<const float4 *>(residual), reinterpret_cast<float4 *>(ys[i]), count4);
+                               reinterpret_cast<const float4 *>(residual), reinterpret_cast<float4 *>(ys[l.first]), count4);
         }
     }
     HIP_TRY(hipGetLastError());
@@ -762,6 +805,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_ROWS_MIN")) g.rows_kernel_min = atoi(e);
+    if (const char *e = getenv("JITNN_HIP_PREFILL_GROUP")) g.prefill_group = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;

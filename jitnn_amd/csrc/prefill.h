@@ -17,6 +17,7 @@
 #pragma once
 #include "common.h"
 #include "dequant.h"
+#include "tu.h"
 
 namespace jitnn {
 
@@ -467,17 +468,18 @@ __device__ __forceinline__ void pf_load_lds(PfRaw<FMT> &r, const uint8_t *b, int
     }
 }
 
+// The work of one workgroup: row tile `tile` of the weight W [n, k] against token tile blockIdx.y, K slice blockIdx.z.
 template <int FMT>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xo,
-                                                            const float *__restrict__ inv_scale, const float *__restrict__ bias,
-                                                            float *__restrict__ y, int m, int n, int k, int split_steps) {
+__device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xo, const float *__restrict__ inv_scale,
+                                                  const float *__restrict__ bias, float *__restrict__ y, const int m, const int n, const int k,
+                                                  const int split_steps, const int tile) {
     using Stage = PfStage<FMT>;
     constexpr bool STAGED = Stage::ON;
     extern __shared__ __align__(16) uint8_t pf_smem[];  // pf_lds_bytes<FMT>()
     _Float16(*As)[PF_BN * PF_LD] = reinterpret_cast<_Float16(*)[PF_BN * PF_LD]>(pf_smem);  // dequantised weights [row][k], two steps
     uint8_t *Rs = pf_smem + 2 * PF_BN * PF_LD * 2;                                         // staged raw blocks [2][row][RP]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n0 = blockIdx.x * PF_BN, m0 = blockIdx.y * PF_BM;
+    const int n0 = tile * PF_BN, m0 = blockIdx.y * PF_BM;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
     // dequantiser role: thread t fills weights [row t/2][32 * (t%2) ... +32) of the step
     const int drow = tid >> 1, dhalf = tid & 1;
@@ -679,6 +681,45 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     }
 }
 
+// Up to three weights of one activation in one launch (the q, k and v projections of a layer): their row tiles are
+// numbered one after the other along blockIdx.x, every workgroup works on its weight exactly as in a launch of its own.
+__device__ __forceinline__ void pf_locate(const PfSegments &sg, int &seg, int &tile) {
+    seg = 0;
+    tile = blockIdx.x;
+    if (tile >= sg.tiles[0]) {
+        tile -= sg.tiles[0];
+        seg = 1;
+        if (tile >= sg.tiles[1]) {
+            tile -= sg.tiles[1];
+            seg = 2;
+        }
+    }
+}
+
+// grid: (row tiles of all segments, token tiles, K slices); 256 threads; pf_lds_bytes<FMT>() of dynamic LDS.
+//   sg.y[i]: [m, n[i]], or for a launch that splits K the first slice's array of partial sums (slice z at + z m n[i]);
+//   bias: one segment only.
+template <int FMT>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_kernel(const PfSegments sg, const _Float16 *__restrict__ xo,
+                                                            const float *__restrict__ inv_scale, const float *__restrict__ bias,
+                                                            int m, int k, int split_steps) {
+    int seg, tile;
+    pf_locate(sg, seg, tile);
+    prefill_mfma_body<FMT>(sg.W[seg], xo, inv_scale, bias, sg.y[seg], m, sg.n[seg], k, split_steps, tile);
+}
+
+// The same for weights of two formats (a Q4_K_M layer keeps q and k as Q4_K and v as Q6_K): segments below first_b are
+// FA, the others FB.  LDS: the larger of the two.
+template <int FA, int FB>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_mixed_kernel(const PfSegments sg, const int first_b,
+                                                            const _Float16 *__restrict__ xo, const float *__restrict__ inv_scale,
+                                                            int m, int k, int split_steps) {
+    int seg, tile;
+    pf_locate(sg, seg, tile);
+    if (seg < first_b) prefill_mfma_body<FA>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, split_steps, tile);
+    else prefill_mfma_body<FB>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, split_steps, tile);
+}
+
 // y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]) (+ res[tok, row]), slices in order: the second half of a
 // split-K launch.  count4 = m * n / 4 (n is a multiple of 4 whenever the launch splits).
 static __global__ void __launch_bounds__(256) prefill_join_kernel(const float *__restrict__ part, const float *__restrict__ bias,
@@ -707,6 +748,26 @@ static __global__ void __launch_bounds__(256) prefill_join_kernel(const float *_
             a.w += b.w;
         }
         reinterpret_cast<float4 *>(y)[i] = a;
+    }
+}
+
+// The join for a launch of several segments: part holds, segment after segment, `splits` arrays [m, n[i]] of partial sums;
+// y[i][tok, row] = their sum in slice order.  n[i] multiples of 4.
+static __global__ void __launch_bounds__(256) prefill_join_group_kernel(const float *__restrict__ part, const PfSegments sg, int m, int splits) {
+    const size_t c0 = (size_t)m * sg.n[0] / 4, c1 = (size_t)m * sg.n[1] / 4, c2 = (size_t)m * sg.n[2] / 4;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < c0 + c1 + c2; i += (size_t)gridDim.x * 256) {
+        const int seg = (i >= c0) + (i >= c0 + c1);
+        const size_t before = seg == 0 ? 0 : seg == 1 ? c0 : c0 + c1, cnt = seg == 0 ? c0 : seg == 1 ? c1 : c2, local = i - before;
+        const float4 *p = reinterpret_cast<const float4 *>(part) + before * splits + local;
+        float4 a = p[0];
+        for (int z = 1; z < splits; ++z) {
+            const float4 b = p[(size_t)z * cnt];
+            a.x += b.x;
+            a.y += b.y;
+            a.z += b.z;
+            a.w += b.w;
+        }
+        reinterpret_cast<float4 *>(sg.y[seg])[local] = a;
     }
 }
 

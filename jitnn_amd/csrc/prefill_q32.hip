@@ -13,12 +13,12 @@ KernelRef prefill_kernel_q32(int fmt) {
     }
 }
 
-void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const _Float16 *xo, const float *inv_scale, const float *bias, float *y,
-                        int m, int n, int k, int split_steps) {
+void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m, int k,
+                      int split_steps) {
     switch (fmt) {
-    case F_Q4_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_0>, grid, dim3(256), pf_lds_bytes<F_Q4_0>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
-    case F_Q4_1: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_1>, grid, dim3(256), pf_lds_bytes<F_Q4_1>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
-    case F_Q8_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q8_0>, grid, dim3(256), pf_lds_bytes<F_Q8_0>(), s, W, xo, inv_scale, bias, y, m, n, k, split_steps); break;
+    case F_Q4_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_0>, grid, dim3(256), pf_lds_bytes<F_Q4_0>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
+    case F_Q4_1: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_1>, grid, dim3(256), pf_lds_bytes<F_Q4_1>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
+    case F_Q8_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q8_0>, grid, dim3(256), pf_lds_bytes<F_Q8_0>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
     default: break;
     }
 }
@@ -48,6 +48,10 @@ void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Flo
 void prefill_join_launch(const float *part, const float *bias, const float *res, float *y, size_t count4, int n, int splits, unsigned blocks,
                          hipStream_t s) {
     hipLaunchKernelGGL(prefill_join_kernel, dim3(blocks), dim3(256), 0, s, part, bias, res, y, count4, n, splits);
+}
+
+void prefill_join_group_launch(const float *part, const PfSegments &sg, int m, int splits, unsigned blocks, hipStream_t s) {
+    hipLaunchKernelGGL(prefill_join_group_kernel, dim3(blocks), dim3(256), 0, s, part, sg, m, splits);
 }
 
 }  // namespace jitnn
