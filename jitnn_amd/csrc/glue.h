@@ -563,6 +563,191 @@ __global__ void __launch_bounds__(256) attn_prefill_h_kernel(const float *__rest
     }
 }
 
+// The same attention on the matrix cores (v_mfma_f32_16x16x32_f16, FP16 operands, FP32 accumulation and softmax), for
+// heads of 64 or 128 values.  A workgroup of AM_WAVES waves takes AM_ROWS (token, query head) rows of one key/value head,
+// every wave 16 of them, and walks the keys in chunks of AM_CH staged once in LDS as binary16 for all of them (the more
+// rows share a chunk, the fewer times the cache is read: 128 rows read it half as often as 64).
+//   * scores, transposed: S^T = K Q^T, so that a lane ends up with the scores of ONE query row (column lane % 16 of the
+//     result) against the keys 4 (lane / 16) + i of every 16-key tile - the running softmax of a row needs its chunk
+//     maximum from the three other lanes that hold the row's other keys (two shuffles), the row sum stays a per-lane
+//     partial sum until the end;
+//   * the contraction index of a matrix-core product may be numbered in any order as long as both operands use the
+//     same one: the probabilities a lane holds after the softmax - keys 4 kq + i of two neighbouring 16-key tiles -
+//     ARE its eight slots of the first operand of P V, when the values are laid out in LDS in that slot order
+//     (transposed, [d][slot]).  No probability goes through LDS;
+//   * the factor that rescales a row's output so far is handed from the lanes that know it (score layout: lane % 16 =
+//     row) to the lanes that hold the output (rows 4 (lane / 16) + i) through 64 bytes of LDS per wave;
+//   * keys and values of the chunk after next are requested into registers while the current one is multiplied; the LDS
+//     tiles are double-buffered, one workgroup barrier per chunk; nothing about the loads is conditional (chunks past
+//     the end repeat the last one, keys past the last visible one re-read it and are masked).
+constexpr int AM_ROWS = 128, AM_CH = 64, AM_WAVES = AM_ROWS / 16, AM_THREADS = 64 * AM_WAVES;
+template <int D>
+constexpr size_t attn_prefill_mfma_lds_bytes() {
+    return (size_t)2 * ((size_t)AM_CH * (D + 8) + (size_t)D * (AM_CH + 8)) * sizeof(_Float16) + AM_WAVES * 16 * sizeof(float);
+}
+template <int D>
+__global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const float *__restrict__ q, const float *__restrict__ kcache,
+                                                                 const float *__restrict__ vcache, float *__restrict__ out, int heads, int kv_heads,
+                                                                 int pos0, int T, float scale) {
+    constexpr int CH = AM_CH, KP = D + 8, VP = CH + 8, DB = D / 32, DT = D / 16, DQ = D / 4;
+    constexpr int NIT = (CH / 2) * DQ / AM_THREADS;  // (key pair, four values of d) items per thread and chunk
+    static_assert((CH / 2) * DQ % AM_THREADS == 0, "whole passes");
+    static_assert(D == 64 || D == 128, "head sizes of this kernel");
+    extern __shared__ __align__(16) float att_smem[];
+    _Float16 *Kh = reinterpret_cast<_Float16 *>(att_smem);  // [2][CH][KP]
+    _Float16 *Vt = Kh + 2 * CH * KP;                        // [2][D][VP]: values transposed, keys in slot order
+    float *fx = reinterpret_cast<float *>(Vt + 2 * D * VP);  // [AM_WAVES][16]: a factor per row, from score layout to output layout
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, kq = lane >> 4;
+    const int group = heads / kv_heads, QT = AM_ROWS / group, rows = QT * group;
+    const int g = blockIdx.y;
+    // early token blocks walk few keys, late ones many: half of the key/value heads take the blocks in reverse
+    const int tb = 2 * (int)blockIdx.y < kv_heads ? (int)blockIdx.x : (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int t0 = tb * QT;
+    const int tl = min(t0 + QT, T) - 1;        // last token of the block
+    const int jlast = pos0 + tl;               // last key any row of the block sees
+    const int nchunks = jlast / CH + 1;
+    // ---- this lane's query row (score layout): row r of the block, as the second operand of S^T = K Q^T
+    const int r = 16 * wave + n, tq = r / group, hq = r - tq * group;
+    const bool live = r < rows && t0 + tq < T;
+    const int jmax = pos0 + t0 + tq;  // the last key the row sees
+    f16x8 qb[DB];
+    {
+        const float *qp = q + ((size_t)(t0 + (live ? tq : 0)) * heads + g * group + (live ? hq : 0)) * D + 8 * kq;
+#pragma unroll
+        for (int b = 0; b < DB; ++b) {
+            const float4 a = *reinterpret_cast<const float4 *>(qp + 32 * b), c = *reinterpret_cast<const float4 *>(qp + 32 * b + 4);
+            qb[b] = live ? f16x8{(_Float16)a.x, (_Float16)a.y, (_Float16)a.z, (_Float16)a.w, (_Float16)c.x, (_Float16)c.y, (_Float16)c.z, (_Float16)c.w}
+                         : f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+    // ---- staging: an item is (key pair jp, values e .. e + 3).  Eight neighbouring lanes take the eight quads of a 128-byte
+    // line of a key's row, the eight groups of eight lanes eight key pairs: a load touches whole lines, and the transposed
+    // LDS stores of the values (a 4-byte word per d) spread over the banks instead of meeting in four of them.
+    float4 rk0[NIT], rk1[NIT], rv0[NIT], rv1[NIT];
+    auto item = [&](int it, int &jp, int &e) {
+        const int wv = (tid >> 6) + it * AM_WAVES;  // wave-sized groups of items
+        e = 4 * ((lane & 7) + 8 * (wv % (DQ / 8)));
+        jp = (lane >> 3) + 8 * (wv / (DQ / 8));
+    };
+    auto fetch = [&](int c) {
+        const int j0 = min(c, nchunks - 1) * CH;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            int jp, e;
+            item(it, jp, e);
+            const size_t r0 = ((size_t)min(j0 + 2 * jp, jlast) * kv_heads + g) * D + e;
+            const size_t r1 = ((size_t)min(j0 + 2 * jp + 1, jlast) * kv_heads + g) * D + e;
+            rk0[it] = *reinterpret_cast<const float4 *>(kcache + r0);
+            rv0[it] = *reinterpret_cast<const float4 *>(vcache + r0);
+            rk1[it] = *reinterpret_cast<const float4 *>(kcache + r1);
+            rv1[it] = *reinterpret_cast<const float4 *>(vcache + r1);
+        }
+    };
+    auto store = [&](int buf) {
+        _Float16 *kh = Kh + buf * CH * KP, *vt = Vt + buf * D * VP;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            int jp, e;
+            item(it, jp, e);
+            const int j = 2 * jp;
+            const float4 k0 = rk0[it], k1 = rk1[it], v0 = rv0[it], v1 = rv1[it];
+            *reinterpret_cast<f16x4 *>(&kh[j * KP + e]) = f16x4{(_Float16)k0.x, (_Float16)k0.y, (_Float16)k0.z, (_Float16)k0.w};
+            *reinterpret_cast<f16x4 *>(&kh[(j + 1) * KP + e]) = f16x4{(_Float16)k1.x, (_Float16)k1.y, (_Float16)k1.z, (_Float16)k1.w};
+            // slot of key j within its 32-key step: lanes kq = (j % 16) / 4 hold keys 4 kq + i of the step's two 16-key tiles
+            const int jj = j & 31, col = (j & ~31) + ((jj & 15) >> 2) * 8 + (jj & 3) + 4 * (jj >> 4);
+            *reinterpret_cast<f16x2 *>(&vt[(e + 0) * VP + col]) = f16x2{(_Float16)v0.x, (_Float16)v1.x};
+            *reinterpret_cast<f16x2 *>(&vt[(e + 1) * VP + col]) = f16x2{(_Float16)v0.y, (_Float16)v1.y};
+            *reinterpret_cast<f16x2 *>(&vt[(e + 2) * VP + col]) = f16x2{(_Float16)v0.z, (_Float16)v1.z};
+            *reinterpret_cast<f16x2 *>(&vt[(e + 3) * VP + col]) = f16x2{(_Float16)v0.w, (_Float16)v1.w};
+        }
+    };
+    f32x4 o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float mrun = -INFINITY, lrun = 0.f;
+    fetch(0);
+    store(0);
+    fetch(1);
+    for (int c = 0; c < nchunks; ++c) {
+        __syncthreads();  // chunk c is in its buffer; the other buffer has been read (chunk c - 1)
+        store((c + 1) & 1);
+        fetch(c + 2);
+        const _Float16 *kh = Kh + (c & 1) * CH * KP, *vt = Vt + (c & 1) * D * VP;
+        const int j0 = c * CH;
+        // ---- S^T: four tiles of 16 keys; the lane ends up with keys j0 + 16 t + 4 kq + i of its row
+        f32x4 st[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            st[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int b = 0; b < DB; ++b) {
+                const f16x8 a = *reinterpret_cast<const f16x8 *>(&kh[(16 * t + n) * KP + 32 * b + 8 * kq]);
+                st[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[b], st[t], 0, 0, 0);
+            }
+        }
+        // ---- running softmax of the row
+        float mc = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const bool seen = live && j0 + 16 * t + 4 * kq + i <= jmax;
+                st[t][i] = seen ? st[t][i] * scale : -INFINITY;
+                mc = fmaxf(mc, st[t][i]);
+            }
+        mc = fmaxf(mc, __shfl_xor(mc, 16));
+        mc = fmaxf(mc, __shfl_xor(mc, 32));
+        const float mn = fmaxf(mrun, mc);
+        const float alpha = mrun > -INFINITY ? __expf(mrun - mn) : 0.f;
+        float ls = 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float pv = st[t][i] > -INFINITY ? __expf(st[t][i] - mn) : 0.f;
+                st[t][i] = pv;
+                ls += pv;
+            }
+        lrun = lrun * alpha + ls;
+        mrun = mn;
+        if (kq == 0) fx[16 * wave + n] = alpha;
+        // (the LDS operations of one wave complete in order: the read below sees the write above)
+        const f32x4 al = *reinterpret_cast<const f32x4 *>(&fx[16 * wave + 4 * kq]);
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+            o[t][0] *= al[0];
+            o[t][1] *= al[1];
+            o[t][2] *= al[2];
+            o[t][3] *= al[3];
+        }
+        // ---- O += P V, two steps of 32 keys
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const f16x8 pa = {(_Float16)st[2 * u][0], (_Float16)st[2 * u][1], (_Float16)st[2 * u][2], (_Float16)st[2 * u][3],
+                              (_Float16)st[2 * u + 1][0], (_Float16)st[2 * u + 1][1], (_Float16)st[2 * u + 1][2], (_Float16)st[2 * u + 1][3]};
+#pragma unroll
+            for (int t = 0; t < DT; ++t) {
+                const f16x8 vb = *reinterpret_cast<const f16x8 *>(&vt[(16 * t + n) * VP + 32 * u + 8 * kq]);
+                o[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, o[t], 0, 0, 0);
+            }
+        }
+    }
+    // ---- the row sums meet, the rows are normalised and written: the lane holds rows 4 kq + i, values 16 t + n
+    lrun += __shfl_xor(lrun, 16);
+    lrun += __shfl_xor(lrun, 32);
+    if (kq == 0) fx[16 * wave + n] = live ? 1.f / lrun : 0.f;
+    const f32x4 il = *reinterpret_cast<const f32x4 *>(&fx[16 * wave + 4 * kq]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ro = 16 * wave + 4 * kq + i, to = ro / group, ho = ro - to * group;
+        if (ro < rows && t0 + to < T) {
+            float *op = out + ((size_t)(t0 + to) * heads + g * group + ho) * D + n;
+#pragma unroll
+            for (int t = 0; t < DT; ++t) op[16 * t] = o[t][i] * il[i];
+        }
+    }
+}
+
 // y = a + b, four values per thread (the residual connections of many rows)
 __global__ void __launch_bounds__(256) add_rows_kernel(const float4 *__restrict__ a, const float4 *__restrict__ b, float4 *__restrict__ y, size_t count4) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < count4; i += (size_t)gridDim.x * 256) {

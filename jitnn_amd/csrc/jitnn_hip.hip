@@ -87,6 +87,7 @@ struct State {
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
+    bool prefill_attn_mfma = true;  // JITNN_HIP_PREFILL_ATTN_MFMA=0: the FP16 attention of long prompts on v_dot2 instead of the matrix cores
     bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
     void *scratch_ptr = nullptr;    // device address of `scratch` on g.device (hipGetSymbolAddress at init)
 };
@@ -596,7 +597,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     // fill the device together with q instead of splitting K eight ways each.
     struct Launch {
         int first, count, first_b;  // weights [first, first + count); first_b: where the second format starts (count: one format)
-        int tiles, splits, split_steps;
+        int splits[3], split_steps[3];
         size_t part_bytes;
     } launch[4];
     int nlaunch = 0;
@@ -606,6 +607,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     const int mtiles = (rows + PF_BM - 1) / PF_BM, mblocks = mtiles * (PF_BM / 32);  // operands padded to whole tiles of tokens
     const int nsteps = (k + PF_BK - 1) / PF_BK;
     auto kq = [](const jitnn_hip_weight *w) { return block_values(w->fmt) == 256; };
+    auto tiles_of = [](const jitnn_hip_weight *w) { return (w->n + PF_BN - 1) / PF_BN; };
     for (int i = 0; i < count; ++i) {
         const jitnn_hip_weight *w = ws[i];
         if (w->k != k) return fail(JITNN_HIP_EINVAL, "weights of %d and %d values per row on one activation", k, w->k);
@@ -620,7 +622,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
         const bool joinable = !bias && !residual && g.prefill_group;  // (several weights: partial sums of all of them are joined by one kernel)
         while (joinable && j < count && j - i < 3 && ws[j]->fmt == ws[i]->fmt && ws[j]->n % 4 == 0 && ws[i]->n % 4 == 0) ++j;
         l.first_b = j - i;
-        if (joinable && j < count && j - i < 3 && ws[j]->fmt != ws[i]->fmt && ws[i]->n % 4 == 0) {
+        if (joinable && j < count && j - i < 3 && ws[j]->fmt != ws[i]->fmt && ws[i]->n % 4 == 0 && ws[j]->n % 4 == 0) {
             const KernelRef kr = prefill_kernel_mixed(ws[i]->fmt, ws[j]->fmt);
             if (kr.fn) {
                 if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
@@ -629,22 +631,34 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
             }
         }
         l.count = j - i;
-        l.tiles = 0;
+        int tiles = 0;
         size_t nsum = 0;
         for (int q = i; q < j; ++q) {
-            l.tiles += (ws[q]->n + PF_BN - 1) / PF_BN;
+            tiles += tiles_of(ws[q]);
             nsum += (size_t)ws[q]->n;
         }
         // A launch that would leave most CUs idle (few, large tiles) splits K: every slice of at least 8 steps writes its
         // own partial y, a second kernel adds the slices in order.
-        l.splits = 1;
-        if (nsum % 4 == 0 && (l.count == 1 ? ws[i]->n % 4 == 0 : true)) {
-            while (l.splits < 8 && l.tiles * mtiles * l.splits * 2 <= g.cus && nsteps / (l.splits * 2) >= g.prefill_min_slice) l.splits *= 2;
+        int splits = 1;
+        if (nsum % 4 == 0 && ws[i]->n % 4 == 0) {
+            while (splits < 8 && tiles * mtiles * splits * 2 <= g.cus && nsteps / (splits * 2) >= g.prefill_min_slice) splits *= 2;
         }
-        // slices of the 256-value formats start on whole blocks (four steps): the kernel stages their raw bytes by block
-        l.split_steps = (nsteps + l.splits - 1) / l.splits;
-        if (kq(ws[i])) l.split_steps = (l.split_steps + 3) & ~3;
-        l.part_bytes = l.splits > 1 ? (size_t)l.splits * rows * nsum * 4 : 0;
+        int wgs = tiles * mtiles * splits;
+        l.part_bytes = 0;
+        for (int q = 0; q < l.count; ++q) {
+            const jitnn_hip_weight *wq = ws[i + q];
+            l.splits[q] = splits;
+            // the second format of a two-format launch (Q6_K beside Q4_K or Q5_K) takes half as long again per step: its
+            // tiles get slices half as long where the device has the room, so that the launch does not wait for them
+            if (q >= l.first_b && splits > 1 && splits < 8 && wgs + tiles_of(wq) * mtiles * splits <= g.cus && nsteps / (splits * 2) >= g.prefill_min_slice) {
+                l.splits[q] = splits * 2;
+                wgs += tiles_of(wq) * mtiles * splits;
+            }
+            // slices of the 256-value formats start on whole blocks (four steps): the kernel stages their raw bytes by block
+            l.split_steps[q] = (nsteps + l.splits[q] - 1) / l.splits[q];
+            if (kq(wq)) l.split_steps[q] = (l.split_steps[q] + 3) & ~3;
+            if (l.splits[q] > 1) l.part_bytes += (size_t)l.splits[q] * rows * wq->n * 4;
+        }
         i = j;
     }
     size_t part_max = 0;
@@ -660,32 +674,39 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     for (int li = 0; li < nlaunch; ++li) {
         const Launch &l = launch[li];
         const jitnn_hip_weight *w = ws[l.first];
+        const bool split = l.splits[0] > 1;  // (the segments of a launch split together or not at all)
         PfSegments sg{}, out{};
+        for (int q = 0; q < 3; ++q) sg.splits[q] = out.splits[q] = 1;
         size_t before = 0;  // floats of partial sums of the segments before this one
+        unsigned gx = 0;
         for (int q = 0; q < l.count; ++q) {
             const jitnn_hip_weight *wq = ws[l.first + q];
             sg.W[q] = wq->dev;
             sg.n[q] = wq->n;
-            sg.tiles[q] = (wq->n + PF_BN - 1) / PF_BN;
-            sg.y[q] = l.splits > 1 ? part + before : (residual ? tmp : ys[l.first + q]);
-            before += (size_t)l.splits * rows * wq->n;
+            sg.tiles[q] = tiles_of(wq);
+            sg.splits[q] = l.splits[q];
+            sg.split_steps[q] = l.split_steps[q];
+            sg.y[q] = split ? part + before : (residual ? tmp : ys[l.first + q]);
+            before += (size_t)l.splits[q] * rows * wq->n;
+            gx += (unsigned)(sg.tiles[q] * sg.splits[q]);
             out.y[q] = ys[l.first + q];
             out.n[q] = wq->n;
+            out.splits[q] = l.splits[q];
         }
-        const float *b1 = l.splits > 1 ? nullptr : bias;
-        const dim3 grid(l.tiles, mtiles, l.splits);
-        if (l.first_b < l.count) prefill_launch_mixed(w->fmt, ws[l.first + l.first_b]->fmt, l.first_b, grid, stream, sg, xo, inv, rows, k, l.split_steps);
-        else if (kq(w)) prefill_launch_k(w->fmt, grid, stream, sg, xo, inv, b1, rows, k, l.split_steps);
-        else prefill_launch_q32(w->fmt, grid, stream, sg, xo, inv, b1, rows, k, l.split_steps);
-        if (l.splits > 1 && l.count > 1) {  // (the stream orders the next launch's partial sums after this join)
+        const float *b1 = split ? nullptr : bias;
+        const dim3 grid(gx, mtiles);
+        if (l.first_b < l.count) prefill_launch_mixed(w->fmt, ws[l.first + l.first_b]->fmt, l.first_b, grid, stream, sg, xo, inv, rows, k);
+        else if (kq(w)) prefill_launch_k(w->fmt, grid, stream, sg, xo, inv, b1, rows, k);
+        else prefill_launch_q32(w->fmt, grid, stream, sg, xo, inv, b1, rows, k);
+        if (split && l.count > 1) {  // (the stream orders the next launch's partial sums after this join)
             size_t count4 = 0;
             for (int q = 0; q < l.count; ++q) count4 += (size_t)rows * sg.n[q] / 4;
             const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
-            prefill_join_group_launch(part, out, rows, l.splits, blocks, stream);
-        } else if (l.splits > 1) {
+            prefill_join_group_launch(part, out, rows, blocks, stream);
+        } else if (split) {
             const size_t count4 = (size_t)rows * w->n / 4;
             const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
-            prefill_join_launch(part, bias, residual, ys[l.first], count4, w->n, l.splits, blocks, stream);
+            prefill_join_launch(part, bias, residual, ys[l.first], count4, w->n, l.splits[0], blocks, stream);
         } else if (residual) {
             const size_t count4 = (size_t)rows * w->n / 4;
             const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
@@ -807,6 +828,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_ROWS_MIN")) g.rows_kernel_min = atoi(e);
     if (const char *e = getenv("JITNN_HIP_PREFILL_GROUP")) g.prefill_group = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_MFMA")) g.prefill_attn_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
@@ -1373,11 +1395,25 @@ int ensure_prefill(jitnn_hip_llama *m, int tokens) {
 
 template <int D>
 int launch_attention_rows(const jitnn_hip_llama *m, int layer, int pos0, int tokens, const float *q, float *att, hipStream_t st) {
-    const int group = m->heads / m->kv, qt = ATT_ROWS / group;
+    const int group = m->heads / m->kv;
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
-    const dim3 grid((tokens + qt - 1) / qt, m->kv);
     const float scale = 1.0f / sqrtf((float)D);
     // prompts beyond the GEMV range have FP16-operand linears on both sides of the attention: FP16 operands here too
+    if (tokens > g.gemv_max_rows && g.prefill_attn_fp16) {
+        if constexpr (D == 64 || D == 128) {
+            if (g.prefill_attn_mfma && group <= AM_ROWS) {
+                const int qt = AM_ROWS / group;
+                const dim3 grid((tokens + qt - 1) / qt, m->kv);
+                constexpr size_t lds = attn_prefill_mfma_lds_bytes<D>();
+                if (int rc = allow_lds((const void *)attn_prefill_mfma_kernel<D>, lds)) return rc;
+                hipLaunchKernelGGL(attn_prefill_mfma_kernel<D>, grid, dim3(AM_THREADS), lds, st, q, m->kc + lo, m->vc + lo, att, m->heads, m->kv, pos0, tokens,
+                                   scale);
+                return JITNN_HIP_OK;
+            }
+        }
+    }
+    const int qt = ATT_ROWS / group;
+    const dim3 grid((tokens + qt - 1) / qt, m->kv);
     if (tokens > g.gemv_max_rows && g.prefill_attn_fp16) {
         constexpr size_t lds = attn_prefill_h_lds_bytes<D>();
         if (int rc = allow_lds((const void *)attn_prefill_h_kernel<D>, lds)) return rc;

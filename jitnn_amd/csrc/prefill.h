@@ -468,11 +468,11 @@ __device__ __forceinline__ void pf_load_lds(PfRaw<FMT> &r, const uint8_t *b, int
     }
 }
 
-// The work of one workgroup: row tile `tile` of the weight W [n, k] against token tile blockIdx.y, K slice blockIdx.z.
+// The work of one workgroup: row tile `tile` of the weight W [n, k] against token tile blockIdx.y, K slice `slice`.
 template <int FMT>
 __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xo, const float *__restrict__ inv_scale,
                                                   const float *__restrict__ bias, float *__restrict__ y, const int m, const int n, const int k,
-                                                  const int split_steps, const int tile) {
+                                                  const int split_steps, const int tile, const int slice) {
     using Stage = PfStage<FMT>;
     constexpr bool STAGED = Stage::ON;
     extern __shared__ __align__(16) uint8_t pf_smem[];  // pf_lds_bytes<FMT>()
@@ -511,11 +511,11 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
     f16x8 ah[4];
     PfRaw<FMT> raw[2];
     f16x8 bq[3][2][4];
-    // this workgroup's K steps: all of them, or slice blockIdx.z of split_steps steps when the launch splits K (then y
+    // this workgroup's K steps: all of them, or slice `slice` of split_steps steps when the launch splits K (then y
     // is the slice's own [m, n] array of partial sums, to be added up by prefill_join_kernel; a slice of a staged
     // format starts on a multiple of four steps)
-    const int sbeg = blockIdx.z * split_steps, nsteps = min((k + PF_BK - 1) / PF_BK, sbeg + split_steps);
-    y += (size_t)blockIdx.z * m * n;
+    const int sbeg = slice * split_steps, nsteps = min((k + PF_BK - 1) / PF_BK, sbeg + split_steps);
+    y += (size_t)slice * m * n;
     auto wk = [&](int s) { return min(min(s, nsteps - 1) * PF_BK + 32 * dhalf, k - 32); };  // first value this thread decodes in step s
     auto fetch_w = [&](PfRaw<FMT> &r, int s) { pf_load<FMT>(r, wrow, wk(s)); };
     auto fetch_b = [&](f16x8(&b)[2][4], int s) {
@@ -683,29 +683,31 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
 
 // Up to three weights of one activation in one launch (the q, k and v projections of a layer): their row tiles are
 // numbered one after the other along blockIdx.x, every workgroup works on its weight exactly as in a launch of its own.
-__device__ __forceinline__ void pf_locate(const PfSegments &sg, int &seg, int &tile) {
+__device__ __forceinline__ void pf_locate(const PfSegments &sg, int &seg, int &tile, int &slice) {
     seg = 0;
-    tile = blockIdx.x;
-    if (tile >= sg.tiles[0]) {
-        tile -= sg.tiles[0];
+    int idx = blockIdx.x;
+    if (idx >= sg.tiles[0] * sg.splits[0]) {
+        idx -= sg.tiles[0] * sg.splits[0];
         seg = 1;
-        if (tile >= sg.tiles[1]) {
-            tile -= sg.tiles[1];
+        if (idx >= sg.tiles[1] * sg.splits[1]) {
+            idx -= sg.tiles[1] * sg.splits[1];
             seg = 2;
         }
     }
+    slice = idx / sg.tiles[seg];
+    tile = idx - slice * sg.tiles[seg];
 }
 
-// grid: (row tiles of all segments, token tiles, K slices); 256 threads; pf_lds_bytes<FMT>() of dynamic LDS.
-//   sg.y[i]: [m, n[i]], or for a launch that splits K the first slice's array of partial sums (slice z at + z m n[i]);
+// grid: (row tiles x K slices of all segments, token tiles); 256 threads; pf_lds_bytes<FMT>() of dynamic LDS.
+//   sg.y[i]: [m, n[i]], or for a segment that splits K the first slice's array of partial sums (slice z at + z m n[i]);
 //   bias: one segment only.
 template <int FMT>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_kernel(const PfSegments sg, const _Float16 *__restrict__ xo,
                                                             const float *__restrict__ inv_scale, const float *__restrict__ bias,
-                                                            int m, int k, int split_steps) {
-    int seg, tile;
-    pf_locate(sg, seg, tile);
-    prefill_mfma_body<FMT>(sg.W[seg], xo, inv_scale, bias, sg.y[seg], m, sg.n[seg], k, split_steps, tile);
+                                                            int m, int k) {
+    int seg, tile, slice;
+    pf_locate(sg, seg, tile, slice);
+    prefill_mfma_body<FMT>(sg.W[seg], xo, inv_scale, bias, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
 }
 
 // The same for weights of two formats (a Q4_K_M layer keeps q and k as Q4_K and v as Q6_K): segments below first_b are
@@ -713,11 +715,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
 template <int FA, int FB>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_mixed_kernel(const PfSegments sg, const int first_b,
                                                             const _Float16 *__restrict__ xo, const float *__restrict__ inv_scale,
-                                                            int m, int k, int split_steps) {
-    int seg, tile;
-    pf_locate(sg, seg, tile);
-    if (seg < first_b) prefill_mfma_body<FA>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, split_steps, tile);
-    else prefill_mfma_body<FB>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, split_steps, tile);
+                                                            int m, int k) {
+    int seg, tile, slice;
+    pf_locate(sg, seg, tile, slice);
+    if (seg < first_b) prefill_mfma_body<FA>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+    else prefill_mfma_body<FB>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
 }
 
 // y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]) (+ res[tok, row]), slices in order: the second half of a
@@ -751,14 +753,16 @@ static __global__ void __launch_bounds__(256) prefill_join_kernel(const float *_
     }
 }
 
-// The join for a launch of several segments: part holds, segment after segment, `splits` arrays [m, n[i]] of partial sums;
-// y[i][tok, row] = their sum in slice order.  n[i] multiples of 4.
-static __global__ void __launch_bounds__(256) prefill_join_group_kernel(const float *__restrict__ part, const PfSegments sg, int m, int splits) {
+// The join for a launch of several segments: part holds, segment after segment, splits[i] arrays [m, n[i]] of partial
+// sums; y[i][tok, row] = their sum in slice order.  n[i] multiples of 4.
+static __global__ void __launch_bounds__(256) prefill_join_group_kernel(const float *__restrict__ part, const PfSegments sg, int m) {
     const size_t c0 = (size_t)m * sg.n[0] / 4, c1 = (size_t)m * sg.n[1] / 4, c2 = (size_t)m * sg.n[2] / 4;
+    const size_t o1 = c0 * sg.splits[0], o2 = o1 + c1 * sg.splits[1];
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < c0 + c1 + c2; i += (size_t)gridDim.x * 256) {
         const int seg = (i >= c0) + (i >= c0 + c1);
-        const size_t before = seg == 0 ? 0 : seg == 1 ? c0 : c0 + c1, cnt = seg == 0 ? c0 : seg == 1 ? c1 : c2, local = i - before;
-        const float4 *p = reinterpret_cast<const float4 *>(part) + before * splits + local;
+        const size_t cnt = seg == 0 ? c0 : seg == 1 ? c1 : c2, local = i - (seg == 0 ? 0 : seg == 1 ? c0 : c0 + c1);
+        const float4 *p = reinterpret_cast<const float4 *>(part) + (seg == 0 ? 0 : seg == 1 ? o1 : o2) + local;
+        const int splits = sg.splits[seg];
         float4 a = p[0];
         for (int z = 1; z < splits; ++z) {
             const float4 b = p[(size_t)z * cnt];

@@ -13,12 +13,11 @@ KernelRef prefill_kernel_k(int fmt) {
     }
 }
 
-void prefill_launch_k(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m, int k,
-                      int split_steps) {
+void prefill_launch_k(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m, int k) {
     switch (fmt) {
-    case F_Q4_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_K>, grid, dim3(256), pf_lds_bytes<F_Q4_K>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
-    case F_Q5_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q5_K>, grid, dim3(256), pf_lds_bytes<F_Q5_K>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
-    case F_Q6_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q6_K>, grid, dim3(256), pf_lds_bytes<F_Q6_K>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
+    case F_Q4_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_K>, grid, dim3(256), pf_lds_bytes<F_Q4_K>(), s, sg, xo, inv_scale, bias, m, k); break;
+    case F_Q5_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q5_K>, grid, dim3(256), pf_lds_bytes<F_Q5_K>(), s, sg, xo, inv_scale, bias, m, k); break;
+    case F_Q6_K: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q6_K>, grid, dim3(256), pf_lds_bytes<F_Q6_K>(), s, sg, xo, inv_scale, bias, m, k); break;
     default: break;
     }
 }

@@ -14,13 +14,11 @@ KernelRef prefill_kernel_mixed(int fmt_a, int fmt_b) {
 }
 
 void prefill_launch_mixed(int fmt_a, int fmt_b, int first_b, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale,
-                          int m, int k, int split_steps) {
+                          int m, int k) {
     if (fmt_a == F_Q4_K && fmt_b == F_Q6_K)
-        hipLaunchKernelGGL((prefill_mfma_mixed_kernel<F_Q4_K, F_Q6_K>), grid, dim3(256), (mixed_lds<F_Q4_K, F_Q6_K>()), s, sg, first_b, xo, inv_scale, m, k,
-                           split_steps);
+        hipLaunchKernelGGL((prefill_mfma_mixed_kernel<F_Q4_K, F_Q6_K>), grid, dim3(256), (mixed_lds<F_Q4_K, F_Q6_K>()), s, sg, first_b, xo, inv_scale, m, k);
     else if (fmt_a == F_Q5_K && fmt_b == F_Q6_K)
-        hipLaunchKernelGGL((prefill_mfma_mixed_kernel<F_Q5_K, F_Q6_K>), grid, dim3(256), (mixed_lds<F_Q5_K, F_Q6_K>()), s, sg, first_b, xo, inv_scale, m, k,
-                           split_steps);
+        hipLaunchKernelGGL((prefill_mfma_mixed_kernel<F_Q5_K, F_Q6_K>), grid, dim3(256), (mixed_lds<F_Q5_K, F_Q6_K>()), s, sg, first_b, xo, inv_scale, m, k);
 }
 
 }  // namespace jitnn

@@ -13,12 +13,11 @@ KernelRef prefill_kernel_q32(int fmt) {
     }
 }
 
-void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m, int k,
-                      int split_steps) {
+void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m, int k) {
     switch (fmt) {
-    case F_Q4_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_0>, grid, dim3(256), pf_lds_bytes<F_Q4_0>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
-    case F_Q4_1: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_1>, grid, dim3(256), pf_lds_bytes<F_Q4_1>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
-    case F_Q8_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q8_0>, grid, dim3(256), pf_lds_bytes<F_Q8_0>(), s, sg, xo, inv_scale, bias, m, k, split_steps); break;
+    case F_Q4_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_0>, grid, dim3(256), pf_lds_bytes<F_Q4_0>(), s, sg, xo, inv_scale, bias, m, k); break;
+    case F_Q4_1: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_1>, grid, dim3(256), pf_lds_bytes<F_Q4_1>(), s, sg, xo, inv_scale, bias, m, k); break;
+    case F_Q8_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q8_0>, grid, dim3(256), pf_lds_bytes<F_Q8_0>(), s, sg, xo, inv_scale, bias, m, k); break;
     default: break;
     }
 }
@@ -50,8 +49,8 @@ void prefill_join_launch(const float *part, const float *bias, const float *res,
     hipLaunchKernelGGL(prefill_join_kernel, dim3(blocks), dim3(256), 0, s, part, bias, res, y, count4, n, splits);
 }
 
-void prefill_join_group_launch(const float *part, const PfSegments &sg, int m, int splits, unsigned blocks, hipStream_t s) {
-    hipLaunchKernelGGL(prefill_join_group_kernel, dim3(blocks), dim3(256), 0, s, part, sg, m, splits);
+void prefill_join_group_launch(const float *part, const PfSegments &sg, int m, unsigned blocks, hipStream_t s) {
+    hipLaunchKernelGGL(prefill_join_group_kernel, dim3(blocks), dim3(256), 0, s, part, sg, m);
 }
 
 }  // namespace jitnn

@@ -16,12 +16,17 @@ struct KernelRef {
 };
 
 // Up to three weights [n[i], k] of one activation in one launch of the many-row kernel: their row tiles (tiles[i] of
-// them, 128 rows each) are numbered one after the other.  Unused segments: n = tiles = 0.
+// them, 128 rows each) are numbered one after the other along blockIdx.x, slice after slice when the segment splits K:
+// segment i takes tiles[i] * splits[i] workgroups, slice z of it the K steps [z * split_steps[i], (z + 1) * split_steps[i])
+// and the array y[i] + z * m * n[i] (partial sums, to be joined).  Segments may split differently: the tiles of a format
+// that takes longer per step get shorter slices.  Unused segments: n = tiles = 0, splits = 1.
 struct PfSegments {
     const uint8_t *W[3];
     float *y[3];
     int n[3];
     int tiles[3];
+    int splits[3];
+    int split_steps[3];
 };
 
 // ---- prefill_k.hip (Q4_K, Q5_K, Q6_K), prefill_q32.hip (Q4_0, Q4_1, Q8_0): prefill_mfma_kernel<fmt>;
@@ -29,12 +34,11 @@ struct PfSegments {
 KernelRef prefill_kernel_k(int fmt);
 KernelRef prefill_kernel_q32(int fmt);
 KernelRef prefill_kernel_mixed(int fmt_a, int fmt_b);  // fn == nullptr: this pair has no kernel
-void prefill_launch_k(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m, int k,
-                      int split_steps);
+void prefill_launch_k(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m, int k);
 void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale, const float *bias, int m,
-                        int k, int split_steps);
+                        int k);
 void prefill_launch_mixed(int fmt_a, int fmt_b, int first_b, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale,
-                          int m, int k, int split_steps);
+                          int m, int k);
 // activation preparation and the join of K slices (prefill_q32.hip)
 // (norm_w != nullptr: RMSNorm with that weight and eps fused into the preparation; swiglu_up != nullptr: the activations
 // are silu(x) * swiglu_up, both [rows, k] - either only where prefill_prepare_fuses_norm(k))
@@ -43,8 +47,8 @@ void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Flo
                             const float *swiglu_up, hipStream_t s);
 void prefill_join_launch(const float *part, const float *bias, const float *res, float *y, size_t count4, int n, int splits, unsigned blocks,
                          hipStream_t s);
-// the join of a launch of several segments: part = per segment `splits` arrays [m, n[i]], one segment after the other
-void prefill_join_group_launch(const float *part, const PfSegments &sg, int m, int splits, unsigned blocks, hipStream_t s);
+// the join of a launch of several segments: part = per segment splits[i] arrays [m, n[i]], one segment after the other
+void prefill_join_group_launch(const float *part, const PfSegments &sg, int m, unsigned blocks, hipStream_t s);
 
 // ---- gemv_mfma.hip: gemv_mfma_kernel<fmt>
 KernelRef gemv_mfma_kernel_ref(int fmt);
