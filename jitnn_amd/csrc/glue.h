@@ -610,6 +610,7 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
     const int r = 16 * wave + n, tq = r / group, hq = r - tq * group;
     const bool live = r < rows && t0 + tq < T;
     const int jmax = pos0 + t0 + tq;  // the last key the row sees
+    const float scale2 = scale * 1.44269504088896341f;
     f16x8 qb[DB];
     {
         const float *qp = q + ((size_t)(t0 + (live ? tq : 0)) * heads + g * group + (live ? hq : 0)) * D + 8 * kq;
@@ -685,29 +686,53 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
                 st[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[b], st[t], 0, 0, 0);
             }
         }
-        // ---- running softmax of the row
+        // ---- running softmax of the row, in base 2: exp(scale s - m) = exp2(scale2 s - m2).  Only the chunks that reach
+        // past the first row's last key (the diagonal of the block, and everything for rows that do not exist) need the
+        // mask; in the others every score counts and no -inf can appear.
         float mc = -INFINITY;
+        const bool masked = j0 + CH - 1 > pos0 + t0 || !(t0 + QT <= T && rows == AM_ROWS);  // workgroup-uniform
+        if (masked) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const bool seen = live && j0 + 16 * t + 4 * kq + i <= jmax;
-                st[t][i] = seen ? st[t][i] * scale : -INFINITY;
-                mc = fmaxf(mc, st[t][i]);
-            }
+                for (int i = 0; i < 4; ++i) {
+                    const bool seen = live && j0 + 16 * t + 4 * kq + i <= jmax;
+                    st[t][i] = seen ? st[t][i] * scale2 : -INFINITY;
+                    mc = fmaxf(mc, st[t][i]);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    st[t][i] *= scale2;
+                    mc = fmaxf(mc, st[t][i]);
+                }
+        }
         mc = fmaxf(mc, __shfl_xor(mc, 16));
         mc = fmaxf(mc, __shfl_xor(mc, 32));
         const float mn = fmaxf(mrun, mc);
-        const float alpha = mrun > -INFINITY ? __expf(mrun - mn) : 0.f;
+        const float alpha = mrun > -INFINITY ? __builtin_amdgcn_exp2f(mrun - mn) : 0.f;
         float ls = 0.f;
+        if (masked) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float pv = st[t][i] > -INFINITY ? __expf(st[t][i] - mn) : 0.f;
-                st[t][i] = pv;
-                ls += pv;
-            }
+                for (int i = 0; i < 4; ++i) {
+                    const float pv = st[t][i] > -INFINITY ? __builtin_amdgcn_exp2f(st[t][i] - mn) : 0.f;
+                    st[t][i] = pv;
+                    ls += pv;
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float pv = __builtin_amdgcn_exp2f(st[t][i] - mn);
+                    st[t][i] = pv;
+                    ls += pv;
+                }
+        }
         lrun = lrun * alpha + ls;
         mrun = mn;
         if (kq == 0) fx[16 * wave + n] = alpha;
