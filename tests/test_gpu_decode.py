@@ -175,6 +175,35 @@ def test_prefill_head_shapes(jn, heads, kv_heads, head_dim, tokens, bar):
     dec.close()
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim", [(4, 4, 128), (8, 2, 128), (8, 1, 64), (5, 1, 64), (6, 3, 128)])
+def test_prefill_long_prompt_attention(jn, heads, kv_heads, head_dim):
+    """The matrix-core attention of long prompts on several key chunks: groups of 1, 2, 4, 5 and 8 query heads per key/value
+    head (with 5 the 128-row block of a workgroup is ragged), 19 cached positions in front of 150 tokens - three chunks of
+    64 keys, the last partly filled, token blocks that end inside the prompt - against the oracle run token by token."""
+    tokens, pos0 = 150, 19
+    cfg = dict(layers=1, d_model=256, heads=heads, kv_heads=kv_heads, head_dim=head_dim, ffn=256, vocab=200, max_ctx=192, rms_eps=1e-5,
+               rope_theta=5e5)
+    dec, layers, out_norm, out_w = build(jn, cfg, 23, {s: "Q8_0" for s in SLOTS}, "Q8_0")
+    rng = np.random.default_rng(6)
+    kc = np.zeros((1, cfg["max_ctx"], kv_heads, head_dim), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :pos0] = rng.standard_normal(kc[:, :pos0].shape)
+    vc[:, :pos0] = rng.standard_normal(vc[:, :pos0].shape)
+    dec.kv_write(0, 0, kc[0, :pos0], vc[0, :pos0])
+    x = rng.standard_normal((tokens, cfg["d_model"])).astype(np.float32)
+    refs = [decode_ref(cfg, layers, out_norm, out_w, kc, vc, x[t], pos0 + t) for t in range(tokens)]
+    y = dec.prefill(x, pos0)
+    assert norm_err(y, refs[-1]) <= 5e-3, norm_err(y, refs[-1])
+    k, v = dec.kv_read(0, pos0, tokens)
+    assert norm_err(k, kc[0, pos0:pos0 + tokens]) <= 2e-3 and norm_err(v, vc[0, pos0:pos0 + tokens]) <= 2e-3
+    # a shorter prompt on a fresh cache ends in the middle of a token block: its last token must match too
+    dec.kv_write(0, 0, kc[0, :pos0], vc[0, :pos0])
+    short = 97
+    y = dec.prefill(x[:short], pos0)
+    assert norm_err(y, refs[short - 1]) <= 5e-3, norm_err(y, refs[short - 1])
+    dec.close()
+
+
 def test_prefill_argument_checks(jn):
     cfg = dict(layers=1, d_model=256, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=64, max_ctx=8, rms_eps=1e-5, rope_theta=1e4)
     dec, *_ = build(jn, cfg, 13, {s: "Q8_0" for s in SLOTS}, "Q8_0")
