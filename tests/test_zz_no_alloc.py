@@ -1,7 +1,8 @@
 """jitnn_hip_linear_noalloc_dev - the entry point that takes the scratch of a many-row launch from the library's fixed
 device array instead of a buffer it may have to allocate - against jitnn_hip_linear_dev on the same inputs: the same
-kernels on the same operands, so the same bits.  Two calls in a row, the second smaller (the array keeps the first
-call's contents), then the GEMV range (no scratch at all) and the size limit."""
+kernels on the same operands, so the same bits.  Calls in a row, each smaller than the first (the array keeps the earlier
+calls' contents): the many-row kernel with K slices, the one-pass kernel for 9..64 rows, the GEMV range (no scratch at
+all); then the size limit."""
 import ctypes as C
 
 import numpy as np
@@ -39,7 +40,10 @@ def test_noalloc_linear_matches_linear_dev(jn):
     rng = np.random.default_rng(12)
     g = torch.Generator(device="cuda").manual_seed(12)
     # 4096 x 4096 at 512 rows splits K into slices (partial sums in the scratch); the second call is smaller in every way
-    calls = [("Q4_K", 4096, 4096, 512, True), ("Q6_K", 300, 1024, 97, False), ("Q8_0", 131, 32 * 9, 70, True), ("Q4_K", 192, 2048, 5, False)]
+    # (then: a ragged Q6_K launch, the one-pass kernel for 9..64 rows of Q4_K / Q5_K - its prepared operands live in the
+    # scratch too -, a 32-value format, and a GEMV call that needs no scratch at all)
+    calls = [("Q4_K", 4096, 4096, 512, True), ("Q6_K", 300, 1024, 97, False), ("Q4_K", 640, 2048, 40, True), ("Q5_K", 100, 1024, 17, False),
+             ("Q8_0", 131, 32 * 9, 70, True), ("Q4_K", 192, 2048, 5, False)]
     for fmt, n, k, rows, with_bias in calls:
         w = jn.Tensor.quantized(jn.DType[fmt], random_valid_blocks(rng, fmt, n, k), n, k)
         x = torch.randn(rows, k, device="cuda", generator=g)
