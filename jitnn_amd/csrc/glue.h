@@ -564,9 +564,12 @@ __global__ void __launch_bounds__(256) attn_prefill_h_kernel(const float *__rest
 }
 
 // The same attention on the matrix cores (v_mfma_f32_16x16x32_f16, FP16 operands, FP32 accumulation and softmax), for
-// heads of 64 or 128 values.  A workgroup of AM_WAVES waves takes AM_ROWS (token, query head) rows of one key/value head,
-// every wave 16 of them, and walks the keys in chunks of AM_CH staged once in LDS as binary16 for all of them (the more
-// rows share a chunk, the fewer times the cache is read: 128 rows read it half as often as 64).
+// heads of 64 or 128 values.  A workgroup of eight waves takes AM_ROWS = 64 (token, query head) rows of one key/value head
+// and walks the keys in chunks of AM_CH = 64 staged once in LDS as binary16 for all of them; a wave takes 16 rows and ONE
+// HALF of every chunk's keys (waves 0-3 the first 32, waves 4-7 the last 32), keeps its own running maximum, sum and
+// output, and the two halves of a row meet once, at the end, through LDS.  What limits this kernel is the length of the
+// dependent chain a wave walks per chunk (operand reads, MFMAs, softmax, MFMAs), not any unit's throughput: 16 rows x 64
+// keys per wave took 20 us per layer at 512 tokens whether a workgroup held 64 or 128 rows.
 //   * scores, transposed: S^T = K Q^T, so that a lane ends up with the scores of ONE query row (column lane % 16 of the
 //     result) against the keys 4 (lane / 16) + i of every 16-key tile - the running softmax of a row needs its chunk
 //     maximum from the three other lanes that hold the row's other keys (two shuffles), the row sum stays a per-lane
@@ -580,10 +583,11 @@ __global__ void __launch_bounds__(256) attn_prefill_h_kernel(const float *__rest
 //   * keys and values of the chunk after next are requested into registers while the current one is multiplied; the LDS
 //     tiles are double-buffered, one workgroup barrier per chunk; nothing about the loads is conditional (chunks past
 //     the end repeat the last one, keys past the last visible one re-read it and are masked).
-constexpr int AM_ROWS = 128, AM_CH = 64, AM_WAVES = AM_ROWS / 16, AM_THREADS = 64 * AM_WAVES;
+constexpr int AM_ROWS = 64, AM_CH = 64, AM_WAVES = 2 * (AM_ROWS / 16), AM_THREADS = 64 * AM_WAVES;
 template <int D>
 constexpr size_t attn_prefill_mfma_lds_bytes() {
-    return (size_t)2 * ((size_t)AM_CH * (D + 8) + (size_t)D * (AM_CH + 8)) * sizeof(_Float16) + AM_WAVES * 16 * sizeof(float);
+    return (size_t)2 * ((size_t)AM_CH * (D + 8) + (size_t)D * (AM_CH + 8)) * sizeof(_Float16) + AM_WAVES * 16 * sizeof(float);  // (the
+    // tiles also hold the second halves' outputs at the end: 4 waves x (16 x D + 32) floats fit for D >= 64)
 }
 template <int D>
 __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const float *__restrict__ q, const float *__restrict__ kcache,
@@ -598,6 +602,7 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
     _Float16 *Vt = Kh + 2 * CH * KP;                        // [2][D][VP]: values transposed, keys in slot order
     float *fx = reinterpret_cast<float *>(Vt + 2 * D * VP);  // [AM_WAVES][16]: a factor per row, from score layout to output layout
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, kq = lane >> 4;
+    const int rt = wave & 3, half = wave >> 2;  // this wave's 16 rows of the block and its half of every chunk's keys
     const int group = heads / kv_heads, QT = AM_ROWS / group, rows = QT * group;
     const int g = blockIdx.y;
     // early token blocks walk few keys, late ones many: half of the key/value heads take the blocks in reverse
@@ -607,7 +612,7 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
     const int jlast = pos0 + tl;               // last key any row of the block sees
     const int nchunks = jlast / CH + 1;
     // ---- this lane's query row (score layout): row r of the block, as the second operand of S^T = K Q^T
-    const int r = 16 * wave + n, tq = r / group, hq = r - tq * group;
+    const int r = 16 * rt + n, tq = r / group, hq = r - tq * group;
     const bool live = r < rows && t0 + tq < T;
     const int jmax = pos0 + t0 + tq;  // the last key the row sees
     const float scale2 = scale * 1.44269504088896341f;
@@ -675,14 +680,14 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
         fetch(c + 2);
         const _Float16 *kh = Kh + (c & 1) * CH * KP, *vt = Vt + (c & 1) * D * VP;
         const int j0 = c * CH;
-        // ---- S^T: four tiles of 16 keys; the lane ends up with keys j0 + 16 t + 4 kq + i of its row
-        f32x4 st[4];
+        // ---- S^T: this half's two tiles of 16 keys; the lane ends up with keys j0 + 32 half + 16 t + 4 kq + i of its row
+        f32x4 st[2];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
+        for (int t = 0; t < 2; ++t) {
             st[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int b = 0; b < DB; ++b) {
-                const f16x8 a = *reinterpret_cast<const f16x8 *>(&kh[(16 * t + n) * KP + 32 * b + 8 * kq]);
+                const f16x8 a = *reinterpret_cast<const f16x8 *>(&kh[(32 * half + 16 * t + n) * KP + 32 * b + 8 * kq]);
                 st[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qb[b], st[t], 0, 0, 0);
             }
         }
@@ -693,16 +698,16 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
         const bool masked = j0 + CH - 1 > pos0 + t0 || !(t0 + QT <= T && rows == AM_ROWS);  // workgroup-uniform
         if (masked) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const bool seen = live && j0 + 16 * t + 4 * kq + i <= jmax;
+                    const bool seen = live && j0 + 32 * half + 16 * t + 4 * kq + i <= jmax;
                     st[t][i] = seen ? st[t][i] * scale2 : -INFINITY;
                     mc = fmaxf(mc, st[t][i]);
                 }
         } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     st[t][i] *= scale2;
@@ -711,12 +716,12 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
         }
         mc = fmaxf(mc, __shfl_xor(mc, 16));
         mc = fmaxf(mc, __shfl_xor(mc, 32));
-        const float mn = fmaxf(mrun, mc);
+        const float mn = fmaxf(mrun, mc);  // (-inf while this half has not met a visible key of the row yet)
         const float alpha = mrun > -INFINITY ? __builtin_amdgcn_exp2f(mrun - mn) : 0.f;
         float ls = 0.f;
         if (masked) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float pv = st[t][i] > -INFINITY ? __builtin_amdgcn_exp2f(st[t][i] - mn) : 0.f;
@@ -725,7 +730,7 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
                 }
         } else {
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const float pv = __builtin_amdgcn_exp2f(st[t][i] - mn);
@@ -745,30 +750,53 @@ __global__ void __launch_bounds__(AM_THREADS) attn_prefill_mfma_kernel(const flo
             o[t][2] *= al[2];
             o[t][3] *= al[3];
         }
-        // ---- O += P V, two steps of 32 keys
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const f16x8 pa = {(_Float16)st[2 * u][0], (_Float16)st[2 * u][1], (_Float16)st[2 * u][2], (_Float16)st[2 * u][3],
-                              (_Float16)st[2 * u + 1][0], (_Float16)st[2 * u + 1][1], (_Float16)st[2 * u + 1][2], (_Float16)st[2 * u + 1][3]};
+        // ---- O += P V over this half's 32 keys
+        {
+            const f16x8 pa = {(_Float16)st[0][0], (_Float16)st[0][1], (_Float16)st[0][2], (_Float16)st[0][3],
+                              (_Float16)st[1][0], (_Float16)st[1][1], (_Float16)st[1][2], (_Float16)st[1][3]};
 #pragma unroll
             for (int t = 0; t < DT; ++t) {
-                const f16x8 vb = *reinterpret_cast<const f16x8 *>(&vt[(16 * t + n) * VP + 32 * u + 8 * kq]);
+                const f16x8 vb = *reinterpret_cast<const f16x8 *>(&vt[(16 * t + n) * VP + 32 * half + 8 * kq]);
                 o[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, vb, o[t], 0, 0, 0);
             }
         }
     }
-    // ---- the row sums meet, the rows are normalised and written: the lane holds rows 4 kq + i, values 16 t + n
+    // ---- the two halves of a row meet: the waves of the second half leave maximum, sum and output in LDS (the tiles are
+    // free after the last chunk), the waves of the first half combine, normalise and write.  The lane holds rows
+    // 4 kq + i, values 16 t + n of the output, and - in score layout - the statistics of row n.
     lrun += __shfl_xor(lrun, 16);
     lrun += __shfl_xor(lrun, 32);
-    if (kq == 0) fx[16 * wave + n] = live ? 1.f / lrun : 0.f;
-    const f32x4 il = *reinterpret_cast<const f32x4 *>(&fx[16 * wave + 4 * kq]);
+    __syncthreads();  // every wave is done with the tiles
+    float *xo = att_smem + rt * (16 * D + 32);  // [DT][4][64] output, then 16 maxima, 16 sums
+    if (half == 1) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ro = 16 * wave + 4 * kq + i, to = ro / group, ho = ro - to * group;
-        if (ro < rows && t0 + to < T) {
-            float *op = out + ((size_t)(t0 + to) * heads + g * group + ho) * D + n;
+        for (int t = 0; t < DT; ++t)
 #pragma unroll
-            for (int t = 0; t < DT; ++t) op[16 * t] = o[t][i] * il[i];
+            for (int i = 0; i < 4; ++i) xo[(t * 4 + i) * 64 + lane] = o[t][i];
+        if (kq == 0) {
+            xo[16 * D + n] = mrun;
+            xo[16 * D + 16 + n] = lrun;
+        }
+    }
+    __syncthreads();
+    if (half == 0) {
+        const float m1 = xo[16 * D + n], l1 = xo[16 * D + 16 + n];
+        const float mm = fmaxf(mrun, m1);
+        const float a0 = mrun > -INFINITY ? __builtin_amdgcn_exp2f(mrun - mm) : 0.f, a1 = m1 > -INFINITY ? __builtin_amdgcn_exp2f(m1 - mm) : 0.f;
+        const float il = live ? 1.f / (lrun * a0 + l1 * a1) : 0.f;
+        if (kq == 0) {
+            fx[16 * wave + n] = a0 * il;
+            fx[16 * (wave + 4) + n] = a1 * il;
+        }
+        const f32x4 f0 = *reinterpret_cast<const f32x4 *>(&fx[16 * wave + 4 * kq]), f1 = *reinterpret_cast<const f32x4 *>(&fx[16 * (wave + 4) + 4 * kq]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int ro = 16 * rt + 4 * kq + i, to = ro / group, ho = ro - to * group;
+            if (ro < rows && t0 + to < T) {
+                float *op = out + ((size_t)(t0 + to) * heads + g * group + ho) * D + n;
+#pragma unroll
+                for (int t = 0; t < DT; ++t) op[16 * t] = o[t][i] * f0[i] + xo[(t * 4 + i) * 64 + lane] * f1[i];
+            }
         }
     }
 }
