@@ -387,8 +387,10 @@ def bench_decode(torch, lib, steps, warmup):
     return out
 
 
-def bench_prefill(torch, lib, steps=20):
-    """512-token linears through the MFMA path at the layer shapes of config 5: achieved TFLOP/s (2*M*N*K per call)."""
+def bench_prefill(torch, lib, steps=20, with_cpu=True):
+    """512-token linears through the MFMA path at the layer shapes of config 5: achieved TFLOP/s (2*M*N*K per call), and beside
+    each the reference's CPU route for a 512-row linear (dequantise on one thread + the multithreaded FP32 GEMM) on the same
+    weight bytes and activations."""
     res = {}
     for name, fmt, n, k in (("q4_k_14336x4096", "Q4_K", 14336, 4096), ("q6_k_4096x14336", "Q6_K", 4096, 14336), ("q4_k_4096x4096", "Q4_K", 4096, 4096)):
         t = quantized_device_weight(torch, lib, fmt, n, k, 1060)
@@ -419,6 +421,22 @@ def bench_prefill(torch, lib, steps=20):
         err = float(np.abs(y.cpu().numpy()[:, sel] - ref).max() / np.abs(ref).max())
         res[name] = {"workload": f"{fmt} linear {n}x{k}, 512 rows (MFMA path)", "ms": ms, "TFLOPs": flops / ms / 1e9,
                      "pct_of_fp16_peak": flops / ms / 1e9 / 2500.0 * 100, "parity_norm_err": err}
+        if with_cpu:
+            threads = oracle.cpu_threads()
+            xh, rawh = x.cpu().numpy(), t.cpu().numpy()
+            runs = []
+            t_all = time.perf_counter()
+            while len(runs) < 3 and (not runs or time.perf_counter() - t_all < 3.0):
+                t0 = time.perf_counter()
+                _, t_deq, t_mm = oracle.dequant_gemm(BLOCK[fmt][0], xh, rawh, None, n, k, threads)
+                runs.append((time.perf_counter() - t0, t_deq, t_mm))
+            med = sorted(runs)[len(runs) // 2]
+            res[name]["cpu_baseline"] = {"value": flops / med[0] / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port", "ms": med[0] * 1e3,
+                                         "dequantize_ms": med[1] * 1e3, "pack_and_gemm_ms": med[2] * 1e3, "route": "dequant_gemm",
+                                         "sample": f"the full {fmt} {n}x{k} linear on 512 rows, median of {len(runs)} runs of the C restatement of "
+                                                   f"Gguf.dequantize (one thread) + the packed K-blocked FP32 GEMM of cpu/Gemm.java on {threads} "
+                                                   f"threads, {oracle.cpu_vector_lanes() * 32}-bit vectors"}
+            del xh, rawh
         lib.lib.jitnn_hip_weight_free(h)
         del t, x, y
     # the seven linears of one layer of config 5 on 512 tokens, back to back (attention and norms are not part of this path)
@@ -529,7 +547,7 @@ def main() -> int:
         if not only or "decode" in only:
             decode = bench_decode(torch, lib, steps=30, warmup=3)
         if (not only or "prefill" in only) and not a.quick:
-            prefill = bench_prefill(torch, lib)
+            prefill = bench_prefill(torch, lib, with_cpu=not a.no_cpu)
 
     ms = head["us_per_step_wall"] / 1e3
     line = {
