@@ -530,6 +530,7 @@ def main() -> int:
             ("q4_k_14336x4096_b16", "Q4_K", 14336, 4096, 16, 16, 1030),
             ("q4_k_14336x4096_b40", "Q4_K", 14336, 4096, 40, 16, 1030),
             ("q4_k_14336x4096_b64", "Q4_K", 14336, 4096, 64, 16, 1030),
+            ("q6_k_4096x14336_b40", "Q6_K", 4096, 14336, 40, 8, 1045),
             ("q6_k_128256x4096_b1", "Q6_K", 128256, 4096, 1, 2, 1040),
         ]
         for name, fmt, n, k, b, copies, seed in extra:

@@ -28,17 +28,19 @@ namespace jitnn {
 constexpr int GR_WAVES = 8, GR_THREADS = GR_WAVES * 64;
 constexpr int GR_MAX_GROUPS = 8;            // groups of eight activation rows: up to 64 rows
 constexpr int GR_OP_HALVES = 9 * 512;       // per (group, column): eight sub-block operands and the block-sum operand, 64 lanes x 8 halves each
-constexpr int GR_T = 2;                 // weight tiles a wave holds as operands at a time
+constexpr int GR_T_MAX = 2;             // weight tiles a wave holds as operands at a time, at most (the kernel's parameter T)
 
 __host__ __device__ constexpr size_t gemv_rows_ops_bytes(int groups, int k) { return (size_t)groups * (k / 256) * GR_OP_HALVES * 2; }
 __host__ __device__ constexpr size_t gemv_rows_inv_bytes(int groups, int k) { return (size_t)groups * (k / 256) * 8 * sizeof(float); }
-__host__ __device__ constexpr size_t gemv_rows_lds_bytes() { return (size_t)GR_T * GR_MAX_GROUPS * GR_THREADS * sizeof(float2); }
+__host__ __device__ constexpr size_t gemv_rows_lds_bytes(int tiles_per_wave) { return (size_t)tiles_per_wave * GR_MAX_GROUPS * GR_THREADS * sizeof(float2); }
 
 // One wave per (group g = blockIdx.y, column c = blockIdx.x): x [rows, k] -> operands.
 // Operand s < 8 (sub-block s of the column): lane m + 16 kq holds, for operand row m = 2 b + part (b = activation row of
 // the group, part 0 = hi, 1 = lo), the eight values 8 kq .. 8 kq + 7 of the sub-block in the order 0 2 1 3 4 6 5 7 - the
-// order in which the weight decoders emit the bytes of a dword.  Operand 8: rows as above, slot j of the lanes kq = 0 =
-// sum of sub-block j of the scaled row / 64, the other lanes zero.
+// order in which the weight decoders emit the bytes of a dword.  Operand 8, GS == 32: rows as above, slot j of the lanes
+// kq = 0 = sum of sub-block j of the scaled row / 64, the other lanes zero.  GS == 16 (Q6_K, whose scales cover 16 values):
+// slot j of the lanes kq = 0 and slot j - 8 of the lanes kq = 1 = sum of the 16-value group j / 64, sixteen groups.
+template <int GS>
 __global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restrict__ x, _Float16 *__restrict__ ops, float *__restrict__ inv, int rows,
                                                            int k) {
     const int lane = threadIdx.x, b = lane >> 3, part = lane & 7;
@@ -63,12 +65,22 @@ __global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restric
     if (!have) scale = 0.f;
     uint8_t *base = reinterpret_cast<uint8_t *>(ops + ((size_t)g * ncol + c) * GR_OP_HALVES);
     const int kq = part >> 1, h = part & 1;  // the quad `part` of a sub-block: lane group and half of its eight slots
-    float sm = 0.f;
+    float sm = 0.f, sm2 = 0.f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
         const float a0 = v[t].x * scale, a1 = v[t].z * scale, a2 = v[t].y * scale, a3 = v[t].w * scale;
-        const float bs = group_sum<8>((a0 + a1) + (a2 + a3));  // sub-block t of row b: its eight quads sit in the eight lanes of b
-        sm = part == t ? bs : sm;
+        const float qs = (a0 + a1) + (a2 + a3);
+        if constexpr (GS == 32) {
+            const float bs = group_sum<8>(qs);  // sub-block t of row b: its eight quads sit in the eight lanes of b
+            sm = part == t ? bs : sm;
+        } else {
+            // the two 16-value groups 2 t and 2 t + 1 of the sub-block: quads 0..3 and 4..7; lane `part` keeps groups
+            // `part` and `part` + 8
+            const float lo = group_sum<8>(part < 4 ? qs : 0.f), hi = group_sum<8>(part < 4 ? 0.f : qs);
+            const float mine = (part & 1) ? hi : lo;
+            sm = (part >> 1) == t ? mine : sm;
+            sm2 = 4 + (part >> 1) == t ? mine : sm2;
+        }
         const h2raw h01 = __builtin_amdgcn_cvt_pkrtz(a0, a1), h23 = __builtin_amdgcn_cvt_pkrtz(a2, a3);
         const h2raw l01 = __builtin_amdgcn_cvt_pkrtz(a0 - (float)h01.x, a1 - (float)h01.y);
         const h2raw l23 = __builtin_amdgcn_cvt_pkrtz(a2 - (float)h23.x, a3 - (float)h23.y);
@@ -79,9 +91,15 @@ __global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restric
     sm *= 0.015625f;
     const _Float16 shi = (_Float16)sm, slo = (_Float16)(sm - (float)shi);
     _Float16 *sop = reinterpret_cast<_Float16 *>(base + 8 * 1024);
-    if (lane >= 16) *reinterpret_cast<u32x4 *>(base + 8 * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
+    if (lane >= (GS == 32 ? 16 : 32)) *reinterpret_cast<u32x4 *>(base + 8 * 1024 + lane * 16) = u32x4{0, 0, 0, 0};
     sop[(2 * b) * 8 + part] = shi;
     sop[(2 * b + 1) * 8 + part] = slo;
+    if constexpr (GS == 16) {
+        sm2 *= 0.015625f;
+        const _Float16 thi = (_Float16)sm2, tlo = (_Float16)(sm2 - (float)thi);
+        sop[(16 + 2 * b) * 8 + part] = thi;
+        sop[(16 + 2 * b + 1) * 8 + part] = tlo;
+    }
     if (part == 0) inv[((size_t)g * ncol + c) * 8 + b] = myinv;
 }
 
@@ -95,6 +113,8 @@ __device__ __forceinline__ f16x2 h2fma(uint32_t bits, f16x2 mul, f16x2 add) { re
 template <>
 struct RTile<F_Q4_K> {
     static constexpr int BYTES = 144;
+    static constexpr int NOPS = 8, SUMS = 32;  // weight operands per tile and column, values per block sum
+    __device__ static constexpr int aidx(int q) { return q; }  // the activation operand weight operand q meets
     struct Raw {
         u32x4 h;
         u32x2 q[4];
@@ -127,6 +147,8 @@ struct RTile<F_Q4_K> {
 template <>
 struct RTile<F_Q5_K> {
     static constexpr int BYTES = 176;
+    static constexpr int NOPS = 8, SUMS = 32;
+    __device__ static constexpr int aidx(int q) { return q; }
     struct Raw {
         u32x4 h;
         u32x2 qh;
@@ -164,15 +186,89 @@ struct RTile<F_Q5_K> {
     }
 };
 
+// Q6_K: 210 bytes = ql[128] (low nibbles), qh[64] (two high bits), 16 int8 scales of 16 values each, d.  Value 128 n + 32 ty
+// + l (n < 2, ty < 4, l < 32) is nibble ty / 2 of ql[64 n + 32 (ty & 1) + l] with bits 2 ty, 2 ty + 1 of qh[32 n + l] on top,
+// minus 32; its scale is number 8 n + 2 ty + l / 16.  The 32-value step s = 4 n + ty of the matrix core takes l = 8 kq .. + 7
+// from lane group kq - one scale per lane and step.  An int8 scale times a 6-bit quant (up to 8001) is not an FP16 integer,
+// but the quant is 16 a + b with sc * b <= 1905 and sc * 16 a a multiple of 16 below 6100: two exact operands per step,
+// both against the same activation operand; the -32 meets the sums of x per 16 values (operand 8 of
+// rows_prepare_kernel<16>) as 32 * sc, a multiple of 32 below 4100.
+template <>
+struct RTile<F_Q6_K> {
+    static constexpr int BYTES = 210;
+    static constexpr int NOPS = 16, SUMS = 16;
+    __device__ static constexpr int aidx(int q) { return q >> 1; }  // operands 2 s (low nibble part) and 2 s + 1 (high bits) of step s
+    struct Raw {
+        u32x2 ql[4];  // [2 n + (ty & 1)]: bytes 64 n + 32 (ty & 1) + 8 kq .. + 7
+        u32x2 qh[2];  // [n]: bytes 32 n + 8 kq .. + 7
+        u32x4 sc;
+        uint32_t d;
+    };
+    __device__ static __forceinline__ void load(Raw &r, const uint8_t *p, int kq) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r.ql[i] = ld64<2>(p + 32 * i + 8 * kq);
+#pragma unroll
+        for (int n = 0; n < 2; ++n) r.qh[n] = ld64<2>(p + 128 + 32 * n + 8 * kq);
+        r.sc = ld128<2>(p + 192);
+        r.d = ld16(p + 208);
+    }
+    __device__ static __forceinline__ void decode(const Raw &r, f16x8 (&B)[16], f16x8 &Bm, float &d, float &dmin) {
+        d = h2f(r.d);
+        dmin = d;  // the offset term is 32 * sc per group: y += d * (sum sc q x - 32 sum sc S)
+        // FP16 64 + b with b in bits 4..7 of a half-word, 16 + a with a in bits 6, 7 (1024 + b, as the 6-bit scales of Q4_K
+        // allow, would overflow: 1024 * 128)
+        const uint32_t mgb = 0x54005400u, mga = 0x4c004c00u;
+        const int kq = (int)(threadIdx.x >> 4) & 3;
+#pragma unroll
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int ty = 0; ty < 4; ++ty) {
+                // the scale of this lane's eight values of the step: number 8 n + 2 ty + kq / 2
+                const int is0 = 8 * n + 2 * ty;  // even (a constant, the loops being unrolled): is0 and is0 + 1 share a dword of the scales
+                const float scf = (float)(int)(int8_t)(r.sc[is0 >> 2] >> (8 * ((is0 & 3) + (kq >> 1))));
+                const f16x2 mb = splat2(scf), ab = splat2(-64.f * scf);           // (64 + b) sc - 64 sc
+                const f16x2 ma = splat2(16.f * scf), aa = splat2(-256.f * scf);   // (16 + a) 16 sc - 256 sc
+                const u32x2 lw = r.ql[2 * n + (ty & 1)], hw = r.qh[n];
+                f16x2 lo[4], hi[4];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const uint32_t w = t ? lw.y : lw.x, h = t ? hw.y : hw.x;
+                    // the nibble (low for ty < 2, high for the others) of bytes 0, 2 (1, 3) to bits 4..7 of the half-words
+                    const uint32_t w02 = ty < 2 ? w << 4 : w, w13 = ty < 2 ? w >> 4 : w >> 8;
+                    lo[2 * t] = h2fma((w02 & 0x00f000f0u) | mgb, mb, ab);
+                    lo[2 * t + 1] = h2fma((w13 & 0x00f000f0u) | mgb, mb, ab);
+                    // bits 2 ty, 2 ty + 1 of bytes 0, 2 (1, 3) to bits 6, 7 of the half-words
+                    const uint32_t h02 = 2 * ty <= 6 ? h << (6 - 2 * ty) : h, h13 = h >> (2 + 2 * ty);
+                    hi[2 * t] = h2fma((h02 & 0x00c000c0u) | mga, ma, aa);
+                    hi[2 * t + 1] = h2fma((h13 & 0x00c000c0u) | mga, ma, aa);
+                }
+                B[2 * (4 * n + ty)] = cat8(lo[0], lo[1], lo[2], lo[3]);
+                B[2 * (4 * n + ty) + 1] = cat8(hi[0], hi[1], hi[2], hi[3]);
+            }
+        // operand of the offsets: slot j of the lanes kq = 0 (1) = 32 * scale j (j + 8); the other lanes zero
+        const uint32_t s0 = kq == 0 ? r.sc.x : r.sc.z, s1 = kq == 0 ? r.sc.y : r.sc.w;
+        f16x2 m[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t sw = j < 2 ? s0 : s1;
+            const float e0 = (float)(int)(int8_t)(sw >> (16 * (j & 1))), e1 = (float)(int)(int8_t)(sw >> (16 * (j & 1) + 8));
+            m[j] = kq < 2 ? f16x2{(_Float16)(32.f * e0), (_Float16)(32.f * e1)} : f16x2{(_Float16)0.f, (_Float16)0.f};
+        }
+        Bm = cat8(m[0], m[1], m[2], m[3]);
+    }
+};
+
 // y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) for b < rows <= 8 * groups; k a multiple of 256, n >= 16.
-//   ops / inv: the output of rows_prepare_kernel for the same x.  grid: up to one workgroup per batch of GR_T tiles of 16
+//   ops / inv: the output of rows_prepare_kernel<RTile<FMT>::SUMS> for the same x.  grid: up to one workgroup per batch of T tiles of 16
 //   weight rows (the host caps it at one per compute unit); GR_THREADS threads; gemv_rows_lds_bytes() of dynamic LDS.
-template <int FMT>
+// T = 2 halves the activation-operand traffic per weight byte; T = 1 is for matrices with too few tiles to give every CU a
+// workgroup otherwise.
+template <int FMT, int T>
 __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ ops,
                                                                 const float *__restrict__ inv, const float *__restrict__ bias, float *__restrict__ y,
                                                                 int n, int k, int rows, int groups) {
     typedef RTile<FMT> R;
-    constexpr int T = GR_T;
+    constexpr int NOPS = R::NOPS;
     extern __shared__ __attribute__((aligned(16))) uint8_t gr_smem[];
     float2 *accl = reinterpret_cast<float2 *>(gr_smem);  // [tile t][group g][thread]
     const int tid = threadIdx.x, lane = tid & 63, nq = lane & 15, kq = lane >> 4;
@@ -201,7 +297,7 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
             for (int t = 0; t < T; ++t) R::load(raw[t], rp[t] + (size_t)c * R::BYTES, kq);
         }
         for (; c < ncol; c += GR_WAVES) {
-            f16x8 B[T][8], Bm[T];
+            f16x8 B[T][NOPS], Bm[T];
             float d[T], dmin64[T];
 #pragma unroll
             for (int t = 0; t < T; ++t) {
@@ -224,7 +320,7 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
                     if (!live[t]) continue;
                     f32x4 cs = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int s = 0; s < 8; ++s) cs = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[s], B[t][s], cs, 0, 0, 0);
+                    for (int s = 0; s < NOPS; ++s) cs = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[R::aidx(s)], B[t][s], cs, 0, 0, 0);
                     const f32x4 cm = mfma16(A[8], Bm[t]);
                     // operand rows 4 kq + i: activation rows 2 kq (hi, lo) and 2 kq + 1 (hi, lo) of the group
                     const float s0 = cs[0] + cs[1], s1 = cs[2] + cs[3], m0 = cm[0] + cm[1], m1 = cm[2] + cm[3];

@@ -4,32 +4,52 @@
 
 namespace jitnn {
 
-bool gemv_rows_supported(int fmt) { return fmt == F_Q4_K || fmt == F_Q5_K; }
+bool gemv_rows_supported(int fmt) { return fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K; }
 
 size_t gemv_rows_scratch_bytes(int rows, int k) {
     const int groups = (rows + 7) / 8;
     return gemv_rows_ops_bytes(groups, k) + gemv_rows_inv_bytes(groups, k);
 }
 
-KernelRef gemv_rows_kernel_ref(int fmt) {
+// Two tiles per wave where that still gives every CU a workgroup - or, for long rows (a wave then walks many columns) and
+// three groups of activation rows or more, every other CU: there the activation operands are what the launch waits for, and
+// two tiles share them (measured: Q6_K 4096 x 14336 at 40 rows 72.7 against 83.0 us; Q4_K 4096 x 4096 22.9 against 19.7, so
+// not for short rows) - else one.
+static int tiles_per_wave(int n, int k, int rows, unsigned max_blocks) {
+    const unsigned pairs = (unsigned)(((n + 15) / 16 + 1) / 2);
+    return pairs >= max_blocks || (rows > 16 && k >= 8192 && 2 * pairs >= max_blocks) ? 2 : 1;
+}
+
+KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blocks) {
+    const bool two = tiles_per_wave(n, k, rows, max_blocks) == 2;
+    const size_t lds = gemv_rows_lds_bytes(two ? 2 : 1);
     switch (fmt) {
-    case F_Q4_K: return {(const void *)gemv_rows_kernel<F_Q4_K>, gemv_rows_lds_bytes()};
-    case F_Q5_K: return {(const void *)gemv_rows_kernel<F_Q5_K>, gemv_rows_lds_bytes()};
+    case F_Q4_K: return {two ? (const void *)gemv_rows_kernel<F_Q4_K, 2> : (const void *)gemv_rows_kernel<F_Q4_K, 1>, lds};
+    case F_Q5_K: return {two ? (const void *)gemv_rows_kernel<F_Q5_K, 2> : (const void *)gemv_rows_kernel<F_Q5_K, 1>, lds};
+    case F_Q6_K: return {two ? (const void *)gemv_rows_kernel<F_Q6_K, 2> : (const void *)gemv_rows_kernel<F_Q6_K, 1>, lds};
     default: return {nullptr, 0};
     }
 }
 
-void gemv_rows_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const float *x, void *scratch, const float *bias, float *y, int n,
-                      int k, int rows) {
+template <int FMT>
+static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const float *x, void *scratch, const float *bias, float *y, int n, int k, int rows) {
+    typedef RTile<FMT> R;
     const int groups = (rows + 7) / 8, ncol = k / 256;
     _Float16 *ops = reinterpret_cast<_Float16 *>(scratch);
     float *inv = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
-    hipLaunchKernelGGL(rows_prepare_kernel, dim3(ncol, groups), dim3(64), 0, s, x, ops, inv, rows, k);
-    const int nbatch = ((n + 15) / 16 + GR_T - 1) / GR_T;
+    hipLaunchKernelGGL(rows_prepare_kernel<R::SUMS>, dim3(ncol, groups), dim3(64), 0, s, x, ops, inv, rows, k);
+    const int T = tiles_per_wave(n, k, rows, max_blocks), nbatch = ((n + 15) / 16 + T - 1) / T;
     const unsigned blocks = (unsigned)nbatch < max_blocks ? (unsigned)nbatch : max_blocks;
+    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(2), s, W, ops, inv, bias, y, n, k, rows, groups);
+    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(1), s, W, ops, inv, bias, y, n, k, rows, groups);
+}
+
+void gemv_rows_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const float *x, void *scratch, const float *bias, float *y, int n,
+                      int k, int rows) {
     switch (fmt) {
-    case F_Q4_K: hipLaunchKernelGGL(gemv_rows_kernel<F_Q4_K>, dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(), s, W, ops, inv, bias, y, n, k, rows, groups); break;
-    case F_Q5_K: hipLaunchKernelGGL(gemv_rows_kernel<F_Q5_K>, dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(), s, W, ops, inv, bias, y, n, k, rows, groups); break;
+    case F_Q4_K: launch<F_Q4_K>(max_blocks, s, W, x, scratch, bias, y, n, k, rows); break;
+    case F_Q5_K: launch<F_Q5_K>(max_blocks, s, W, x, scratch, bias, y, n, k, rows); break;
+    case F_Q6_K: launch<F_Q6_K>(max_blocks, s, W, x, scratch, bias, y, n, k, rows); break;
     default: break;
     }
 }

@@ -976,7 +976,7 @@ int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const fl
     if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s, src);
     // several rows, rows of whole 256-value columns: every row meets the weights in one pass over them (gemv_rows.h)
     if (g.rows_kernel_min > 0 && rows >= g.rows_kernel_min && rows <= 64 && gemv_rows_supported(w->fmt) && w->k % 256 == 0 && w->n >= 16 && !g.force_lds) {
-        const KernelRef kr = gemv_rows_kernel_ref(w->fmt);
+        const KernelRef kr = gemv_rows_kernel_ref(w->fmt, w->n, w->k, rows, (unsigned)g.cus);
         if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
         void *scratch = nullptr;
         if (int rc = workspace(gemv_rows_scratch_bytes(rows, w->k), s, &scratch, src)) return rc;

@@ -57,7 +57,7 @@ void gemv_mfma_launch(int fmt, unsigned blocks, hipStream_t s, const uint8_t *W,
 // ---- gemv_rows.hip: rows_prepare_kernel + gemv_rows_kernel<fmt>: 2..64 rows in one pass over the weights
 bool gemv_rows_supported(int fmt);
 size_t gemv_rows_scratch_bytes(int rows, int k);   // operands + scales of `rows` activation rows of k values
-KernelRef gemv_rows_kernel_ref(int fmt);
+KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blocks);  // the variant gemv_rows_launch picks for this shape
 void gemv_rows_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const float *x, void *scratch, const float *bias, float *y, int n,
                       int k, int rows);
 

@@ -202,6 +202,34 @@ def test_small_k_32_blocks_and_many_rows(jn, fmt):
         assert norm_err(y, ref) <= bar(rows), (fmt, rows, norm_err(y, ref))
 
 
+@pytest.mark.parametrize("fmt", ["Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("n,k", [(16, 256), (100, 2048), (1000, 4096 + 256), (259, 14336)])
+def test_one_pass_rows_kernel(jn, fmt, n, k):
+    """9..64 rows of the K-quants take one pass over the weights (block scales folded into FP16 weight operands, the
+    activations split hi + lo): whole and ragged tiles of 16 weight rows, one to many 256-value columns, every number of
+    groups of eight rows, bias, and activation rows of very different magnitudes - bar 1e-4 of the largest output per
+    row."""
+    from oracle import oracle
+    rng = np.random.default_rng(n + k + GGML_ID[fmt])
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    for rows in (9, 16, 24, 33, 40, 57, 64):
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        x[1] *= np.float32(1e6)
+        x[2] *= np.float32(1e-6)
+        x[3] = 0
+        x[4, rng.integers(0, k, size=max(1, k // 256))] *= np.float32(1e4)
+        x[rows - 1] *= np.float32(1e-30)
+        b = bias if rows % 2 == 0 else None
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, b, n, k).astype(np.float64)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(b) if b is not None else None).numpy()
+        for r in range(rows):
+            scale = max(float(np.abs(ref[r]).max()), 1e-37)
+            assert float(np.abs(y[r].astype(np.float64) - ref[r]).max()) / scale <= GEMV_BAR, (fmt, n, k, rows, r)
+        assert not y[3].any() if b is None else np.array_equal(y[3], bias)
+
+
 @pytest.mark.parametrize("fmt", ["Q4_0", "Q4_1", "Q8_0"])
 @pytest.mark.parametrize("k", [96, 160])
 def test_odd_block_counts_at_every_batch_size(jn, fmt, k):
