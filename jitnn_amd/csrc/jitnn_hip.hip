@@ -84,6 +84,7 @@ struct State {
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
     bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
     bool prefill_group = true;   // JITNN_HIP_PREFILL_GROUP=0: every weight of a group of linears in a launch of its own
+    bool rows_kernel_min_set = false;  // JITNN_HIP_ROWS_MIN was given: no per-shape exceptions
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
@@ -825,7 +826,10 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_ROWS_MIN")) g.rows_kernel_min = atoi(e);
+    if (const char *e = getenv("JITNN_HIP_ROWS_MIN")) {
+        g.rows_kernel_min = atoi(e);
+        g.rows_kernel_min_set = true;
+    }
     if (const char *e = getenv("JITNN_HIP_PREFILL_GROUP")) g.prefill_group = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_MFMA")) g.prefill_attn_mfma = atoi(e) != 0;
@@ -975,7 +979,10 @@ int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const fl
     count_op(many ? ST_MFMA : ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n) + (bias_dev ? 4ll * w->n : 0));
     if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s, src);
     // several rows, rows of whole 256-value columns: every row meets the weights in one pass over them (gemv_rows.h)
-    if (g.rows_kernel_min > 0 && rows >= g.rows_kernel_min && rows <= 64 && gemv_rows_supported(w->fmt) && w->k % 256 == 0 && w->n >= 16 && !g.force_lds) {
+    // (from 9 rows; Q6_K rows of 8192 values and more - the ffn_down of a Q4_K_M layer - from 3: 35.6 against 41.5-44.6 us for
+    // 4096 x 14336, where the kernels for up to 8 rows pay their activation set-up per 4096-value slice)
+    const int rows_min = g.rows_kernel_min_set || !(w->fmt == F_Q6_K && w->k >= 8192) ? g.rows_kernel_min : 3;
+    if (g.rows_kernel_min > 0 && rows >= rows_min && rows <= 64 && gemv_rows_supported(w->fmt) && w->k % 256 == 0 && w->n >= 16 && !g.force_lds) {
         const KernelRef kr = gemv_rows_kernel_ref(w->fmt, w->n, w->k, rows, (unsigned)g.cus);
         if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
         void *scratch = nullptr;
