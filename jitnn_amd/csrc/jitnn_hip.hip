@@ -979,9 +979,10 @@ int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const fl
     count_op(many ? ST_MFMA : ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n) + (bias_dev ? 4ll * w->n : 0));
     if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s, src);
     // several rows, rows of whole 256-value columns: every row meets the weights in one pass over them (gemv_rows.h)
-    // (from 9 rows; Q6_K rows of 8192 values and more - the ffn_down of a Q4_K_M layer - from 3: 35.6 against 41.5-44.6 us for
-    // 4096 x 14336, where the kernels for up to 8 rows pay their activation set-up per 4096-value slice)
-    const int rows_min = g.rows_kernel_min_set || !(w->fmt == F_Q6_K && w->k >= 8192) ? g.rows_kernel_min : 3;
+    // (from 9 rows; rows of 12288 values and more - the ffn_down of an 8B layer, 4096 x 14336 - from 3: Q6_K 35.6 against
+    // 41.5-44.6 us, Q4_K 24.5 against 26.6-27.6, where the kernels for up to 8 rows pay their activation set-up per
+    // 4096-value slice; at 8192 values they are still ahead, 15.0 against 16.9)
+    const int rows_min = g.rows_kernel_min_set || w->k < 12288 ? g.rows_kernel_min : 3;
     if (g.rows_kernel_min > 0 && rows >= rows_min && rows <= 64 && gemv_rows_supported(w->fmt) && w->k % 256 == 0 && w->n >= 16 && !g.force_lds) {
         const KernelRef kr = gemv_rows_kernel_ref(w->fmt, w->n, w->k, rows, (unsigned)g.cus);
         if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
