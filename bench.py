@@ -381,6 +381,27 @@ def bench_decode(torch, lib, steps, warmup):
                               "last_logits_vs_512_decode_steps_norm_err": err, "logits_finite": bool(torch.isfinite(pl).all().item())}
     except Exception as e:  # report, never hide
         out["prefill_512_error"] = f"{type(e).__name__}: {e}"
+    # a short prompt: 40 tokens stay in the GEMV range (FP32-grade accuracy), every K-quant weight in one pass over its bytes
+    try:
+        xs = torch.randn(40, 4096, device="cuda", generator=torch.Generator(device="cuda").manual_seed(13))
+        pl = torch.empty(cfg["vocab"], device="cuda")
+        for _ in range(2):
+            dec.prefill_dev(xs.data_ptr(), 0, 40, pl.data_ptr(), st)
+        torch.cuda.synchronize()
+        reps = 10
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            dec.prefill_dev(xs.data_ptr(), 0, 40, pl.data_ptr(), st)
+        torch.cuda.synchronize()
+        pw = (time.perf_counter() - t0) / reps
+        for t in range(40):
+            dec.decode_dev(xs[t].data_ptr(), t, logits.data_ptr(), st)
+        torch.cuda.synchronize()
+        err = float((pl - logits).abs().max() / logits.abs().max())
+        out["prefill_40"] = {"workload": "the same model on a 40-token prompt from an empty cache, one call (GEMV range)", "ms": pw * 1e3,
+                             "tokens_per_s": 40 / pw, "last_logits_vs_40_decode_steps_norm_err": err}
+    except Exception as e:  # report, never hide
+        out["prefill_40_error"] = f"{type(e).__name__}: {e}"
     for h in handles + [hh]:
         lib.lib.jitnn_hip_weight_free(h)
     dec.close()
