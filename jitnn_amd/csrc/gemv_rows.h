@@ -258,15 +258,16 @@ struct RTile<F_Q6_K> {
     }
 };
 
-// y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) for b < rows <= 8 * groups; k a multiple of 256, n >= 16.
+// y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) (+ res[b, row]) for b < rows <= 8 * groups; k a multiple of 256, n >= 16.
 //   ops / inv: the output of rows_prepare_kernel<RTile<FMT>::SUMS> for the same x.  grid: up to one workgroup per batch of T tiles of 16
 //   weight rows (the host caps it at one per compute unit); GR_THREADS threads; gemv_rows_lds_bytes() of dynamic LDS.
 // T = 2 halves the activation-operand traffic per weight byte; T = 1 is for matrices with too few tiles to give every CU a
 // workgroup otherwise.
 template <int FMT, int T>
 __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ ops,
-                                                                const float *__restrict__ inv, const float *__restrict__ bias, float *__restrict__ y,
-                                                                int n, int k, int rows, int groups) {
+                                                                const float *__restrict__ inv, const float *__restrict__ bias,
+                                                                const float *res, float *y, int n, int k, int rows,  // (res may be y)
+                                                                int groups) {
     typedef RTile<FMT> R;
     constexpr int NOPS = R::NOPS;
     extern __shared__ __attribute__((aligned(16))) uint8_t gr_smem[];
@@ -347,8 +348,9 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
                 const int r = l & 15, row = min(tile * 16, n - 16) + r, b0 = g * 8 + 2 * (l >> 4);
                 if (row >= tile * 16) {  // rows of a ragged last tile that an earlier tile already wrote are skipped
                     const float bv = bias ? bias[row] : 0.f;
-                    if (b0 < rows) y[(size_t)b0 * n + row] = sum.x + bv;
-                    if (b0 + 1 < rows) y[(size_t)(b0 + 1) * n + row] = sum.y + bv;
+                    // (res [rows, n]: a residual that rides along, y = res + x W^T - the layers of a model)
+                    if (b0 < rows) y[(size_t)b0 * n + row] = sum.x + bv + (res ? res[(size_t)b0 * n + row] : 0.f);
+                    if (b0 + 1 < rows) y[(size_t)(b0 + 1) * n + row] = sum.y + bv + (res ? res[(size_t)(b0 + 1) * n + row] : 0.f);
                 }
             }
         }

@@ -31,25 +31,41 @@ KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blo
     }
 }
 
-template <int FMT>
-static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const float *x, void *scratch, const float *bias, float *y, int n, int k, int rows) {
-    typedef RTile<FMT> R;
+int gemv_rows_sums(int fmt) {
+    switch (fmt) {
+    case F_Q4_K: return RTile<F_Q4_K>::SUMS;
+    case F_Q5_K: return RTile<F_Q5_K>::SUMS;
+    case F_Q6_K: return RTile<F_Q6_K>::SUMS;
+    default: return 0;
+    }
+}
+
+void gemv_rows_prepare_launch(int sums, hipStream_t s, const float *x, void *scratch, int k, int rows) {
     const int groups = (rows + 7) / 8, ncol = k / 256;
     _Float16 *ops = reinterpret_cast<_Float16 *>(scratch);
     float *inv = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
-    hipLaunchKernelGGL(rows_prepare_kernel<R::SUMS>, dim3(ncol, groups), dim3(64), 0, s, x, ops, inv, rows, k);
-    const int T = tiles_per_wave(n, k, rows, max_blocks), nbatch = ((n + 15) / 16 + T - 1) / T;
-    const unsigned blocks = (unsigned)nbatch < max_blocks ? (unsigned)nbatch : max_blocks;
-    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(2), s, W, ops, inv, bias, y, n, k, rows, groups);
-    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(1), s, W, ops, inv, bias, y, n, k, rows, groups);
+    if (sums == 16) hipLaunchKernelGGL(rows_prepare_kernel<16>, dim3(ncol, groups), dim3(64), 0, s, x, ops, inv, rows, k);
+    else hipLaunchKernelGGL(rows_prepare_kernel<32>, dim3(ncol, groups), dim3(64), 0, s, x, ops, inv, rows, k);
 }
 
-void gemv_rows_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const float *x, void *scratch, const float *bias, float *y, int n,
-                      int k, int rows) {
+template <int FMT>
+static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y, int n, int k,
+                   int rows) {
+    const int groups = (rows + 7) / 8;
+    const _Float16 *ops = reinterpret_cast<const _Float16 *>(scratch);
+    const float *inv = reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
+    const int T = tiles_per_wave(n, k, rows, max_blocks), nbatch = ((n + 15) / 16 + T - 1) / T;
+    const unsigned blocks = (unsigned)nbatch < max_blocks ? (unsigned)nbatch : max_blocks;
+    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(2), s, W, ops, inv, bias, res, y, n, k, rows, groups);
+    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(1), s, W, ops, inv, bias, res, y, n, k, rows, groups);
+}
+
+void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,
+                           int n, int k, int rows) {
     switch (fmt) {
-    case F_Q4_K: launch<F_Q4_K>(max_blocks, s, W, x, scratch, bias, y, n, k, rows); break;
-    case F_Q5_K: launch<F_Q5_K>(max_blocks, s, W, x, scratch, bias, y, n, k, rows); break;
-    case F_Q6_K: launch<F_Q6_K>(max_blocks, s, W, x, scratch, bias, y, n, k, rows); break;
+    case F_Q4_K: launch<F_Q4_K>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
+    case F_Q5_K: launch<F_Q5_K>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
+    case F_Q6_K: launch<F_Q6_K>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
     default: break;
     }
 }

@@ -971,6 +971,41 @@ int jitnn_hip_dequantize(const jitnn_hip_weight *w, float *y_host) {
 
 namespace {
 
+// Does a linear of `rows` rows on this weight take the one-pass kernel of gemv_rows.h?  From 9 rows; rows of 12288 values and
+// more - the ffn_down of an 8B layer, 4096 x 14336 - from 3: Q6_K 35.6 against 41.5-44.6 us, Q4_K 24.5 against 26.6-27.6,
+// where the kernels for up to 8 rows pay their activation set-up per 4096-value slice (at 8192 values they are still
+// ahead, 15.0 against 16.9).
+bool rows_path(const jitnn_hip_weight *w, int rows) {
+    const int rows_min = g.rows_kernel_min_set || w->k < 12288 ? g.rows_kernel_min : 3;
+    return g.rows_kernel_min > 0 && rows >= rows_min && rows <= 64 && rows <= g.gemv_max_rows && gemv_rows_supported(w->fmt) && w->k % 256 == 0 &&
+           w->n >= 16 && !g.force_lds;
+}
+
+// ys[i] = x ws[i]^T (+ bias) (+ residual [rows, n]; bias and residual with one weight only) for weights that all pass
+// rows_path: the activation operands are prepared once per granularity of block sums and shared by the weights.
+int launch_rows_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias, const float *residual,
+                      hipStream_t s, ScratchSource src) {
+    const int k = ws[0]->k;
+    bool need[2] = {false, false};  // block sums per 32 values, per 16 values
+    for (int i = 0; i < count; ++i) {
+        if (ws[i]->k != k) return fail(JITNN_HIP_EINVAL, "weights of %d and %d values per row on one activation", k, ws[i]->k);
+        const KernelRef kr = gemv_rows_kernel_ref(ws[i]->fmt, ws[i]->n, k, rows, (unsigned)g.cus);
+        if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
+        need[gemv_rows_sums(ws[i]->fmt) == 16] = true;
+    }
+    const size_t one = (gemv_rows_scratch_bytes(rows, k) + 255) & ~(size_t)255;
+    void *scratch = nullptr;
+    if (int rc = workspace(one * ((int)need[0] + (int)need[1]), s, &scratch, src)) return rc;
+    uint8_t *sc32 = (uint8_t *)scratch, *sc16 = sc32 + (need[0] ? one : 0);
+    if (need[0]) gemv_rows_prepare_launch(32, s, x, sc32, k, rows);
+    if (need[1]) gemv_rows_prepare_launch(16, s, x, sc16, k, rows);
+    for (int i = 0; i < count; ++i)
+        gemv_rows_main_launch(ws[i]->fmt, (unsigned)g.cus, s, ws[i]->dev, gemv_rows_sums(ws[i]->fmt) == 16 ? sc16 : sc32, bias, residual, ys[i], ws[i]->n,
+                              k, rows);
+    HIP_TRY(hipGetLastError());
+    return workspace_done(s, src);
+}
+
 int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const float *bias_dev, float *y_dev, hipStream_t s, ScratchSource src) {
     if (!w || !x_dev || !y_dev) return fail(JITNN_HIP_EINVAL, "weight, input or output is NULL");
     if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
@@ -979,19 +1014,7 @@ int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const fl
     count_op(many ? ST_MFMA : ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n) + (bias_dev ? 4ll * w->n : 0));
     if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s, src);
     // several rows, rows of whole 256-value columns: every row meets the weights in one pass over them (gemv_rows.h)
-    // (from 9 rows; rows of 12288 values and more - the ffn_down of an 8B layer, 4096 x 14336 - from 3: Q6_K 35.6 against
-    // 41.5-44.6 us, Q4_K 24.5 against 26.6-27.6, where the kernels for up to 8 rows pay their activation set-up per
-    // 4096-value slice; at 8192 values they are still ahead, 15.0 against 16.9)
-    const int rows_min = g.rows_kernel_min_set || w->k < 12288 ? g.rows_kernel_min : 3;
-    if (g.rows_kernel_min > 0 && rows >= rows_min && rows <= 64 && gemv_rows_supported(w->fmt) && w->k % 256 == 0 && w->n >= 16 && !g.force_lds) {
-        const KernelRef kr = gemv_rows_kernel_ref(w->fmt, w->n, w->k, rows, (unsigned)g.cus);
-        if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
-        void *scratch = nullptr;
-        if (int rc = workspace(gemv_rows_scratch_bytes(rows, w->k), s, &scratch, src)) return rc;
-        gemv_rows_launch(w->fmt, (unsigned)g.cus, s, w->dev, x_dev, scratch, bias_dev, y_dev, w->n, w->k, rows);
-        HIP_TRY(hipGetLastError());
-        return workspace_done(s, src);
-    }
+    if (rows_path(w, rows)) return launch_rows_group(&w, &y_dev, 1, x_dev, rows, bias_dev, nullptr, s, src);
     for (int r0 = 0; r0 < rows; r0 += 8) {
         const int nb = rows - r0 < 8 ? rows - r0 : 8;
         if (int rc = launch_gemv(w, x_dev + (size_t)r0 * w->k, nb, bias_dev, y_dev + (size_t)r0 * w->n, s)) return rc;
@@ -1347,6 +1370,13 @@ int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const 
     for (int i = 0; i < count; ++i) group = group && !is_extra_format(ws[i]->fmt);
     if (group) return launch_prefill_group(ws, ys, count, x, rows, nullptr, nw, m->eps, st);
     hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(256), 0, st, x, nw, xn, m->d, m->eps);
+    // the one-pass kernel for several rows prepares its activation operands once for all the weights that take it
+    bool shared = count > 1;
+    for (int i = 0; i < count; ++i) shared = shared && rows_path(ws[i], rows);
+    if (shared) {
+        for (int i = 0; i < count; ++i) count_op(ST_GEMV, (long long)ws[i]->nbytes + 4ll * rows * ((long long)ws[i]->k + ws[i]->n));
+        return launch_rows_group(ws, ys, count, xn, rows, nullptr, nullptr, st, SCRATCH_THREAD);
+    }
     for (int i = 0; i < count; ++i)
         if (int rc = jitnn_hip_linear_dev(ws[i], xn, rows, nullptr, ys[i], (void *)st)) return rc;
     return JITNN_HIP_OK;
@@ -1367,6 +1397,10 @@ int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, co
         hipLaunchKernelGGL(swiglu_kernel, dim3(blocks), dim3(256), 0, st, x, up, h, (int)count);
         x = h;
         if (many) return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp);
+    }
+    if (rows_path(w, rows)) {  // the one-pass kernel adds the residual as it stores
+        count_op(ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n));
+        return launch_rows_group(&w, &y, 1, x, rows, nullptr, res, st, SCRATCH_THREAD);
     }
     if (int rc = jitnn_hip_linear_dev(w, x, rows, nullptr, tmp, (void *)st)) return rc;
     const size_t count4 = (size_t)rows * w->n / 4;
