@@ -6,13 +6,15 @@
 //   * rows_prepare_kernel builds the activation operands once per call: per group of eight rows and 256-value column of
 //     K, the rows scaled by a power of two (from the column's largest magnitude per row) and split into two FP16 parts,
 //     x 2^e = hi + lo, written in matrix-core operand order (hi and lo of a row in neighbouring operand rows, so that
-//     their block sums meet in one lane) together with the column's eight block sums of x and the inverse scales.  The
-//     main kernel streams them from L2: one 16-byte load per lane and operand.
+//     their block sums meet in one lane) together with the column's block sums of x (per 32 values, or per 16 for Q6_K)
+//     and the inverse scales - once per activation, for every weight that meets it.  The main kernel streams them from
+//     L2: one 16-byte load per lane and operand.
 //   * the block scales are folded into the weight operand where that is exact: a Q4_K / Q5_K quant times its 6-bit
 //     scale is an integer below 2048, so sc * q is an FP16 value without rounding, and the matrix core accumulates the
 //     eight sub-blocks of a super-block in one FP32 chain; only the super-block's d and dmin (and the activation scale)
 //     meet the sums in FP32, once per 16 x 256 tile instead of once per block.  The conversion costs what the plain one
-//     did: (1024 + q) * sc - 1024 * sc is one packed FMA on the pattern 0x6400 | q.
+//     did: (1024 + q) * sc - 1024 * sc is one packed FMA on the pattern 0x6400 | q.  Q6_K's int8 scale times 6-bit quant
+//     is not an FP16 integer, but its two parts are (RTile<F_Q6_K>): two operands per 32-value step.
 // A workgroup of eight waves owns tiles of 16 weight rows; wave w walks the 256-value columns w, w + 8, ... of K for the
 // workgroup's tiles, T tiles at a time: every lane fetches the bytes of its own weight row straight from global memory
 // (the four 8-byte pieces of a row's 128 quant bytes share a cache line, so the line is used whole), turns them into
