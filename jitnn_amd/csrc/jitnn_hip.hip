@@ -83,6 +83,7 @@ struct State {
     bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
     bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
     bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
+    bool prefill_defer_join = true;  // JITNN_HIP_PREFILL_DEFER_JOIN=0: every split-K linear of the prefill step is joined by a kernel of its own
     bool prefill_group = true;   // JITNN_HIP_PREFILL_GROUP=0: every weight of a group of linears in a launch of its own
     bool rows_kernel_min_set = false;  // JITNN_HIP_ROWS_MIN was given: no per-shape exceptions
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
@@ -589,9 +590,13 @@ int stage_reserve(size_t pinned_bytes, size_t dev_bytes) {
 // XP_MAXK values; the caller checks with prefill_prepare_fuses_norm).
 // residual != nullptr (one weight only): y = residual + x w^T, added by the join of the K slices, or, for a launch that
 // does not split K, by a pass of its own over the product left in `tmp` [rows, n].
+// part_ext / defer (one weight with a residual): the K slices go to part_ext ([8][rows, n] floats, the caller's) and, when the
+// launch does split K, their join is left to the caller - *defer describes it, and the activation preparation of the next
+// linears can do it on the way (pend: this call's activations are that pending row, not x).
 int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias,
                          const float *norm_w, float eps, hipStream_t stream, const float *residual = nullptr, float *tmp = nullptr,
-                         const float *swiglu_up = nullptr, ScratchSource src = SCRATCH_THREAD) {
+                         const float *swiglu_up = nullptr, ScratchSource src = SCRATCH_THREAD, float *part_ext = nullptr, PfPending *defer = nullptr,
+                         const PfPending *pend = nullptr) {
     // (the kernels live in prefill_k.hip, prefill_q32.hip and prefill_mixed.hip)
     // Weights of one format - and a run of one K-quant format followed by a run of another for which a two-format kernel
     // exists - share a launch: their row tiles are numbered one after the other, so that the 1024-row k and v projections
@@ -670,8 +675,8 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     if (int rc = workspace(xo_bytes + scale_bytes + part_max, stream, &wsp, src)) return rc;
     _Float16 *xo = (_Float16 *)wsp;
     float *scale = (float *)((uint8_t *)wsp + xo_bytes), *inv = scale + rows;
-    float *part = (float *)((uint8_t *)wsp + xo_bytes + scale_bytes);
-    prefill_prepare_launch(x, scale, inv, xo, rows, k, mblocks, norm_w, eps, swiglu_up, stream);
+    float *part = part_ext && count == 1 && residual ? part_ext : (float *)((uint8_t *)wsp + xo_bytes + scale_bytes);
+    prefill_prepare_launch(x, scale, inv, xo, rows, k, mblocks, norm_w, eps, swiglu_up, stream, pend);
     for (int li = 0; li < nlaunch; ++li) {
         const Launch &l = launch[li];
         const jitnn_hip_weight *w = ws[l.first];
@@ -704,6 +709,12 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
             for (int q = 0; q < l.count; ++q) count4 += (size_t)rows * sg.n[q] / 4;
             const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
             prefill_join_group_launch(part, out, rows, blocks, stream);
+        } else if (split && defer && part == part_ext && !bias) {  // the join rides with the next activation preparation
+            defer->part = part;
+            defer->res = residual;
+            defer->out = ys[l.first];
+            defer->splits = l.splits[0];
+            defer->n = w->n;
         } else if (split) {
             const size_t count4 = (size_t)rows * w->n / 4;
             const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
@@ -831,6 +842,7 @@ int jitnn_hip_init(int device_ordinal) {
         g.rows_kernel_min_set = true;
     }
     if (const char *e = getenv("JITNN_HIP_PREFILL_GROUP")) g.prefill_group = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_PREFILL_DEFER_JOIN")) g.prefill_defer_join = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_MFMA")) g.prefill_attn_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
@@ -1284,7 +1296,7 @@ struct jitnn_hip_llama {
     int chunks_max;
     // many-token (prefill) buffers, [pf_cap, ...] each, allocated by the first prefill call and grown when a longer one comes
     int pf_cap;
-    float *pf[10];  // xn, q, k, v, att, xa, xb, gate, up, h
+    float *pf[11];  // xn, q, k, v, att, xa, xb, gate, up, h, the K slices of a linear whose join is deferred (8 x d per token)
     int rope_interleaved;  // 0: rotate-half pairs (i, i + D/2); 1: pairs (2i, 2i + 1)
     // token embedding table [vocab, d] in ggml type embd_fmt (F32 = 0, F16 = 1 or a block format), owned
     uint8_t *embd;
@@ -1364,11 +1376,29 @@ long long model_weight_bytes(const jitnn_hip_llama *m) {
 // ys[i] = RMSNorm(x) ws[i]^T for `rows` rows.  With more rows than the GEMV kernels take (and formats the many-row
 // kernels know) the norm is part of the one activation preparation the weights share; otherwise it is a kernel of its
 // own into `xn` [rows, d] and the linears take their usual route.
+// The join of a linear's K slices that a caller deferred and nobody could fuse: prefill_join_kernel after all.
+void flush_pending(PfPending &p, int rows, hipStream_t st) {
+    if (!p.part) return;
+    const size_t count4 = (size_t)rows * p.n / 4;
+    const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
+    prefill_join_launch(p.part, nullptr, p.res, p.out, count4, p.n, p.splits, blocks, st);
+    p = PfPending{};
+}
+
+// (pend: x - the output of the linear before - may still be in K slices; the shared preparation then adds them up)
 int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows,
-                        const float *nw, float *xn, hipStream_t st) {
+                        const float *nw, float *xn, hipStream_t st, PfPending *pend = nullptr) {
     bool group = rows > g.gemv_max_rows && prefill_prepare_fuses_norm(m->d);
     for (int i = 0; i < count; ++i) group = group && !is_extra_format(ws[i]->fmt);
-    if (group) return launch_prefill_group(ws, ys, count, x, rows, nullptr, nw, m->eps, st);
+    if (group) {
+        const bool fused = pend && pend->part && pend->out == x && pend->n == m->d;
+        const int rc = launch_prefill_group(ws, ys, count, x, rows, nullptr, nw, m->eps, st, nullptr, nullptr, nullptr, SCRATCH_THREAD, nullptr, nullptr,
+                                            fused ? pend : nullptr);
+        if (fused) *pend = PfPending{};
+        else if (pend) flush_pending(*pend, rows, st);  // (never both: a pending join is flushed before anybody reads its row)
+        return rc;
+    }
+    if (pend) flush_pending(*pend, rows, st);
     hipLaunchKernelGGL(rms_norm_rows_kernel, dim3(rows), dim3(256), 0, st, x, nw, xn, m->d, m->eps);
     // the one-pass kernel for several rows prepares its activation operands once for all the weights that take it
     bool shared = count > 1;
@@ -1385,11 +1415,13 @@ int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const 
 // y = res + x w^T for `rows` rows (tmp [rows, n] is scratch).  up != nullptr: the activations are silu(x) * up (the FFN's
 // gate and up projections); on the many-row path they are formed inside the activation preparation, otherwise by
 // swiglu_kernel into `h` [rows, k].
+// part / defer: see launch_prefill_group - the join of the K slices may be left to the caller.
 int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, const float *res, float *tmp, float *y, hipStream_t st,
-                         const float *up = nullptr, float *h = nullptr) {
+                         const float *up = nullptr, float *h = nullptr, float *part = nullptr, PfPending *defer = nullptr) {
     const bool many = rows > g.gemv_max_rows && !is_extra_format(w->fmt) && w->n % 4 == 0;
     if (many && (!up || (g.prefill_fuse_swiglu && prefill_prepare_fuses_norm(w->k)))) {
-        return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp, up);
+        return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp, up, SCRATCH_THREAD, g.prefill_defer_join ? part : nullptr,
+                                    g.prefill_defer_join ? defer : nullptr);
     }
     if (up) {
         const long long count = (long long)rows * w->k;
@@ -1420,8 +1452,8 @@ int ensure_prefill(jitnn_hip_llama *m, int tokens) {
     }
     m->pf_cap = 0;
     const size_t qd = (size_t)m->heads * m->hd, kd = (size_t)m->kv * m->hd;
-    const size_t per[10] = {(size_t)m->d, qd, kd, kd, qd, (size_t)m->d, (size_t)m->d, (size_t)m->ffn, (size_t)m->ffn, (size_t)m->ffn};
-    for (int i = 0; i < 10; ++i) {
+    const size_t per[11] = {(size_t)m->d, qd, kd, kd, qd, (size_t)m->d, (size_t)m->d, (size_t)m->ffn, (size_t)m->ffn, (size_t)m->ffn, (size_t)8 * m->d};
+    for (int i = 0; i < 11; ++i) {
         if (hipMalloc(&m->pf[i], per[i] * tokens * sizeof(float)) != hipSuccess) {
             (void)hipGetLastError();
             for (float *&b : m->pf) {
@@ -1665,6 +1697,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
     float *xn = m->pf[0], *q = m->pf[1], *k = m->pf[2], *v = m->pf[3], *att = m->pf[4], *xa = m->pf[5], *xb = m->pf[6], *gate = m->pf[7],
           *up = m->pf[8], *h = m->pf[9];
     const float *x = x_dev;
+    PfPending pend;  // the K slices of the linear that wrote x, when their join is still to come
     for (int l = 0; l < m->layers; ++l) {
         const jitnn_hip_weight *const *w = m->w + (size_t)l * 7;
         const float *nw = m->norms + (size_t)l * 2 * d;
@@ -1672,7 +1705,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         {
             const jitnn_hip_weight *ws[3] = {w[JITNN_HIP_W_ATTN_Q], w[JITNN_HIP_W_ATTN_K], w[JITNN_HIP_W_ATTN_V]};
             float *ys[3] = {q, k, v};
-            if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st)) return rc;
+            if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st, &pend)) return rc;
         }
         hipLaunchKernelGGL(rope_append_rows_kernel, dim3(T), dim3(256), 0, st, q, k, v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads, m->kv, m->hd,
                            pos0, m->rope_interleaved);
@@ -1685,16 +1718,17 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         }
         if (arc) return arc;
         // xa = x + Wo att, xb = xa + W2 (silu(W1 n) * (W3 n)), n = RMSNorm(xa)
-        if (int rc = residual_linear_rows(w[JITNN_HIP_W_ATTN_O], att, T, x, xn, xa, st)) return rc;
+        if (int rc = residual_linear_rows(w[JITNN_HIP_W_ATTN_O], att, T, x, xn, xa, st, nullptr, nullptr, m->pf[10], &pend)) return rc;
         {
             const jitnn_hip_weight *ws[2] = {w[JITNN_HIP_W_FFN_GATE], w[JITNN_HIP_W_FFN_UP]};
             float *ys[2] = {gate, up};
-            if (int rc = normed_linears_rows(m, ws, ys, 2, xa, T, nw + d, xn, st)) return rc;
+            if (int rc = normed_linears_rows(m, ws, ys, 2, xa, T, nw + d, xn, st, &pend)) return rc;
         }
-        if (int rc = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], gate, T, xa, xn, xb, st, up, h)) return rc;
+        if (int rc = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], gate, T, xa, xn, xb, st, up, h, m->pf[10], &pend)) return rc;
         x = xb;
     }
     (void)qd;
+    flush_pending(pend, T, st);  // the last layer's output exists whole
     if (logits_dev) {  // the last token's logits
         const jitnn_hip_weight *ws[1] = {m->w_out};
         float *ys[1] = {logits_dev};

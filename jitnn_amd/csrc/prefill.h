@@ -96,11 +96,15 @@ static __global__ void __launch_bounds__(256) x_to_operand_kernel(const float *_
 // MODE XP_SWIGLU: the row is silu(x) * nw, nw being a second [m, k] array (F.swiglu, F.java:1159-1161, in front of the
 // down projection of an FFN): the gated activations exist only as these operands.
 constexpr int XP_MAXJ = 8, XP_MAXK = XP_MAXJ * 256 * 8;
-constexpr int XP_PLAIN = 0, XP_NORM = 1, XP_SWIGLU = 2;
+// MODE XP_NORM_JOIN: XP_NORM on a row that does not exist yet - the linear in front of it split K and left its slices
+// unjoined: the row is x (the residual) + the slices part[z] [m, k] in slice order, exactly what prefill_join_kernel would
+// have stored; it is written to xsum [m, k] on the way (the next residual) and normalised from the registers.
+constexpr int XP_PLAIN = 0, XP_NORM = 1, XP_SWIGLU = 2, XP_NORM_JOIN = 3;
 template <int J, int MODE>
 __global__ void __launch_bounds__(256) x_prepare_kernel(const float *__restrict__ x, float *__restrict__ inv_scale, _Float16 *__restrict__ xo,
-                                                         int m, int k, const float *__restrict__ nw, float eps) {
-    constexpr bool NORM = MODE == XP_NORM;
+                                                         int m, int k, const float *__restrict__ nw, float eps, const float *__restrict__ part,
+                                                         int splits, float *__restrict__ xsum) {
+    constexpr bool NORM = MODE == XP_NORM || MODE == XP_NORM_JOIN;
     __shared__ float red[4];
     __shared__ float red2[4];
     const int b = blockIdx.x, tok = (b & ~63) | ((b & 7) << 3) | ((b >> 3) & 7), t = threadIdx.x;
@@ -123,6 +127,28 @@ __global__ void __launch_bounds__(256) x_prepare_kernel(const float *__restrict_
             const float4 *src = reinterpret_cast<const float4 *>(wr + min(8 * (t + 256 * j), k - 8));
             w[j][0] = src[0];
             w[j][1] = src[1];
+        }
+    }
+    if constexpr (MODE == XP_NORM_JOIN) {
+        const size_t row = (size_t)min(tok, m - 1) * k, slice = (size_t)m * k;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const int kk = min(8 * (t + 256 * j), k - 8);
+            float4 a[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) a[h] = reinterpret_cast<const float4 *>(part + row + kk)[h];
+            for (int z = 1; z < splits; ++z) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 b = reinterpret_cast<const float4 *>(part + z * slice + row + kk)[h];
+                    a[h] = make_float4(a[h].x + b.x, a[h].y + b.y, a[h].z + b.z, a[h].w + b.w);
+                }
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                v[j][h] = make_float4(a[h].x + v[j][h].x, a[h].y + v[j][h].y, a[h].z + v[j][h].z, a[h].w + v[j][h].w);
+                if (tok < m && 8 * (t + 256 * j) < k) reinterpret_cast<float4 *>(xsum + row + kk)[h] = v[j][h];
+            }
         }
     }
     if constexpr (MODE == XP_SWIGLU) {

@@ -23,19 +23,21 @@ void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg,
 }
 
 template <int MODE>
-static void prepare_one_launch(const float *x, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *nw, float eps, hipStream_t s) {
+static void prepare_one_launch(const float *x, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *nw, float eps, hipStream_t s,
+                               const float *part = nullptr, int splits = 0, float *xsum = nullptr) {
     const int pieces = pf_ksteps(k) * 2;  // per row; 256 threads take J each
-    if (pieces <= 512) hipLaunchKernelGGL((x_prepare_kernel<2, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
-    else if (pieces <= 1024) hipLaunchKernelGGL((x_prepare_kernel<4, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
-    else hipLaunchKernelGGL((x_prepare_kernel<8, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps);
+    if (pieces <= 512) hipLaunchKernelGGL((x_prepare_kernel<2, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps, part, splits, xsum);
+    else if (pieces <= 1024) hipLaunchKernelGGL((x_prepare_kernel<4, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps, part, splits, xsum);
+    else hipLaunchKernelGGL((x_prepare_kernel<8, MODE>), dim3(mblocks * 32), dim3(256), 0, s, x, inv_scale, xo, rows, k, nw, eps, part, splits, xsum);
 }
 
 bool prefill_prepare_fuses_norm(int k) { return k <= XP_MAXK; }
 
 void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *norm_w, float eps,
-                            const float *swiglu_up, hipStream_t s) {
+                            const float *swiglu_up, hipStream_t s, const PfPending *pend) {
     if (k <= XP_MAXK) {
-        if (swiglu_up) prepare_one_launch<XP_SWIGLU>(x, inv_scale, xo, rows, k, mblocks, swiglu_up, 0.f, s);
+        if (pend) prepare_one_launch<XP_NORM_JOIN>(pend->res, inv_scale, xo, rows, k, mblocks, norm_w, eps, s, pend->part, pend->splits, pend->out);
+        else if (swiglu_up) prepare_one_launch<XP_SWIGLU>(x, inv_scale, xo, rows, k, mblocks, swiglu_up, 0.f, s);
         else if (norm_w) prepare_one_launch<XP_NORM>(x, inv_scale, xo, rows, k, mblocks, norm_w, eps, s);
         else prepare_one_launch<XP_PLAIN>(x, inv_scale, xo, rows, k, mblocks, nullptr, 0.f, s);
     } else {  // (callers ask prefill_prepare_fuses_norm first: rows this long take no norm or gate here)

@@ -43,8 +43,17 @@ void prefill_launch_mixed(int fmt_a, int fmt_b, int first_b, dim3 grid, hipStrea
 // (norm_w != nullptr: RMSNorm with that weight and eps fused into the preparation; swiglu_up != nullptr: the activations
 // are silu(x) * swiglu_up, both [rows, k] - either only where prefill_prepare_fuses_norm(k))
 bool prefill_prepare_fuses_norm(int k);
+// The K slices of a linear whose join was left to the activation preparation that follows it: the row the preparation
+// normalises is res + the slices in slice order, and is stored to out on the way.
+struct PfPending {
+    const float *part = nullptr;  // [splits][rows, n]
+    const float *res = nullptr;   // [rows, n]
+    float *out = nullptr;         // [rows, n]
+    int splits = 0, n = 0;
+};
+// (pend != nullptr: x is ignored, the rows come from *pend - with norm_w and rows the preparation normalises only)
 void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *norm_w, float eps,
-                            const float *swiglu_up, hipStream_t s);
+                            const float *swiglu_up, hipStream_t s, const PfPending *pend = nullptr);
 void prefill_join_launch(const float *part, const float *bias, const float *res, float *y, size_t count4, int n, int splits, unsigned blocks,
                          hipStream_t s);
 // the join of a launch of several segments: part = per segment splits[i] arrays [m, n[i]], one segment after the other
