@@ -15,6 +15,10 @@ CONFIGS = [  # (format, n, k, batch sizes): BASELINE configs 1-4, and the 16 / 4
     ("Q4_0", 11008, 4096, (1, 4)),
     ("Q4_K", 14336, 4096, (1, 2, 8, 16, 40, 64)),
     ("Q6_K", 128256, 4096, (1,)),
+    # the other weights of a Q4_K_M / Q5_K_M layer at the row counts of a short prompt: ffn_down (long rows: the one-pass
+    # kernel from three rows on, two tiles per wave from 17) and a Q5_K gate
+    ("Q6_K", 4096, 14336, (1, 5, 40)),
+    ("Q5_K", 14336, 4096, (1, 16, 64)),
 ]
 
 
