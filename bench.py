@@ -546,6 +546,8 @@ def main() -> int:
             ("q8_0_4096x4096_b1", "Q8_0", 4096, 4096, 1, 24, 1010),
             ("q4_0_11008x4096_b1", "Q4_0", 11008, 4096, 1, 16, 1020),
             ("q4_0_11008x4096_b4", "Q4_0", 11008, 4096, 4, 16, 1020),
+            ("q4_0_11008x4096_b40", "Q4_0", 11008, 4096, 40, 16, 1020),
+            ("q8_0_4096x4096_b40", "Q8_0", 4096, 4096, 40, 24, 1010),
             ("q4_k_14336x4096_b2", "Q4_K", 14336, 4096, 2, 16, 1030),
             ("q4_k_14336x4096_b8", "Q4_K", 14336, 4096, 8, 16, 1030),
             ("q4_k_14336x4096_b16", "Q4_K", 14336, 4096, 16, 16, 1030),

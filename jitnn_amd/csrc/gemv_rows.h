@@ -42,7 +42,9 @@ __host__ __device__ constexpr size_t gemv_rows_lds_bytes(int tiles_per_wave) { r
 // order in which the weight decoders emit the bytes of a dword.  Operand 8, GS == 32: rows as above, slot j of the lanes
 // kq = 0 = sum of sub-block j of the scaled row / 64, the other lanes zero.  GS == 16 (Q6_K, whose scales cover 16 values):
 // slot j of the lanes kq = 0 and slot j - 8 of the lanes kq = 1 = sum of the 16-value group j / 64, sixteen groups.
-template <int GS>
+// HALVES (the 4-bit 32-value formats, whose byte i holds values i and i + 16 of a block): lane group kq holds values
+// 4 kq .. 4 kq + 3 and 16 + 4 kq .. + 3 of the sub-block instead of 8 kq .. 8 kq + 7, each four in the order 0 2 1 3.
+template <int GS, bool HALVES>
 __global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restrict__ x, _Float16 *__restrict__ ops, float *__restrict__ inv, int rows,
                                                            int k) {
     const int lane = threadIdx.x, b = lane >> 3, part = lane & 7;
@@ -66,7 +68,7 @@ __global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restric
     const float myinv = 1.f / scale;
     if (!have) scale = 0.f;
     uint8_t *base = reinterpret_cast<uint8_t *>(ops + ((size_t)g * ncol + c) * GR_OP_HALVES);
-    const int kq = part >> 1, h = part & 1;  // the quad `part` of a sub-block: lane group and half of its eight slots
+    const int kq = HALVES ? part & 3 : part >> 1, h = HALVES ? part >> 2 : part & 1;  // the quad `part` of a sub-block: lane group and half of its eight slots
     float sm = 0.f, sm2 = 0.f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
@@ -116,6 +118,9 @@ template <>
 struct RTile<F_Q4_K> {
     static constexpr int BYTES = 144;
     static constexpr int NOPS = 8, SUMS = 32;  // weight operands per tile and column, values per block sum
+    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true, STAGED = false;
+    static constexpr int STAGE_BYTES = 0;
+    typedef int Ptr;  // (see the 32-value formats below)
     __device__ static constexpr int aidx(int q) { return q; }  // the activation operand weight operand q meets
     struct Raw {
         u32x4 h;
@@ -150,6 +155,9 @@ template <>
 struct RTile<F_Q5_K> {
     static constexpr int BYTES = 176;
     static constexpr int NOPS = 8, SUMS = 32;
+    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true, STAGED = false;
+    static constexpr int STAGE_BYTES = 0;
+    typedef int Ptr;
     __device__ static constexpr int aidx(int q) { return q; }
     struct Raw {
         u32x4 h;
@@ -199,6 +207,9 @@ template <>
 struct RTile<F_Q6_K> {
     static constexpr int BYTES = 210;
     static constexpr int NOPS = 16, SUMS = 16;
+    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true, STAGED = false;
+    static constexpr int STAGE_BYTES = 0;
+    typedef int Ptr;
     __device__ static constexpr int aidx(int q) { return q >> 1; }  // operands 2 s (low nibble part) and 2 s + 1 (high bits) of step s
     struct Raw {
         u32x2 ql[4];  // [2 n + (ty & 1)]: bytes 64 n + 32 (ty & 1) + 8 kq .. + 7
@@ -260,6 +271,123 @@ struct RTile<F_Q6_K> {
     }
 };
 
+// The 32-value formats: a 256-value column of a row is eight blocks, each with an FP16 scale d of its own (and an FP16
+// offset m for Q4_1).  d times a quant is not an FP16 value, so nothing is folded: the operands are the quants as small
+// integers, the eight steps of a column keep eight separate sums, and each meets its block's d in FP32 (BLOCK_SCALES) -
+// what gemv_mfma_kernel does too, but once for all groups of activation rows.
+//
+// A lane needs four bytes (eight for Q8_0) of every block and the block's d: fetched like that, sixteen narrow loads per
+// tile and column, each touching sixteen lines, the launch is bound by the requests (46 us for 14336 x 4096 Q4_0 at 9
+// rows).  So the wave fetches the tile's bytes of the column once, sixteen bytes a lane (STAGED: four chunks of a row per
+// lane quad and load, the odd chunks in a last load), parks them in LDS of its own and every lane picks its pieces there.
+template <int BLOCK_BYTES, int ROW_STRIDE>
+struct RStaged {
+    static constexpr int BYTES = 8 * BLOCK_BYTES;  // of a row in a 256-value column: 144, 160, 272
+    static constexpr int CHUNKS = BYTES / 16, FULL = CHUNKS / 4, REST = CHUNKS % 4;
+    static constexpr int STRIDE = ROW_STRIDE;      // of a row in LDS: >= BYTES, a multiple of 16, and 4 * odd dwords where that is free
+    static constexpr int STAGE_BYTES = 16 * STRIDE;
+    static constexpr int NOPS = 8, SUMS = 32;
+    static constexpr bool BLOCK_SCALES = true, STAGED = true;
+    static_assert(BYTES % 16 == 0 && REST > 0 && STRIDE >= BYTES && STRIDE % 16 == 0, "chunks of sixteen bytes");
+    struct Raw {
+        u32x4 c[FULL + 1];
+    };
+    struct Ptr {
+        const uint8_t *full, *rest;
+    };
+    // r0: first row of the tile
+    __device__ static __forceinline__ Ptr ptr(const uint8_t *W, int r0, size_t rowbytes, int lane) {
+        return {W + (size_t)(r0 + (lane >> 2)) * rowbytes + 16 * (lane & 3), W + (size_t)(r0 + ((lane / REST) & 15)) * rowbytes + 16 * (4 * FULL + lane % REST)};
+    }
+    __device__ static __forceinline__ void load(Raw &r, const Ptr &p, int c) {
+#pragma unroll
+        for (int i = 0; i < FULL; ++i) r.c[i] = ld128<4>(p.full + (size_t)c * BYTES + 64 * i);
+        r.c[FULL] = ld128<4>(p.rest + (size_t)c * BYTES);  // (lanes past 16 REST repeat rows: the same lines)
+    }
+    // -> this lane's row (lane & 15 of the tile) in the wave's stage
+    __device__ static __forceinline__ const uint8_t *park(const Raw &r, uint8_t *stage, int lane) {
+#pragma unroll
+        for (int i = 0; i < FULL; ++i) *reinterpret_cast<u32x4 *>(stage + (lane >> 2) * STRIDE + 16 * (lane & 3) + 64 * i) = r.c[i];
+        if (lane < 16 * REST) *reinterpret_cast<u32x4 *>(stage + (lane / REST) * STRIDE + 16 * (4 * FULL + lane % REST)) = r.c[FULL];
+        // the lanes of a wave run in step and LDS serves them in order: a fence for the compiler is all this needs
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        return stage + (lane & 15) * STRIDE;
+    }
+};
+
+template <>
+struct RTile<F_Q4_0> : RStaged<18, 144> {
+    static constexpr bool HALVES = true, MINS = false;
+    __device__ static __forceinline__ void decode(const Raw &r, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float (&dblk)[8]) {
+        const uint8_t *row = park(r, stage, lane);
+        const int kq = lane >> 4;
+        const uint32_t mg = magic1024();
+        const f16x2 off = splat2(-1032.f);  // -1024 of the exponent trick, -8 of the format
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint32_t w = ld32<2>(row + 18 * s + 2 + 4 * kq);
+            // bytes 4 kq .. + 3: low nibbles = values 4 kq + (0 2 | 1 3), high nibbles = values 16 + 4 kq + (0 2 | 1 3)
+            B[s] = cat8(as_h2((w & 0x000f000fu) | mg) + off, as_h2(((w >> 8) & 0x000f000fu) | mg) + off,
+                        as_h2(((w >> 4) & 0x000f000fu) | mg) + off, as_h2(((w >> 12) & 0x000f000fu) | mg) + off);
+            dblk[s] = h2f(ld16(row + 18 * s));
+        }
+        Bm = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+};
+
+template <>
+struct RTile<F_Q4_1> : RStaged<20, 176> {
+    static constexpr bool HALVES = true, MINS = true;
+    __device__ static __forceinline__ void decode(const Raw &r, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float (&dblk)[8]) {
+        const uint8_t *row = park(r, stage, lane);
+        const int kq = lane >> 4;
+        const uint32_t mg = magic1024();
+        const f16x2 off = splat2(-1024.f);
+        uint32_t dm[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const uint32_t w = ld32<4>(row + 20 * s + 4 + 4 * kq);
+            B[s] = cat8(as_h2((w & 0x000f000fu) | mg) + off, as_h2(((w >> 8) & 0x000f000fu) | mg) + off,
+                        as_h2(((w >> 4) & 0x000f000fu) | mg) + off, as_h2(((w >> 12) & 0x000f000fu) | mg) + off);
+            dm[s] = ld32<4>(row + 20 * s);
+            dblk[s] = h2f(dm[s]);
+        }
+        // the offsets m of the eight blocks against the block sums of x: slot s of the lanes kq = 0, FP16 as they are
+        u32x4 mb;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mb[j] = kq == 0 ? (dm[2 * j] >> 16) | (dm[2 * j + 1] & 0xffff0000u) : 0u;
+        Bm = __builtin_bit_cast(f16x8, mb);
+    }
+};
+
+template <>
+struct RTile<F_Q8_0> : RStaged<34, 272> {
+    static constexpr bool HALVES = false, MINS = false;
+    __device__ static __forceinline__ void decode(const Raw &r, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float (&dblk)[8]) {
+        const uint8_t *row = park(r, stage, lane);
+        const int kq = lane >> 4;
+        const uint32_t mg = magic1024();
+        const f16x2 off = splat2(-1152.f);  // -1024 of the exponent trick, -128 of the sign flip below
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const u32x2 q = ld64<2>(row + 34 * s + 2 + 8 * kq);
+            const uint32_t w0 = q.x ^ 0x80808080u, w1 = q.y ^ 0x80808080u;  // int8 + 128: bytes 0 .. 255
+            B[s] = cat8(as_h2((w0 & 0x00ff00ffu) | mg) + off, as_h2(((w0 >> 8) & 0x00ff00ffu) | mg) + off,
+                        as_h2((w1 & 0x00ff00ffu) | mg) + off, as_h2(((w1 >> 8) & 0x00ff00ffu) | mg) + off);
+            dblk[s] = h2f(ld16(row + 34 * s));
+        }
+        Bm = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+};
+
+template <int FMT>
+__host__ __device__ constexpr size_t gemv_rows_stage_bytes(int tiles_per_wave) {
+    if constexpr (RTile<FMT>::STAGED) return (size_t)GR_WAVES * tiles_per_wave * RTile<FMT>::STAGE_BYTES;
+    else return 0;
+}
+
 // y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) (+ res[b, row]) for b < rows <= 8 * groups; k a multiple of 256, n >= 16.
 //   ops / inv: the output of rows_prepare_kernel<RTile<FMT>::SUMS> for the same x.  grid: up to one workgroup per batch of T tiles of 16
 //   weight rows (the host caps it at one per compute unit); GR_THREADS threads; gemv_rows_lds_bytes() of dynamic LDS.
@@ -276,6 +404,8 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
     float2 *accl = reinterpret_cast<float2 *>(gr_smem);  // [tile t][group g][thread]
     const int tid = threadIdx.x, lane = tid & 63, nq = lane & 15, kq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // (staged formats: behind accl, per wave and tile the sixteen rows of the column being decoded)
+    [[maybe_unused]] uint8_t *stage = gr_smem + gemv_rows_lds_bytes(T) + gemv_rows_stage_bytes<FMT>(T) / GR_WAVES * wave;
     const int ncol = k >> 8, ntiles = (n + 15) >> 4, nbatch = (ntiles + T - 1) / T;
     const size_t rowbytes = (size_t)ncol * R::BYTES;
 
@@ -283,35 +413,44 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
         // this lane's row of each tile of the batch (the last tile of a ragged matrix is the last 16 rows: in bounds, its
         // first rows computed twice, stored once)
         const uint8_t *rp[T];
+        [[maybe_unused]] typename R::Ptr sp[T];
         bool live[T];
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const int tile = tb * T + t;
             live[t] = tile < ntiles;  // workgroup-uniform
-            rp[t] = W + (size_t)(min((live[t] ? tile : ntiles - 1) * 16, n - 16) + nq) * rowbytes;
+            const int r0 = min((live[t] ? tile : ntiles - 1) * 16, n - 16);
+            rp[t] = W + (size_t)(r0 + nq) * rowbytes;
+            if constexpr (R::STAGED) sp[t] = R::ptr(W, r0, rowbytes, lane);
         }
         for (int i = tid; i < T * groups * GR_THREADS; i += GR_THREADS) accl[i] = make_float2(0.f, 0.f);
         // (each thread only ever touches its own slots of accl until the final reduction: no barrier needed here)
 
         typename R::Raw raw[T];
-        int c = wave;
-        if (c < ncol) {
+        auto fetch = [&](int col) {
 #pragma unroll
-            for (int t = 0; t < T; ++t) R::load(raw[t], rp[t] + (size_t)c * R::BYTES, kq);
-        }
+            for (int t = 0; t < T; ++t) {
+                if constexpr (R::STAGED) R::load(raw[t], sp[t], col);
+                else R::load(raw[t], rp[t] + (size_t)col * R::BYTES, kq);
+            }
+        };
+        int c = wave;
+        if (c < ncol) fetch(c);
         for (; c < ncol; c += GR_WAVES) {
             f16x8 B[T][NOPS], Bm[T];
             float d[T], dmin64[T];
+            float dblk[R::BLOCK_SCALES ? T : 1][8];
 #pragma unroll
             for (int t = 0; t < T; ++t) {
-                float dm;
-                R::decode(raw[t], B[t], Bm[t], d[t], dm);
-                dmin64[t] = dm * 64.f;
+                if constexpr (R::BLOCK_SCALES) {
+                    R::decode(raw[t], stage + t * R::STAGE_BYTES, lane, B[t], Bm[t], dblk[t]);
+                } else {
+                    float dm;
+                    R::decode(raw[t], B[t], Bm[t], d[t], dm);
+                    dmin64[t] = dm * 64.f;
+                }
             }
-            if (c + GR_WAVES < ncol) {  // the next column's bytes are on their way while this one meets the activations
-#pragma unroll
-                for (int t = 0; t < T; ++t) R::load(raw[t], rp[t] + (size_t)(c + GR_WAVES) * R::BYTES, kq);
-            }
+            if (c + GR_WAVES < ncol) fetch(c + GR_WAVES);  // the next column's bytes are on their way while this one meets the activations
             for (int g = 0; g < groups; ++g) {
                 const _Float16 *op = ops + ((size_t)g * ncol + c) * GR_OP_HALVES + lane * 8;
                 f16x8 A[9];
@@ -321,15 +460,33 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
 #pragma unroll
                 for (int t = 0; t < T; ++t) {
                     if (!live[t]) continue;
-                    f32x4 cs = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int s = 0; s < NOPS; ++s) cs = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[R::aidx(s)], B[t][s], cs, 0, 0, 0);
-                    const f32x4 cm = mfma16(A[8], Bm[t]);
                     // operand rows 4 kq + i: activation rows 2 kq (hi, lo) and 2 kq + 1 (hi, lo) of the group
-                    const float s0 = cs[0] + cs[1], s1 = cs[2] + cs[3], m0 = cm[0] + cm[1], m1 = cm[2] + cm[3];
+                    float u0, u1;
+                    if constexpr (R::BLOCK_SCALES) {
+                        u0 = u1 = 0.f;
+#pragma unroll
+                        for (int s = 0; s < 8; ++s) {  // eight independent products, each block sum with its own d
+                            const f32x4 cs = mfma16(A[s], B[t][s]);
+                            u0 = __builtin_fmaf(dblk[t][s], cs[0] + cs[1], u0);
+                            u1 = __builtin_fmaf(dblk[t][s], cs[2] + cs[3], u1);
+                        }
+                        if constexpr (R::MINS) {  // + m * (sum of x over the block): the sums were stored / 64
+                            const f32x4 cm = mfma16(A[8], Bm[t]);
+                            u0 = __builtin_fmaf(64.f, cm[0] + cm[1], u0);
+                            u1 = __builtin_fmaf(64.f, cm[2] + cm[3], u1);
+                        }
+                    } else {
+                        f32x4 cs = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int s = 0; s < NOPS; ++s) cs = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[R::aidx(s)], B[t][s], cs, 0, 0, 0);
+                        const f32x4 cm = mfma16(A[8], Bm[t]);
+                        const float s0 = cs[0] + cs[1], s1 = cs[2] + cs[3], m0 = cm[0] + cm[1], m1 = cm[2] + cm[3];
+                        u0 = __builtin_fmaf(d[t], s0, -dmin64[t] * m0);
+                        u1 = __builtin_fmaf(d[t], s1, -dmin64[t] * m1);
+                    }
                     float2 a = accl[(t * groups + g) * GR_THREADS + tid];
-                    a.x = __builtin_fmaf(iv.x, __builtin_fmaf(d[t], s0, -dmin64[t] * m0), a.x);
-                    a.y = __builtin_fmaf(iv.y, __builtin_fmaf(d[t], s1, -dmin64[t] * m1), a.y);
+                    a.x = __builtin_fmaf(iv.x, u0, a.x);
+                    a.y = __builtin_fmaf(iv.y, u1, a.y);
                     accl[(t * groups + g) * GR_THREADS + tid] = a;
                 }
             }

@@ -4,7 +4,7 @@
 
 namespace jitnn {
 
-bool gemv_rows_supported(int fmt) { return fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K; }
+bool gemv_rows_supported(int fmt) { return gemv_rows_layout(fmt) >= 0; }
 
 size_t gemv_rows_scratch_bytes(int rows, int k) {
     const int groups = (rows + 7) / 8;
@@ -20,32 +20,53 @@ static int tiles_per_wave(int n, int k, int rows, unsigned max_blocks) {
     return pairs >= max_blocks || (rows > 16 && k >= 8192 && 2 * pairs >= max_blocks) ? 2 : 1;
 }
 
+template <int FMT>
+static KernelRef kernel_ref(bool two) {
+    return {two ? (const void *)gemv_rows_kernel<FMT, 2> : (const void *)gemv_rows_kernel<FMT, 1>,
+            gemv_rows_lds_bytes(two ? 2 : 1) + gemv_rows_stage_bytes<FMT>(two ? 2 : 1)};
+}
+
 KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blocks) {
     const bool two = tiles_per_wave(n, k, rows, max_blocks) == 2;
-    const size_t lds = gemv_rows_lds_bytes(two ? 2 : 1);
     switch (fmt) {
-    case F_Q4_K: return {two ? (const void *)gemv_rows_kernel<F_Q4_K, 2> : (const void *)gemv_rows_kernel<F_Q4_K, 1>, lds};
-    case F_Q5_K: return {two ? (const void *)gemv_rows_kernel<F_Q5_K, 2> : (const void *)gemv_rows_kernel<F_Q5_K, 1>, lds};
-    case F_Q6_K: return {two ? (const void *)gemv_rows_kernel<F_Q6_K, 2> : (const void *)gemv_rows_kernel<F_Q6_K, 1>, lds};
+    case F_Q4_K: return kernel_ref<F_Q4_K>(two);
+    case F_Q5_K: return kernel_ref<F_Q5_K>(two);
+    case F_Q6_K: return kernel_ref<F_Q6_K>(two);
+    case F_Q4_0: return kernel_ref<F_Q4_0>(two);
+    case F_Q4_1: return kernel_ref<F_Q4_1>(two);
+    case F_Q8_0: return kernel_ref<F_Q8_0>(two);
     default: return {nullptr, 0};
     }
 }
 
-int gemv_rows_sums(int fmt) {
+template <int FMT>
+static constexpr int layout_of() {
+    using R = RTile<FMT>;
+    return R::SUMS == 16 ? GR_LAYOUT_SUMS16 : R::HALVES ? GR_LAYOUT_HALVES : GR_LAYOUT_PLAIN;
+}
+
+int gemv_rows_layout(int fmt) {
     switch (fmt) {
-    case F_Q4_K: return RTile<F_Q4_K>::SUMS;
-    case F_Q5_K: return RTile<F_Q5_K>::SUMS;
-    case F_Q6_K: return RTile<F_Q6_K>::SUMS;
-    default: return 0;
+    case F_Q4_K: return layout_of<F_Q4_K>();
+    case F_Q5_K: return layout_of<F_Q5_K>();
+    case F_Q6_K: return layout_of<F_Q6_K>();
+    case F_Q4_0: return layout_of<F_Q4_0>();
+    case F_Q4_1: return layout_of<F_Q4_1>();
+    case F_Q8_0: return layout_of<F_Q8_0>();
+    default: return -1;
     }
 }
 
-void gemv_rows_prepare_launch(int sums, hipStream_t s, const float *x, void *scratch, int k, int rows) {
+void gemv_rows_prepare_launch(int layout, hipStream_t s, const float *x, void *scratch, int k, int rows) {
     const int groups = (rows + 7) / 8, ncol = k / 256;
     _Float16 *ops = reinterpret_cast<_Float16 *>(scratch);
     float *inv = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
-    if (sums == 16) hipLaunchKernelGGL(rows_prepare_kernel<16>, dim3(ncol, groups), dim3(64), 0, s, x, ops, inv, rows, k);
-    else hipLaunchKernelGGL(rows_prepare_kernel<32>, dim3(ncol, groups), dim3(64), 0, s, x, ops, inv, rows, k);
+    const dim3 grid(ncol, groups);
+    switch (layout) {
+    case GR_LAYOUT_SUMS16: hipLaunchKernelGGL((rows_prepare_kernel<16, false>), grid, dim3(64), 0, s, x, ops, inv, rows, k); break;
+    case GR_LAYOUT_HALVES: hipLaunchKernelGGL((rows_prepare_kernel<32, true>), grid, dim3(64), 0, s, x, ops, inv, rows, k); break;
+    default: hipLaunchKernelGGL((rows_prepare_kernel<32, false>), grid, dim3(64), 0, s, x, ops, inv, rows, k); break;
+    }
 }
 
 template <int FMT>
@@ -56,8 +77,8 @@ static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const v
     const float *inv = reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
     const int T = tiles_per_wave(n, k, rows, max_blocks), nbatch = ((n + 15) / 16 + T - 1) / T;
     const unsigned blocks = (unsigned)nbatch < max_blocks ? (unsigned)nbatch : max_blocks;
-    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(2), s, W, ops, inv, bias, res, y, n, k, rows, groups);
-    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(1), s, W, ops, inv, bias, res, y, n, k, rows, groups);
+    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, bias, res, y, n, k, rows, groups);
+    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, bias, res, y, n, k, rows, groups);
 }
 
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,
@@ -66,6 +87,9 @@ void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const ui
     case F_Q4_K: launch<F_Q4_K>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
     case F_Q5_K: launch<F_Q5_K>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
     case F_Q6_K: launch<F_Q6_K>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
+    case F_Q4_0: launch<F_Q4_0>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
+    case F_Q4_1: launch<F_Q4_1>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
+    case F_Q8_0: launch<F_Q8_0>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
     default: break;
     }
 }

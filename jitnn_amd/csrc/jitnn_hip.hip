@@ -985,10 +985,16 @@ namespace {
 
 // Does a linear of `rows` rows on this weight take the one-pass kernel of gemv_rows.h?  From 9 rows; rows of 12288 values and
 // more - the ffn_down of an 8B layer, 4096 x 14336 - from 3: Q6_K 35.6 against 41.5-44.6 us, Q4_K 24.5 against 26.6-27.6,
-// where the kernels for up to 8 rows pay their activation set-up per 4096-value slice (at 8192 values they are still
-// ahead, 15.0 against 16.9).
+// Q4_0 22.3 against 25.4, Q8_0 27.2 against 34.4, where the kernels for up to 8 rows pay their activation set-up per
+// 4096-value slice (at 8192 values they are still ahead, 15.0 against 16.9).  Q4_0 and Q4_1 with shorter rows from 12: their
+// kernels for up to 8 rows are the fastest of all, and 8 + 1..3 rows in two passes still beat the one pass (14336 x 4096
+// Q4_0 at 9 rows 21.9 against 27.0 us, at 12 rows 26.2 against 27.0, at 20 rows 38.9 against 29.9).
 bool rows_path(const jitnn_hip_weight *w, int rows) {
-    const int rows_min = g.rows_kernel_min_set || w->k < 12288 ? g.rows_kernel_min : 3;
+    int rows_min = g.rows_kernel_min;
+    if (!g.rows_kernel_min_set) {
+        if (w->k >= 12288) rows_min = 3;
+        else if (w->fmt == F_Q4_0 || w->fmt == F_Q4_1) rows_min = 12;
+    }
     return g.rows_kernel_min > 0 && rows >= rows_min && rows <= 64 && rows <= g.gemv_max_rows && gemv_rows_supported(w->fmt) && w->k % 256 == 0 &&
            w->n >= 16 && !g.force_lds;
 }
@@ -998,22 +1004,26 @@ bool rows_path(const jitnn_hip_weight *w, int rows) {
 int launch_rows_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias, const float *residual,
                       hipStream_t s, ScratchSource src) {
     const int k = ws[0]->k;
-    bool need[2] = {false, false};  // block sums per 32 values, per 16 values
+    bool need[GR_LAYOUTS] = {};  // the operand layouts the weights ask for
     for (int i = 0; i < count; ++i) {
         if (ws[i]->k != k) return fail(JITNN_HIP_EINVAL, "weights of %d and %d values per row on one activation", k, ws[i]->k);
         const KernelRef kr = gemv_rows_kernel_ref(ws[i]->fmt, ws[i]->n, k, rows, (unsigned)g.cus);
         if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
-        need[gemv_rows_sums(ws[i]->fmt) == 16] = true;
+        need[gemv_rows_layout(ws[i]->fmt)] = true;
     }
     const size_t one = (gemv_rows_scratch_bytes(rows, k) + 255) & ~(size_t)255;
     void *scratch = nullptr;
-    if (int rc = workspace(one * ((int)need[0] + (int)need[1]), s, &scratch, src)) return rc;
-    uint8_t *sc32 = (uint8_t *)scratch, *sc16 = sc32 + (need[0] ? one : 0);
-    if (need[0]) gemv_rows_prepare_launch(32, s, x, sc32, k, rows);
-    if (need[1]) gemv_rows_prepare_launch(16, s, x, sc16, k, rows);
+    int layouts = 0;
+    for (int l = 0; l < GR_LAYOUTS; ++l) layouts += need[l];
+    if (int rc = workspace(one * layouts, s, &scratch, src)) return rc;
+    uint8_t *sc[GR_LAYOUTS] = {};
+    for (int l = 0, used = 0; l < GR_LAYOUTS; ++l) {
+        if (!need[l]) continue;
+        sc[l] = (uint8_t *)scratch + one * used++;
+        gemv_rows_prepare_launch(l, s, x, sc[l], k, rows);
+    }
     for (int i = 0; i < count; ++i)
-        gemv_rows_main_launch(ws[i]->fmt, (unsigned)g.cus, s, ws[i]->dev, gemv_rows_sums(ws[i]->fmt) == 16 ? sc16 : sc32, bias, residual, ys[i], ws[i]->n,
-                              k, rows);
+        gemv_rows_main_launch(ws[i]->fmt, (unsigned)g.cus, s, ws[i]->dev, sc[gemv_rows_layout(ws[i]->fmt)], bias, residual, ys[i], ws[i]->n, k, rows);
     HIP_TRY(hipGetLastError());
     return workspace_done(s, src);
 }

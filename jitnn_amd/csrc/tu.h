@@ -64,13 +64,15 @@ KernelRef gemv_mfma_kernel_ref(int fmt);
 void gemv_mfma_launch(int fmt, unsigned blocks, hipStream_t s, const uint8_t *W, const float *x, const float *bias, float *y, int n, int k, int rows);
 
 // ---- gemv_rows.hip: rows_prepare_kernel + gemv_rows_kernel<fmt>: 2..64 rows in one pass over the weights.  The operands of
-// the activations are prepared once (per granularity of the block sums a format needs: gemv_rows_sums, 32 or 16) into a
-// scratch of gemv_rows_scratch_bytes and serve every weight of that granularity that meets the same activations.
+// the activations are prepared once per operand layout a format needs (gemv_rows_layout: block sums per 32 or per 16
+// values, the values of a lane consecutive or in the two halves of a 4-bit block) into a scratch of
+// gemv_rows_scratch_bytes and serve every weight of that layout that meets the same activations.
+constexpr int GR_LAYOUT_PLAIN = 0, GR_LAYOUT_SUMS16 = 1, GR_LAYOUT_HALVES = 2, GR_LAYOUTS = 3;
 bool gemv_rows_supported(int fmt);
-int gemv_rows_sums(int fmt);
+int gemv_rows_layout(int fmt);                     // GR_LAYOUT_* of the format, -1: the kernel is not built for it
 size_t gemv_rows_scratch_bytes(int rows, int k);   // operands + scales of `rows` activation rows of k values
 KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blocks);  // the variant gemv_rows_main_launch picks for this shape
-void gemv_rows_prepare_launch(int sums, hipStream_t s, const float *x, void *scratch, int k, int rows);
+void gemv_rows_prepare_launch(int layout, hipStream_t s, const float *x, void *scratch, int k, int rows);
 // y = x W^T (+ bias [n]) (+ res [rows, n])
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,
                            int n, int k, int rows);

@@ -10,9 +10,9 @@ from helpers import BLOCK, GGML_ID, norm_err, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 
-CONFIGS = [  # (format, n, k, batch sizes): BASELINE configs 1-4, and the 16 / 40 / 64 rows bench.py times on config 3's matrix
-    ("Q8_0", 4096, 4096, (1,)),
-    ("Q4_0", 11008, 4096, (1, 4)),
+CONFIGS = [  # (format, n, k, batch sizes): BASELINE configs 1-4, and the 16 / 40 / 64 rows bench.py times on configs 1-3's matrices
+    ("Q8_0", 4096, 4096, (1, 40)),
+    ("Q4_0", 11008, 4096, (1, 4, 40)),
     ("Q4_K", 14336, 4096, (1, 2, 8, 16, 40, 64)),
     ("Q6_K", 128256, 4096, (1,)),
     # the other weights of a Q4_K_M / Q5_K_M layer at the row counts of a short prompt: ffn_down (long rows: the one-pass

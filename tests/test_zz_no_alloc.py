@@ -40,10 +40,10 @@ def test_noalloc_linear_matches_linear_dev(jn):
     rng = np.random.default_rng(12)
     g = torch.Generator(device="cuda").manual_seed(12)
     # 4096 x 4096 at 512 rows splits K into slices (partial sums in the scratch); the second call is smaller in every way
-    # (then: a ragged Q6_K launch, the one-pass kernel for 9..64 rows of Q4_K / Q5_K - its prepared operands live in the
-    # scratch too -, a 32-value format, and a GEMV call that needs no scratch at all)
+    # (then: a ragged Q6_K launch, the one-pass kernel for 9..64 rows of Q4_K / Q5_K / Q4_1 - its prepared operands live in
+    # the scratch too -, a 32-value format with rows of odd block counts, and a GEMV call that needs no scratch at all)
     calls = [("Q4_K", 4096, 4096, 512, True), ("Q6_K", 300, 1024, 97, False), ("Q4_K", 640, 2048, 40, True), ("Q5_K", 100, 1024, 17, False),
-             ("Q8_0", 131, 32 * 9, 70, True), ("Q4_K", 192, 2048, 5, False)]
+             ("Q4_1", 250, 1536, 33, True), ("Q8_0", 131, 32 * 9, 70, True), ("Q4_K", 192, 2048, 5, False)]
     for fmt, n, k, rows, with_bias in calls:
         w = jn.Tensor.quantized(jn.DType[fmt], random_valid_blocks(rng, fmt, n, k), n, k)
         x = torch.randn(rows, k, device="cuda", generator=g)
