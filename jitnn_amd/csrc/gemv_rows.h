@@ -114,25 +114,71 @@ struct RTile;
 
 __device__ __forceinline__ f16x2 h2fma(uint32_t bits, f16x2 mul, f16x2 add) { return __builtin_elementwise_fma(as_h2(bits), mul, add); }
 
-template <>
-struct RTile<F_Q4_K> {
-    static constexpr int BYTES = 144;
-    static constexpr int NOPS = 8, SUMS = 32;  // weight operands per tile and column, values per block sum
-    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true, STAGED = false;
-    static constexpr int STAGE_BYTES = 0;
-    typedef int Ptr;  // (see the 32-value formats below)
-    __device__ static constexpr int aidx(int q) { return q; }  // the activation operand weight operand q meets
+// How a wave gets a tile's bytes of a column (16 rows x BYTES).  A lane needs a few bytes of every field of its row's
+// block; fetched like that - each load instruction touching sixteen lines for 4 or 8 bytes a lane - the launch is bound by
+// the requests, not the bytes (14336 x 4096 Q4_0 at 9 rows: 46 us with sixteen narrow loads per tile and column, 27 us as
+// below).  So the wave fetches the bytes once, sixteen a lane (four chunks of a row per lane quad and load, the odd chunks
+// in a last load), parks them in LDS of its own and every lane picks its pieces there.
+// CHUNKS * 16 <= BYTES bytes of a row go this way (a format fetches a tail of its own); STRIDE: of a row in LDS, a
+// multiple of 16 and 4 * odd dwords where that is free (sixteen rows x four lane groups then hit 64 different banks).
+template <int ROW_BYTES, int ROW_STRIDE, int ALIGN>
+struct RStaged {
+    static constexpr int BYTES = ROW_BYTES;
+    static constexpr int CHUNKS = BYTES / 16, FULL = CHUNKS / 4, REST = CHUNKS % 4;
+    static constexpr int STRIDE = ROW_STRIDE;
+    static constexpr int STAGE_BYTES = 16 * STRIDE;
+    static constexpr bool STAGED = true;
+    static_assert(REST > 0 && STRIDE >= 16 * CHUNKS && STRIDE % 16 == 0, "chunks of sixteen bytes");
     struct Raw {
+        u32x4 c[FULL + 1];
+        uint32_t tail;  // (formats with bytes past the chunks)
+    };
+    struct Ptr {
+        const uint8_t *full;  // the lane's four-chunk loads
+        int rest, row;        // from there to its load of the odd chunks, and to the row lane & 15 (rows of a tile are < 2 GiB apart)
+    };
+    // r0: first row of the tile
+    __device__ static __forceinline__ Ptr ptr(const uint8_t *W, int r0, size_t rowbytes, int lane) {
+        const int rb = (int)rowbytes, lr = lane >> 2;
+        return {W + (size_t)(r0 + lr) * rowbytes + 16 * (lane & 3), (((lane / REST) & 15) - lr) * rb + 16 * (4 * FULL + lane % REST - (lane & 3)),
+                ((lane & 15) - lr) * rb - 16 * (lane & 3)};
+    }
+    __device__ static __forceinline__ void load(Raw &r, const Ptr &p, int c) {
+        const uint8_t *q = p.full + (size_t)c * BYTES;
+#pragma unroll
+        for (int i = 0; i < FULL; ++i) r.c[i] = ld128<ALIGN>(q + 64 * i);
+        r.c[FULL] = ld128<ALIGN>(q + p.rest);  // (lanes past 16 REST repeat rows: the same lines)
+    }
+    // -> this lane's row (lane & 15 of the tile) in the wave's stage
+    __device__ static __forceinline__ const uint8_t *park(const Raw &r, uint8_t *stage, int lane) {
+#pragma unroll
+        for (int i = 0; i < FULL; ++i) *reinterpret_cast<u32x4 *>(stage + (lane >> 2) * STRIDE + 16 * (lane & 3) + 64 * i) = r.c[i];
+        if (lane < 16 * REST) *reinterpret_cast<u32x4 *>(stage + (lane / REST) * STRIDE + 16 * (4 * FULL + lane % REST)) = r.c[FULL];
+        // the lanes of a wave run in step and LDS serves them in order: a fence for the compiler is all this needs
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        return stage + (lane & 15) * STRIDE;
+    }
+};
+
+template <>
+struct RTile<F_Q4_K> : RStaged<144, 144, 16> {
+    static constexpr int NOPS = 8, SUMS = 32;  // weight operands per tile and column, values per block sum
+    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true;
+    __device__ static constexpr int aidx(int q) { return q; }  // the activation operand weight operand q meets
+    struct Fields {
         u32x4 h;
         u32x2 q[4];
     };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *p, int kq) {
-        r.h = ld128<16>(p);
+    // B[s]: sc_s * q of sub-block s; Bm: the eight mins in the first eight K slots; d, dmin of the super-block
+    __device__ static __forceinline__ void decode(const Raw &raw, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float &d, float &dmin) {
+        const uint8_t *p = park(raw, stage, lane);
+        const int kq = lane >> 4;
+        Fields r;
+        r.h = *reinterpret_cast<const u32x4 *>(p);
 #pragma unroll
         for (int c = 0; c < 4; ++c) r.q[c] = *reinterpret_cast<const u32x2 *>(p + 16 + 32 * c + 8 * kq);
-    }
-    // B[s]: sc_s * q of sub-block s; Bm: the eight mins in the first eight K slots; d, dmin of the super-block
-    __device__ static __forceinline__ void decode(const Raw &r, f16x8 (&B)[8], f16x8 &Bm, float &d, float &dmin) {
         const K4Scales k = k4_scales(r.h);
         d = k.d;
         dmin = k.dmin;
@@ -152,25 +198,23 @@ struct RTile<F_Q4_K> {
 };
 
 template <>
-struct RTile<F_Q5_K> {
-    static constexpr int BYTES = 176;
+struct RTile<F_Q5_K> : RStaged<176, 176, 16> {
     static constexpr int NOPS = 8, SUMS = 32;
-    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true, STAGED = false;
-    static constexpr int STAGE_BYTES = 0;
-    typedef int Ptr;
+    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true;
     __device__ static constexpr int aidx(int q) { return q; }
-    struct Raw {
+    struct Fields {
         u32x4 h;
         u32x2 qh;
         u32x2 q[4];
     };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *p, int kq) {
-        r.h = ld128<16>(p);
+    __device__ static __forceinline__ void decode(const Raw &raw, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float &d, float &dmin) {
+        const uint8_t *p = park(raw, stage, lane);
+        const int kq = lane >> 4;
+        Fields r;
+        r.h = *reinterpret_cast<const u32x4 *>(p);
         r.qh = *reinterpret_cast<const u32x2 *>(p + 16 + 8 * kq);
 #pragma unroll
         for (int c = 0; c < 4; ++c) r.q[c] = *reinterpret_cast<const u32x2 *>(p + 48 + 32 * c + 8 * kq);
-    }
-    __device__ static __forceinline__ void decode(const Raw &r, f16x8 (&B)[8], f16x8 &Bm, float &d, float &dmin) {
         const K4Scales k = k4_scales(r.h);
         d = k.d;
         dmin = k.dmin;
@@ -204,29 +248,32 @@ struct RTile<F_Q5_K> {
 // both against the same activation operand; the -32 meets the sums of x per 16 values (operand 8 of
 // rows_prepare_kernel<16>) as 32 * sc, a multiple of 32 below 4100.
 template <>
-struct RTile<F_Q6_K> {
-    static constexpr int BYTES = 210;
+struct RTile<F_Q6_K> : RStaged<210, 208, 2> {
     static constexpr int NOPS = 16, SUMS = 16;
-    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true, STAGED = false;
-    static constexpr int STAGE_BYTES = 0;
-    typedef int Ptr;
+    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true;
     __device__ static constexpr int aidx(int q) { return q >> 1; }  // operands 2 s (low nibble part) and 2 s + 1 (high bits) of step s
-    struct Raw {
+    struct Fields {
         u32x2 ql[4];  // [2 n + (ty & 1)]: bytes 64 n + 32 (ty & 1) + 8 kq .. + 7
         u32x2 qh[2];  // [n]: bytes 32 n + 8 kq .. + 7
         u32x4 sc;
-        uint32_t d;
     };
-    __device__ static __forceinline__ void load(Raw &r, const uint8_t *p, int kq) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) r.ql[i] = ld64<2>(p + 32 * i + 8 * kq);
-#pragma unroll
-        for (int n = 0; n < 2; ++n) r.qh[n] = ld64<2>(p + 128 + 32 * n + 8 * kq);
-        r.sc = ld128<2>(p + 192);
-        r.d = ld16(p + 208);
+    // thirteen chunks and d, the last two bytes of the block, straight to the lanes of its row
+    __device__ static __forceinline__ void load(Raw &r, const Ptr &p, int c) {
+        RStaged<210, 208, 2>::load(r, p, c);
+        r.tail = ld16(p.full + (size_t)c * BYTES + p.row + 208);
     }
-    __device__ static __forceinline__ void decode(const Raw &r, f16x8 (&B)[16], f16x8 &Bm, float &d, float &dmin) {
-        d = h2f(r.d);
+    __device__ static __forceinline__ void decode(const Raw &raw, uint8_t *stage, int lane, f16x8 (&B)[16], f16x8 &Bm, float &d, float &dmin) {
+        const uint8_t *p = park(raw, stage, lane);
+        Fields r;
+        {
+            const int kq = lane >> 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r.ql[i] = *reinterpret_cast<const u32x2 *>(p + 32 * i + 8 * kq);
+#pragma unroll
+            for (int n = 0; n < 2; ++n) r.qh[n] = *reinterpret_cast<const u32x2 *>(p + 128 + 32 * n + 8 * kq);
+            r.sc = *reinterpret_cast<const u32x4 *>(p + 192);
+        }
+        d = h2f(raw.tail);
         dmin = d;  // the offset term is 32 * sc per group: y += d * (sum sc q x - 32 sum sc S)
         // FP16 64 + b with b in bits 4..7 of a half-word, 16 + a with a in bits 6, 7 (1024 + b, as the 6-bit scales of Q4_K
         // allow, would overflow: 1024 * 128)
@@ -275,51 +322,10 @@ struct RTile<F_Q6_K> {
 // offset m for Q4_1).  d times a quant is not an FP16 value, so nothing is folded: the operands are the quants as small
 // integers, the eight steps of a column keep eight separate sums, and each meets its block's d in FP32 (BLOCK_SCALES) -
 // what gemv_mfma_kernel does too, but once for all groups of activation rows.
-//
-// A lane needs four bytes (eight for Q8_0) of every block and the block's d: fetched like that, sixteen narrow loads per
-// tile and column, each touching sixteen lines, the launch is bound by the requests (46 us for 14336 x 4096 Q4_0 at 9
-// rows).  So the wave fetches the tile's bytes of the column once, sixteen bytes a lane (STAGED: four chunks of a row per
-// lane quad and load, the odd chunks in a last load), parks them in LDS of its own and every lane picks its pieces there.
-template <int BLOCK_BYTES, int ROW_STRIDE>
-struct RStaged {
-    static constexpr int BYTES = 8 * BLOCK_BYTES;  // of a row in a 256-value column: 144, 160, 272
-    static constexpr int CHUNKS = BYTES / 16, FULL = CHUNKS / 4, REST = CHUNKS % 4;
-    static constexpr int STRIDE = ROW_STRIDE;      // of a row in LDS: >= BYTES, a multiple of 16, and 4 * odd dwords where that is free
-    static constexpr int STAGE_BYTES = 16 * STRIDE;
-    static constexpr int NOPS = 8, SUMS = 32;
-    static constexpr bool BLOCK_SCALES = true, STAGED = true;
-    static_assert(BYTES % 16 == 0 && REST > 0 && STRIDE >= BYTES && STRIDE % 16 == 0, "chunks of sixteen bytes");
-    struct Raw {
-        u32x4 c[FULL + 1];
-    };
-    struct Ptr {
-        const uint8_t *full, *rest;
-    };
-    // r0: first row of the tile
-    __device__ static __forceinline__ Ptr ptr(const uint8_t *W, int r0, size_t rowbytes, int lane) {
-        return {W + (size_t)(r0 + (lane >> 2)) * rowbytes + 16 * (lane & 3), W + (size_t)(r0 + ((lane / REST) & 15)) * rowbytes + 16 * (4 * FULL + lane % REST)};
-    }
-    __device__ static __forceinline__ void load(Raw &r, const Ptr &p, int c) {
-#pragma unroll
-        for (int i = 0; i < FULL; ++i) r.c[i] = ld128<4>(p.full + (size_t)c * BYTES + 64 * i);
-        r.c[FULL] = ld128<4>(p.rest + (size_t)c * BYTES);  // (lanes past 16 REST repeat rows: the same lines)
-    }
-    // -> this lane's row (lane & 15 of the tile) in the wave's stage
-    __device__ static __forceinline__ const uint8_t *park(const Raw &r, uint8_t *stage, int lane) {
-#pragma unroll
-        for (int i = 0; i < FULL; ++i) *reinterpret_cast<u32x4 *>(stage + (lane >> 2) * STRIDE + 16 * (lane & 3) + 64 * i) = r.c[i];
-        if (lane < 16 * REST) *reinterpret_cast<u32x4 *>(stage + (lane / REST) * STRIDE + 16 * (4 * FULL + lane % REST)) = r.c[FULL];
-        // the lanes of a wave run in step and LDS serves them in order: a fence for the compiler is all this needs
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        return stage + (lane & 15) * STRIDE;
-    }
-};
-
 template <>
-struct RTile<F_Q4_0> : RStaged<18, 144> {
-    static constexpr bool HALVES = true, MINS = false;
+struct RTile<F_Q4_0> : RStaged<8 * 18, 144, 2> {
+    static constexpr int NOPS = 8, SUMS = 32;
+    static constexpr bool BLOCK_SCALES = true, HALVES = true, MINS = false;
     __device__ static __forceinline__ void decode(const Raw &r, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float (&dblk)[8]) {
         const uint8_t *row = park(r, stage, lane);
         const int kq = lane >> 4;
@@ -338,8 +344,9 @@ struct RTile<F_Q4_0> : RStaged<18, 144> {
 };
 
 template <>
-struct RTile<F_Q4_1> : RStaged<20, 176> {
-    static constexpr bool HALVES = true, MINS = true;
+struct RTile<F_Q4_1> : RStaged<8 * 20, 176, 4> {
+    static constexpr int NOPS = 8, SUMS = 32;
+    static constexpr bool BLOCK_SCALES = true, HALVES = true, MINS = true;
     __device__ static __forceinline__ void decode(const Raw &r, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float (&dblk)[8]) {
         const uint8_t *row = park(r, stage, lane);
         const int kq = lane >> 4;
@@ -363,8 +370,9 @@ struct RTile<F_Q4_1> : RStaged<20, 176> {
 };
 
 template <>
-struct RTile<F_Q8_0> : RStaged<34, 272> {
-    static constexpr bool HALVES = false, MINS = false;
+struct RTile<F_Q8_0> : RStaged<8 * 34, 272, 2> {
+    static constexpr int NOPS = 8, SUMS = 32;
+    static constexpr bool BLOCK_SCALES = true, HALVES = false, MINS = false;
     __device__ static __forceinline__ void decode(const Raw &r, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float (&dblk)[8]) {
         const uint8_t *row = park(r, stage, lane);
         const int kq = lane >> 4;
@@ -384,8 +392,7 @@ struct RTile<F_Q8_0> : RStaged<34, 272> {
 
 template <int FMT>
 __host__ __device__ constexpr size_t gemv_rows_stage_bytes(int tiles_per_wave) {
-    if constexpr (RTile<FMT>::STAGED) return (size_t)GR_WAVES * tiles_per_wave * RTile<FMT>::STAGE_BYTES;
-    else return 0;
+    return (size_t)GR_WAVES * tiles_per_wave * RTile<FMT>::STAGE_BYTES;
 }
 
 // y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) (+ res[b, row]) for b < rows <= 8 * groups; k a multiple of 256, n >= 16.
@@ -402,26 +409,24 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
     constexpr int NOPS = R::NOPS;
     extern __shared__ __attribute__((aligned(16))) uint8_t gr_smem[];
     float2 *accl = reinterpret_cast<float2 *>(gr_smem);  // [tile t][group g][thread]
-    const int tid = threadIdx.x, lane = tid & 63, nq = lane & 15, kq = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, kq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // (staged formats: behind accl, per wave and tile the sixteen rows of the column being decoded)
-    [[maybe_unused]] uint8_t *stage = gr_smem + gemv_rows_lds_bytes(T) + gemv_rows_stage_bytes<FMT>(T) / GR_WAVES * wave;
+    uint8_t *stage = gr_smem + gemv_rows_lds_bytes(T) + gemv_rows_stage_bytes<FMT>(T) / GR_WAVES * wave;
     const int ncol = k >> 8, ntiles = (n + 15) >> 4, nbatch = (ntiles + T - 1) / T;
     const size_t rowbytes = (size_t)ncol * R::BYTES;
 
     for (int tb = blockIdx.x; tb < nbatch; tb += gridDim.x) {
         // this lane's row of each tile of the batch (the last tile of a ragged matrix is the last 16 rows: in bounds, its
         // first rows computed twice, stored once)
-        const uint8_t *rp[T];
-        [[maybe_unused]] typename R::Ptr sp[T];
+        typename R::Ptr sp[T];
         bool live[T];
 #pragma unroll
         for (int t = 0; t < T; ++t) {
             const int tile = tb * T + t;
             live[t] = tile < ntiles;  // workgroup-uniform
             const int r0 = min((live[t] ? tile : ntiles - 1) * 16, n - 16);
-            rp[t] = W + (size_t)(r0 + nq) * rowbytes;
-            if constexpr (R::STAGED) sp[t] = R::ptr(W, r0, rowbytes, lane);
+            sp[t] = R::ptr(W, r0, rowbytes, lane);
         }
         for (int i = tid; i < T * groups * GR_THREADS; i += GR_THREADS) accl[i] = make_float2(0.f, 0.f);
         // (each thread only ever touches its own slots of accl until the final reduction: no barrier needed here)
@@ -429,10 +434,7 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
         typename R::Raw raw[T];
         auto fetch = [&](int col) {
 #pragma unroll
-            for (int t = 0; t < T; ++t) {
-                if constexpr (R::STAGED) R::load(raw[t], sp[t], col);
-                else R::load(raw[t], rp[t] + (size_t)col * R::BYTES, kq);
-            }
+            for (int t = 0; t < T; ++t) R::load(raw[t], sp[t], col);
         };
         int c = wave;
         if (c < ncol) fetch(c);
@@ -446,7 +448,7 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
                     R::decode(raw[t], stage + t * R::STAGE_BYTES, lane, B[t], Bm[t], dblk[t]);
                 } else {
                     float dm;
-                    R::decode(raw[t], B[t], Bm[t], d[t], dm);
+                    R::decode(raw[t], stage + t * R::STAGE_BYTES, lane, B[t], Bm[t], d[t], dm);
                     dmin64[t] = dm * 64.f;
                 }
             }
