@@ -11,13 +11,13 @@ size_t gemv_rows_scratch_bytes(int rows, int k) {
     return gemv_rows_ops_bytes(groups, k) + gemv_rows_inv_bytes(groups, k);
 }
 
-// Two tiles per wave where that still gives every CU a workgroup - or, for long rows (a wave then walks many columns) and
-// three groups of activation rows or more, every other CU: there the activation operands are what the launch waits for, and
-// two tiles share them (measured: Q6_K 4096 x 14336 at 40 rows 72.7 against 83.0 us; Q4_K 4096 x 4096 22.9 against 19.7, so
-// not for short rows) - else one.
-static int tiles_per_wave(int n, int k, int rows, unsigned max_blocks) {
+// Two tiles per wave where that still gives every CU a workgroup, else one - but Q6_K with long rows (a wave then walks
+// many columns) and three groups of activation rows or more keeps two even if only every other CU gets a workgroup: its
+// sixteen operands per tile make the activation operands what the launch waits for, and two tiles share them (4096 x 14336
+// at 40 rows: 64.9 against 81.1 us; Q4_K on the same shape 47.0 against 41.5, Q8_0 58.5 against 46.0 - so not for those).
+static int tiles_per_wave(int fmt, int n, int k, int rows, unsigned max_blocks) {
     const unsigned pairs = (unsigned)(((n + 15) / 16 + 1) / 2);
-    return pairs >= max_blocks || (rows > 16 && k >= 8192 && 2 * pairs >= max_blocks) ? 2 : 1;
+    return pairs >= max_blocks || (fmt == F_Q6_K && rows > 16 && k >= 8192 && 2 * pairs >= max_blocks) ? 2 : 1;
 }
 
 template <int FMT>
@@ -27,7 +27,7 @@ static KernelRef kernel_ref(bool two) {
 }
 
 KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blocks) {
-    const bool two = tiles_per_wave(n, k, rows, max_blocks) == 2;
+    const bool two = tiles_per_wave(fmt, n, k, rows, max_blocks) == 2;
     switch (fmt) {
     case F_Q4_K: return kernel_ref<F_Q4_K>(two);
     case F_Q5_K: return kernel_ref<F_Q5_K>(two);
@@ -75,7 +75,7 @@ static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const v
     const int groups = (rows + 7) / 8;
     const _Float16 *ops = reinterpret_cast<const _Float16 *>(scratch);
     const float *inv = reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
-    const int T = tiles_per_wave(n, k, rows, max_blocks), nbatch = ((n + 15) / 16 + T - 1) / T;
+    const int T = tiles_per_wave(FMT, n, k, rows, max_blocks), nbatch = ((n + 15) / 16 + T - 1) / T;
     const unsigned blocks = (unsigned)nbatch < max_blocks ? (unsigned)nbatch : max_blocks;
     if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, bias, res, y, n, k, rows, groups);
     else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, bias, res, y, n, k, rows, groups);
