@@ -114,7 +114,7 @@ JITNN_HIP_API int jitnn_hip_dequantize_dev(const jitnn_hip_weight *w, float *y_d
  * core/ops/Quant.java:66-80,147-187).  rows >= 1; bias may be NULL.
  * Up to 64 rows run the GEMV kernels at FP32-grade accuracy (error ~1e-6 of the largest output): FP32 arithmetic for
  * one and two rows, FP16 hi/lo splits of the activations on the matrix cores for more - 3 to 8 rows in one launch, 9 to
- * 64 rows of Q4_K / Q5_K / Q6_K in one pass over the weights, of the other formats in passes of 8; more rows (prefill) run the
+ * 64 rows in one pass over the weights (rows of whole 256-value columns; else in passes of 8); more rows (prefill) run the
  * dequantise-to-LDS MFMA kernel (FP16 operands, FP32 accumulation, error < 2e-3).
  * JITNN_HIP_GEMV_MAX_ROWS in the environment moves the switch. */
 JITNN_HIP_API int jitnn_hip_linear(const jitnn_hip_weight *w, const float *x_host, int rows, const float *bias_host, float *y_host);
