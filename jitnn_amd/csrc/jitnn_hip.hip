@@ -88,6 +88,7 @@ struct State {
     bool rows_kernel_min_set = false;  // JITNN_HIP_ROWS_MIN was given: no per-shape exceptions
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
+    bool prefill_dual = true;         // JITNN_HIP_PREFILL_DUAL=0: gate and up of a prefill step as two products, SwiGLU by the next preparation
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
     bool prefill_attn_mfma = true;  // JITNN_HIP_PREFILL_ATTN_MFMA=0: the FP16 attention of long prompts on v_dot2 instead of the matrix cores
     bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
@@ -730,6 +731,36 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
     return workspace_done(stream, src);
 }
 
+// h [rows, n] = silu(n(x) gate^T) * (n(x) up^T), n = RMSNorm with norm_w (which must fit the fused preparation): the gate
+// and the up projection of a Llama FFN as one product whose epilogue forms the SwiGLU - the two [rows, n] products are
+// neither stored nor read back.  pend: as in launch_prefill_group.
+bool prefill_dual_ok(const jitnn_hip_weight *gate, const jitnn_hip_weight *up) {
+    return g.prefill_dual && gate->fmt == up->fmt && gate->n == up->n && gate->k == up->k && !is_extra_format(gate->fmt) &&
+           prefill_prepare_fuses_norm(gate->k);
+}
+
+int launch_prefill_dual(const jitnn_hip_weight *gate, const jitnn_hip_weight *up, float *h, const float *x, int rows, const float *norm_w, float eps,
+                        hipStream_t stream, const PfPending *pend) {
+    const bool kq = block_values(gate->fmt) == 256;
+    const KernelRef kr = kq ? prefill_kernel_dual_k(gate->fmt) : prefill_kernel_dual_q32(gate->fmt);
+    if (!kr.fn) return fail(JITNN_HIP_EUNSUPPORTED, "no many-row kernel for format %d", gate->fmt);
+    if (int rc = allow_lds(kr.fn, kr.lds)) return rc;
+    const int k = gate->k, n = gate->n;
+    const int mtiles = (rows + PF_BM - 1) / PF_BM, mblocks = mtiles * (PF_BM / 32);
+    const size_t xo_bytes = (size_t)mblocks * pf_ksteps(k) * 1024;
+    const size_t scale_bytes = ((size_t)rows * 8 + 255) & ~(size_t)255;
+    void *wsp = nullptr;
+    if (int rc = workspace(xo_bytes + scale_bytes, stream, &wsp, SCRATCH_THREAD)) return rc;
+    _Float16 *xo = (_Float16 *)wsp;
+    float *scale = (float *)((uint8_t *)wsp + xo_bytes), *inv = scale + rows;
+    prefill_prepare_launch(x, scale, inv, xo, rows, k, mblocks, norm_w, eps, nullptr, stream, pend);
+    const dim3 grid((unsigned)((n + PF_BN / 2 - 1) / (PF_BN / 2)), mtiles);
+    if (kq) prefill_launch_dual_k(gate->fmt, grid, stream, gate->dev, up->dev, xo, inv, h, rows, n, k);
+    else prefill_launch_dual_q32(gate->fmt, grid, stream, gate->dev, up->dev, xo, inv, h, rows, n, k);
+    HIP_TRY(hipGetLastError());
+    return workspace_done(stream, SCRATCH_THREAD);
+}
+
 int launch_prefill(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream,
                    ScratchSource src = SCRATCH_THREAD) {
     return launch_prefill_group(&w, &y, 1, x, rows, bias, nullptr, 0.f, stream, nullptr, nullptr, nullptr, src);
@@ -846,6 +877,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_MFMA")) g.prefill_attn_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_PREFILL_DUAL")) g.prefill_dual = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
     g.ready = true;
@@ -1729,12 +1761,20 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         if (arc) return arc;
         // xa = x + Wo att, xb = xa + W2 (silu(W1 n) * (W3 n)), n = RMSNorm(xa)
         if (int rc = residual_linear_rows(w[JITNN_HIP_W_ATTN_O], att, T, x, xn, xa, st, nullptr, nullptr, m->pf[10], &pend)) return rc;
-        {
+        if (T > g.gemv_max_rows && prefill_dual_ok(w[JITNN_HIP_W_FFN_GATE], w[JITNN_HIP_W_FFN_UP])) {
+            // gate and up as one product with the SwiGLU in its epilogue: h = silu(W1 n) * (W3 n) directly
+            const bool fused = pend.part && pend.out == xa && pend.n == d;
+            if (!fused) flush_pending(pend, T, st);
+            const int rc = launch_prefill_dual(w[JITNN_HIP_W_FFN_GATE], w[JITNN_HIP_W_FFN_UP], h, xa, T, nw + d, m->eps, st, fused ? &pend : nullptr);
+            if (fused) pend = PfPending{};
+            if (rc) return rc;
+            if (int rc2 = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], h, T, xa, xn, xb, st, nullptr, nullptr, m->pf[10], &pend)) return rc2;
+        } else {
             const jitnn_hip_weight *ws[2] = {w[JITNN_HIP_W_FFN_GATE], w[JITNN_HIP_W_FFN_UP]};
             float *ys[2] = {gate, up};
             if (int rc = normed_linears_rows(m, ws, ys, 2, xa, T, nw + d, xn, st, &pend)) return rc;
+            if (int rc = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], gate, T, xa, xn, xb, st, up, h, m->pf[10], &pend)) return rc;
         }
-        if (int rc = residual_linear_rows(w[JITNN_HIP_W_FFN_DOWN], gate, T, xa, xn, xb, st, up, h, m->pf[10], &pend)) return rc;
         x = xb;
     }
     (void)qd;

@@ -495,21 +495,25 @@ __device__ __forceinline__ void pf_load_lds(PfRaw<FMT> &r, const uint8_t *b, int
 }
 
 // The work of one workgroup: row tile `tile` of the weight W [n, k] against token tile blockIdx.y, K slice `slice`.
-template <int FMT>
+// DUAL (the gate and up projections of a Llama FFN, F.swiglu, F.java:1159-1161): the tile is rows [64 tile, +64) of W in
+// its first two 32-row blocks and the same rows of W2 [n, k] in the other two, so that a lane holds the gate and the up
+// product of one output in the same element of two accumulators, and y [m, n] = silu(x W^T) * (x W2^T) - the two products
+// never go to memory.  No K slices, no bias.
+template <int FMT, bool DUAL = false>
 __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xo, const float *__restrict__ inv_scale,
                                                   const float *__restrict__ bias, float *__restrict__ y, const int m, const int n, const int k,
-                                                  const int split_steps, const int tile, const int slice) {
+                                                  const int split_steps, const int tile, const int slice, const uint8_t *__restrict__ W2 = nullptr) {
     using Stage = PfStage<FMT>;
     constexpr bool STAGED = Stage::ON;
     extern __shared__ __align__(16) uint8_t pf_smem[];  // pf_lds_bytes<FMT>()
     _Float16(*As)[PF_BN * PF_LD] = reinterpret_cast<_Float16(*)[PF_BN * PF_LD]>(pf_smem);  // dequantised weights [row][k], two steps
     uint8_t *Rs = pf_smem + 2 * PF_BN * PF_LD * 2;                                         // staged raw blocks [2][row][RP]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int n0 = tile * PF_BN, m0 = blockIdx.y * PF_BM;
+    const int n0 = tile * (DUAL ? PF_BN / 2 : PF_BN), m0 = blockIdx.y * PF_BM;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
     // dequantiser role: thread t fills weights [row t/2][32 * (t%2) ... +32) of the step
     const int drow = tid >> 1, dhalf = tid & 1;
-    const uint8_t *wrow = W + (size_t)min(n0 + drow, n - 1) * rowbytes;
+    const uint8_t *wrow = (DUAL && drow >= PF_BN / 2 ? W2 : W) + (size_t)min(n0 + (DUAL ? drow & (PF_BN / 2 - 1) : drow), n - 1) * rowbytes;
     // MFMA role: wave w owns all 128 output rows x tokens [64 w, +64) as 4 x 2 tiles of 32 x 32: every weight operand
     // read from LDS feeds two MFMAs, every activation operand loaded from L2 feeds four
     const int ksteps = pf_ksteps(k);
@@ -684,6 +688,24 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
     for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) isc[j][r] = inv_scale[min(tok0 + 32 * j + 8 * (r >> 2) + (r & 3), m - 1)];
+    if constexpr (DUAL) {
+        // (the same expression, on the same two floats, as the activation preparation that forms silu(gate) * up from
+        // stored products: XP_SWIGLU)
+        auto sw = [](float g, float u) { return (g / (1.f + __expf(-g))) * u; };
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int row = n0 + 32 * i + (lane & 31);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int tok = tok0 + 32 * j + 8 * (r >> 2) + (r & 3);
+                    if (row < n && tok < m) y[(size_t)tok * n + row] = sw(acc[i][j][r] * isc[j][r], acc[i + 2][j][r] * isc[j][r]);
+                }
+            }
+        }
+        return;
+    }
     float bv[4];
     {
         const float *bp = bias ? bias : inv_scale;  // some readable address when there is no bias: the value is dropped
@@ -746,6 +768,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
     pf_locate(sg, seg, tile, slice);
     if (seg < first_b) prefill_mfma_body<FA>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
     else prefill_mfma_body<FB>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+}
+
+// y [m, n] = silu(x W^T) * (x W2^T) for two weights [n, k] of one format: grid (ceil(n / 64), token tiles).
+template <int FMT>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) prefill_mfma_dual_kernel(const uint8_t *__restrict__ W,
+                                                                                                            const uint8_t *__restrict__ W2,
+                                                                                                            const _Float16 *__restrict__ xo,
+                                                                                                            const float *__restrict__ inv_scale,
+                                                                                                            float *__restrict__ y, int m, int n, int k) {
+    prefill_mfma_body<FMT, true>(W, xo, inv_scale, nullptr, y, m, n, k, (k + PF_BK - 1) / PF_BK, blockIdx.x, 0, W2);
 }
 
 // y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]) (+ res[tok, row]), slices in order: the second half of a

@@ -39,6 +39,14 @@ void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg,
                         int k);
 void prefill_launch_mixed(int fmt_a, int fmt_b, int first_b, dim3 grid, hipStream_t s, const PfSegments &sg, const _Float16 *xo, const float *inv_scale,
                           int m, int k);
+// prefill_dual_k.hip, prefill_dual_q32.hip: prefill_mfma_dual_kernel<fmt>, y [m, n] = silu(x W^T) * (x W2^T) for two weights
+// [n, k] of one format; grid (ceil(n / 64), token tiles)
+KernelRef prefill_kernel_dual_k(int fmt);
+KernelRef prefill_kernel_dual_q32(int fmt);
+void prefill_launch_dual_k(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const uint8_t *W2, const _Float16 *xo, const float *inv_scale, float *y,
+                           int m, int n, int k);
+void prefill_launch_dual_q32(int fmt, dim3 grid, hipStream_t s, const uint8_t *W, const uint8_t *W2, const _Float16 *xo, const float *inv_scale, float *y,
+                             int m, int n, int k);
 // activation preparation and the join of K slices (prefill_q32.hip)
 // (norm_w != nullptr: RMSNorm with that weight and eps fused into the preparation; swiglu_up != nullptr: the activations
 // are silu(x) * swiglu_up, both [rows, k] - either only where prefill_prepare_fuses_norm(k))

@@ -175,6 +175,28 @@ def test_prefill_head_shapes(jn, heads, kv_heads, head_dim, tokens, bar):
     dec.close()
 
 
+@pytest.mark.parametrize("fmt,ffn", [("Q4_K", 768), ("Q5_K", 768), ("Q6_K", 768), ("Q4_0", 1056), ("Q4_1", 1056), ("Q8_0", 1056)])
+def test_prefill_ffn_formats(jn, fmt, ffn):
+    """A prompt beyond the GEMV range in every format: the gate and up projections are one matrix-core product with the
+    SwiGLU in its epilogue (64 gate rows and 64 up rows per workgroup; 1056 rows leave the last tile half empty), 130
+    tokens are a whole token tile and a ragged one."""
+    cfg = dict(layers=1, d_model=512, heads=4, kv_heads=2, head_dim=128, ffn=ffn, vocab=300, max_ctx=160, rms_eps=1e-5, rope_theta=5e5)
+    dec, layers, out_norm, out_w = build(jn, cfg, 23, {s: fmt for s in SLOTS}, "Q8_0")
+    rng = np.random.default_rng(6)
+    tokens, pos0 = 130, 3
+    kc = np.zeros((1, cfg["max_ctx"], 2, 128), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :pos0] = rng.standard_normal(kc[:, :pos0].shape)
+    vc[:, :pos0] = rng.standard_normal(vc[:, :pos0].shape)
+    dec.kv_write(0, 0, kc[0, :pos0], vc[0, :pos0])
+    x = rng.standard_normal((tokens, cfg["d_model"])).astype(np.float32)
+    for t in range(tokens):
+        ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x[t], pos0 + t)
+    y = dec.prefill(x, pos0)
+    assert norm_err(y, ref) <= 5e-3, (fmt, norm_err(y, ref))
+    dec.close()
+
+
 @pytest.mark.parametrize("heads,kv_heads,head_dim", [(4, 4, 128), (8, 2, 128), (8, 1, 64), (5, 1, 64), (6, 3, 128)])
 def test_prefill_long_prompt_attention(jn, heads, kv_heads, head_dim):
     """The matrix-core attention of long prompts on several key chunks: groups of 1, 2, 4, 5 and 8 query heads per key/value
