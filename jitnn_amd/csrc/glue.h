@@ -246,6 +246,52 @@ __global__ void __launch_bounds__(256) rope_append_rows_kernel(float *__restrict
     for (int i = threadIdx.x; i < kv_heads * D; i += 256) vc[i] = vt[i];
 }
 
+// The same on projections that still lie in K slices (the many-row launch of q, k and v split K and left the join to this
+// kernel): part holds splits[0] arrays [T, nq] of partial sums of q, then splits[1] arrays [T, nk] of k, then splits[2]
+// arrays [T, nk] of v; an element is the sum of its slices in slice order, as the join kernel would have stored it.  The
+// rotated queries go to q [T, heads, D].
+__global__ void __launch_bounds__(256) rope_append_rows_join_kernel(const float *__restrict__ part, int s0, int s1, int s2, int T, float *__restrict__ q,
+                                                                     float *__restrict__ kcache, float *__restrict__ vcache,
+                                                                     const float *__restrict__ cosv, const float *__restrict__ sinv, int heads,
+                                                                     int kv_heads, int D, int pos0, int interleaved) {
+    const int t = blockIdx.x, pos = pos0 + t, half = D / 2;
+    const int nq = heads * D, nk = kv_heads * D;
+    const size_t zq = (size_t)T * nq, zk = (size_t)T * nk;  // floats per slice
+    const float *pq = part + (size_t)t * nq, *pk = part + zq * s0 + (size_t)t * nk, *pv = part + zq * s0 + zk * s1 + (size_t)t * nk;
+    const float *cp = cosv + (size_t)pos * half, *sp = sinv + (size_t)pos * half;
+    float *qt = q + (size_t)t * nq;
+    for (int i = threadIdx.x; i < heads * half; i += 256) {
+        const int h = i / half, p = i - h * half;
+        const int i0 = h * D + (interleaved ? 2 * p : p), i1 = h * D + (interleaved ? 2 * p + 1 : p + half);
+        float a = pq[i0], b = pq[i1];
+        for (int z = 1; z < s0; ++z) {
+            a += pq[z * zq + i0];
+            b += pq[z * zq + i1];
+        }
+        const float cs = cp[p], sn = sp[p];
+        qt[i0] = a * cs - b * sn;
+        qt[i1] = a * sn + b * cs;
+    }
+    float *kc = kcache + (size_t)pos * nk, *vc = vcache + (size_t)pos * nk;
+    for (int i = threadIdx.x; i < kv_heads * half; i += 256) {
+        const int h = i / half, p = i - h * half;
+        const int i0 = h * D + (interleaved ? 2 * p : p), i1 = h * D + (interleaved ? 2 * p + 1 : p + half);
+        float a = pk[i0], b = pk[i1];
+        for (int z = 1; z < s1; ++z) {
+            a += pk[z * zk + i0];
+            b += pk[z * zk + i1];
+        }
+        const float cs = cp[p], sn = sp[p];
+        kc[i0] = a * cs - b * sn;
+        kc[i1] = a * sn + b * cs;
+    }
+    for (int i = threadIdx.x; i < nk; i += 256) {
+        float a = pv[i];
+        for (int z = 1; z < s2; ++z) a += pv[z * zk + i];
+        vc[i] = a;
+    }
+}
+
 // Causal attention of a block of consecutive tokens: the (token, query head) pairs of one key/value head - ATT_ROWS
 // rows, i.e. ATT_ROWS / group tokens - walk the keys in chunks of CH, each chunk staged once in LDS for all of them; row
 // r = tq * group + h sees key j when j <= pos0 + t0 + tq.  q is already rotated, every key comes from the cache.

@@ -88,6 +88,7 @@ struct State {
     bool rows_kernel_min_set = false;  // JITNN_HIP_ROWS_MIN was given: no per-shape exceptions
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
+    bool prefill_rope_join = true;    // JITNN_HIP_PREFILL_ROPE_JOIN=0: the K slices of q, k and v of a prefill step joined by a kernel of its own
     bool prefill_dual = true;         // JITNN_HIP_PREFILL_DUAL=0: gate and up of a prefill step as two products, SwiGLU by the next preparation
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
     bool prefill_attn_mfma = true;  // JITNN_HIP_PREFILL_ATTN_MFMA=0: the FP16 attention of long prompts on v_dot2 instead of the matrix cores
@@ -597,7 +598,7 @@ int stage_reserve(size_t pinned_bytes, size_t dev_bytes) {
 int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias,
                          const float *norm_w, float eps, hipStream_t stream, const float *residual = nullptr, float *tmp = nullptr,
                          const float *swiglu_up = nullptr, ScratchSource src = SCRATCH_THREAD, float *part_ext = nullptr, PfPending *defer = nullptr,
-                         const PfPending *pend = nullptr) {
+                         const PfPending *pend = nullptr, PfGroupPending *gdefer = nullptr) {
     // (the kernels live in prefill_k.hip, prefill_q32.hip and prefill_mixed.hip)
     // Weights of one format - and a run of one K-quant format followed by a run of another for which a two-format kernel
     // exists - share a launch: their row tiles are numbered one after the other, so that the 1024-row k and v projections
@@ -705,7 +706,12 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
         if (l.first_b < l.count) prefill_launch_mixed(w->fmt, ws[l.first + l.first_b]->fmt, l.first_b, grid, stream, sg, xo, inv, rows, k);
         else if (kq(w)) prefill_launch_k(w->fmt, grid, stream, sg, xo, inv, b1, rows, k);
         else prefill_launch_q32(w->fmt, grid, stream, sg, xo, inv, b1, rows, k);
-        if (split && l.count > 1) {  // (the stream orders the next launch's partial sums after this join)
+        if (split && l.count > 1 && gdefer && nlaunch == 1) {
+            // the caller's next kernel adds the slices up as it reads them (they stay in this thread's scratch until its
+            // next many-row call)
+            gdefer->part = part;
+            gdefer->sg = out;
+        } else if (split && l.count > 1) {  // (the stream orders the next launch's partial sums after this join)
             size_t count4 = 0;
             for (int q = 0; q < l.count; ++q) count4 += (size_t)rows * sg.n[q] / 4;
             const unsigned blocks = (unsigned)std::min<size_t>((count4 + 255) / 256, (size_t)g.cus * 8);
@@ -878,6 +884,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_MFMA")) g.prefill_attn_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_DUAL")) g.prefill_dual = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_PREFILL_ROPE_JOIN")) g.prefill_rope_join = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
     g.ready = true;
@@ -1429,13 +1436,13 @@ void flush_pending(PfPending &p, int rows, hipStream_t st) {
 
 // (pend: x - the output of the linear before - may still be in K slices; the shared preparation then adds them up)
 int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows,
-                        const float *nw, float *xn, hipStream_t st, PfPending *pend = nullptr) {
+                        const float *nw, float *xn, hipStream_t st, PfPending *pend = nullptr, PfGroupPending *gdefer = nullptr) {
     bool group = rows > g.gemv_max_rows && prefill_prepare_fuses_norm(m->d);
     for (int i = 0; i < count; ++i) group = group && !is_extra_format(ws[i]->fmt);
     if (group) {
         const bool fused = pend && pend->part && pend->out == x && pend->n == m->d;
         const int rc = launch_prefill_group(ws, ys, count, x, rows, nullptr, nw, m->eps, st, nullptr, nullptr, nullptr, SCRATCH_THREAD, nullptr, nullptr,
-                                            fused ? pend : nullptr);
+                                            fused ? pend : nullptr, gdefer);
         if (fused) *pend = PfPending{};
         else if (pend) flush_pending(*pend, rows, st);  // (never both: a pending join is flushed before anybody reads its row)
         return rc;
@@ -1740,6 +1747,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
           *up = m->pf[8], *h = m->pf[9];
     const float *x = x_dev;
     PfPending pend;  // the K slices of the linear that wrote x, when their join is still to come
+    PfGroupPending gp;  // the K slices of q, k and v between their launch and the rotation
     for (int l = 0; l < m->layers; ++l) {
         const jitnn_hip_weight *const *w = m->w + (size_t)l * 7;
         const float *nw = m->norms + (size_t)l * 2 * d;
@@ -1747,10 +1755,16 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         {
             const jitnn_hip_weight *ws[3] = {w[JITNN_HIP_W_ATTN_Q], w[JITNN_HIP_W_ATTN_K], w[JITNN_HIP_W_ATTN_V]};
             float *ys[3] = {q, k, v};
-            if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st, &pend)) return rc;
+            if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st, &pend, g.prefill_rope_join ? &gp : nullptr)) return rc;
         }
-        hipLaunchKernelGGL(rope_append_rows_kernel, dim3(T), dim3(256), 0, st, q, k, v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads, m->kv, m->hd,
-                           pos0, m->rope_interleaved);
+        if (gp.part) {  // q, k and v still lie in K slices: the rotation adds them up as it reads them
+            hipLaunchKernelGGL(rope_append_rows_join_kernel, dim3(T), dim3(256), 0, st, gp.part, gp.sg.splits[0], gp.sg.splits[1], gp.sg.splits[2], T, q,
+                               m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads, m->kv, m->hd, pos0, m->rope_interleaved);
+            gp.part = nullptr;
+        } else {
+            hipLaunchKernelGGL(rope_append_rows_kernel, dim3(T), dim3(256), 0, st, q, k, v, m->kc + lo, m->vc + lo, m->cosv, m->sinv, m->heads, m->kv,
+                               m->hd, pos0, m->rope_interleaved);
+        }
         int arc;
         switch (m->hd) {
         case 64: arc = launch_attention_rows<64>(m, l, pos0, T, q, att, st); break;

@@ -59,6 +59,12 @@ struct PfPending {
     float *out = nullptr;         // [rows, n]
     int splits = 0, n = 0;
 };
+// The K slices of a launch of several segments whose join was left to the kernel that reads the products next: part holds,
+// segment after segment, sg.splits[i] arrays [rows, sg.n[i]].
+struct PfGroupPending {
+    const float *part = nullptr;
+    PfSegments sg;
+};
 // (pend != nullptr: x is ignored, the rows come from *pend - with norm_w and rows the preparation normalises only)
 void prefill_prepare_launch(const float *x, float *scale, float *inv_scale, _Float16 *xo, int rows, int k, int mblocks, const float *norm_w, float eps,
                             const float *swiglu_up, hipStream_t s, const PfPending *pend = nullptr);
