@@ -44,17 +44,11 @@ __host__ __device__ constexpr size_t gemv_rows_lds_bytes(int tiles_per_wave) { r
 // slot j of the lanes kq = 0 and slot j - 8 of the lanes kq = 1 = sum of the 16-value group j / 64, sixteen groups.
 // HALVES (the 4-bit 32-value formats, whose byte i holds values i and i + 16 of a block): lane group kq holds values
 // 4 kq .. 4 kq + 3 and 16 + 4 kq .. + 3 of the sub-block instead of 8 kq .. 8 kq + 7, each four in the order 0 2 1 3.
+// The work of one wave: column c of group g, the lane's eight quads v of its row already loaded (and normalised / gated).
 template <int GS, bool HALVES>
-__global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restrict__ x, _Float16 *__restrict__ ops, float *__restrict__ inv, int rows,
-                                                           int k) {
-    const int lane = threadIdx.x, b = lane >> 3, part = lane & 7;
-    const int c = blockIdx.x, g = blockIdx.y, ncol = k >> 8;
-    const int row = g * 8 + b;
-    const bool have = row < rows;
-    const float *xp = x + (size_t)(have ? row : 0) * k + (size_t)c * 256 + 4 * part;
-    float4 v[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t) v[t] = *reinterpret_cast<const float4 *>(xp + 32 * t);
+__device__ __forceinline__ void rows_prepare_column(const float4 (&v)[8], _Float16 *__restrict__ ops, float *__restrict__ inv, int c, int g, int ncol,
+                                                    bool have, int lane) {
+    const int b = lane >> 3, part = lane & 7;
     float amax = 0.f;
 #pragma unroll
     for (int t = 0; t < 8; ++t) amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[t].x), fabsf(v[t].y)), fmaxf(fabsf(v[t].z), fabsf(v[t].w))));
@@ -105,6 +99,37 @@ __global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restric
         sop[(16 + 2 * b + 1) * 8 + part] = tlo;
     }
     if (part == 0) inv[((size_t)g * ncol + c) * 8 + b] = myinv;
+}
+
+// One wave per (column c = blockIdx.x, group g = blockIdx.y): the lane's eight quads of its row, once, into every operand
+// layout somebody asked for (weights of several kinds on one activation).  SWIGLU: the rows are silu(x) * up, up [rows, k]
+// (F.swiglu, F.java:1159-1161) - the expression of swiglu_kernel.
+struct RowsPrepareOut {
+    _Float16 *ops[3];  // per layout (plain, sums per 16 values, halves): nullptr = not wanted
+    float *inv[3];
+};
+template <bool SWIGLU>
+__global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restrict__ x, const float *__restrict__ up, const RowsPrepareOut o, int rows,
+                                                           int k) {
+    const int lane = threadIdx.x, b = lane >> 3, part = lane & 7;
+    const int c = blockIdx.x, g = blockIdx.y, ncol = k >> 8;
+    const int row = g * 8 + b;
+    const bool have = row < rows;
+    const size_t at = (size_t)(have ? row : 0) * k + (size_t)c * 256 + 4 * part;
+    float4 v[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) v[t] = *reinterpret_cast<const float4 *>(x + at + 32 * t);
+    if constexpr (SWIGLU) {
+        auto sw = [](float gt, float u) { return (gt / (1.f + __expf(-gt))) * u; };
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const float4 u = *reinterpret_cast<const float4 *>(up + at + 32 * t);
+            v[t] = make_float4(sw(v[t].x, u.x), sw(v[t].y, u.y), sw(v[t].z, u.z), sw(v[t].w, u.w));
+        }
+    }
+    if (o.ops[0]) rows_prepare_column<32, false>(v, o.ops[0], o.inv[0], c, g, ncol, have, lane);
+    if (o.ops[1]) rows_prepare_column<16, false>(v, o.ops[1], o.inv[1], c, g, ncol, have, lane);
+    if (o.ops[2]) rows_prepare_column<32, true>(v, o.ops[2], o.inv[2], c, g, ncol, have, lane);
 }
 
 // Per format: the bytes a lane (weight row n = lane & 15 of the tile, lane group kq = lane >> 4) fetches of a 256-value

@@ -57,16 +57,19 @@ int gemv_rows_layout(int fmt) {
     }
 }
 
-void gemv_rows_prepare_launch(int layout, hipStream_t s, const float *x, void *scratch, int k, int rows) {
+static_assert(GR_LAYOUT_PLAIN == 0 && GR_LAYOUT_SUMS16 == 1 && GR_LAYOUT_HALVES == 2 && GR_LAYOUTS == 3, "RowsPrepareOut is indexed by layout");
+
+void gemv_rows_prepare_launch(hipStream_t s, const float *x, const float *swiglu_up, void *const *scratch, int k, int rows) {
     const int groups = (rows + 7) / 8, ncol = k / 256;
-    _Float16 *ops = reinterpret_cast<_Float16 *>(scratch);
-    float *inv = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
-    const dim3 grid(ncol, groups);
-    switch (layout) {
-    case GR_LAYOUT_SUMS16: hipLaunchKernelGGL((rows_prepare_kernel<16, false>), grid, dim3(64), 0, s, x, ops, inv, rows, k); break;
-    case GR_LAYOUT_HALVES: hipLaunchKernelGGL((rows_prepare_kernel<32, true>), grid, dim3(64), 0, s, x, ops, inv, rows, k); break;
-    default: hipLaunchKernelGGL((rows_prepare_kernel<32, false>), grid, dim3(64), 0, s, x, ops, inv, rows, k); break;
+    RowsPrepareOut o{};
+    for (int l = 0; l < GR_LAYOUTS; ++l) {
+        if (!scratch[l]) continue;
+        o.ops[l] = reinterpret_cast<_Float16 *>(scratch[l]);
+        o.inv[l] = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(scratch[l]) + gemv_rows_ops_bytes(groups, k));
     }
+    const dim3 grid(ncol, groups);
+    if (swiglu_up) hipLaunchKernelGGL(rows_prepare_kernel<true>, grid, dim3(64), 0, s, x, swiglu_up, o, rows, k);
+    else hipLaunchKernelGGL(rows_prepare_kernel<false>, grid, dim3(64), 0, s, x, swiglu_up, o, rows, k);
 }
 
 template <int FMT>

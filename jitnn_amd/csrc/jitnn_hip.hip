@@ -88,6 +88,7 @@ struct State {
     bool rows_kernel_min_set = false;  // JITNN_HIP_ROWS_MIN was given: no per-shape exceptions
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
+    bool rows_prepare_fused = true;   // JITNN_HIP_ROWS_PREPARE_FUSED=0: the SwiGLU in front of a one-pass ffn_down by a kernel of its own
     bool prefill_rope_join = true;    // JITNN_HIP_PREFILL_ROPE_JOIN=0: the K slices of q, k and v of a prefill step joined by a kernel of its own
     bool prefill_dual = true;         // JITNN_HIP_PREFILL_DUAL=0: gate and up of a prefill step as two products, SwiGLU by the next preparation
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
@@ -885,6 +886,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_DUAL")) g.prefill_dual = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ROPE_JOIN")) g.prefill_rope_join = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_ROWS_PREPARE_FUSED")) g.rows_prepare_fused = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
     g.ready = true;
@@ -1040,8 +1042,9 @@ bool rows_path(const jitnn_hip_weight *w, int rows) {
 
 // ys[i] = x ws[i]^T (+ bias) (+ residual [rows, n]; bias and residual with one weight only) for weights that all pass
 // rows_path: the activation operands are prepared once per granularity of block sums and shared by the weights.
+// swiglu_up: the activations are silu(x) * swiglu_up, formed by the preparation as it reads x.
 int launch_rows_group(const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows, const float *bias, const float *residual,
-                      hipStream_t s, ScratchSource src) {
+                      hipStream_t s, ScratchSource src, const float *swiglu_up = nullptr) {
     const int k = ws[0]->k;
     bool need[GR_LAYOUTS] = {};  // the operand layouts the weights ask for
     for (int i = 0; i < count; ++i) {
@@ -1056,11 +1059,9 @@ int launch_rows_group(const jitnn_hip_weight *const *ws, float *const *ys, int c
     for (int l = 0; l < GR_LAYOUTS; ++l) layouts += need[l];
     if (int rc = workspace(one * layouts, s, &scratch, src)) return rc;
     uint8_t *sc[GR_LAYOUTS] = {};
-    for (int l = 0, used = 0; l < GR_LAYOUTS; ++l) {
-        if (!need[l]) continue;
-        sc[l] = (uint8_t *)scratch + one * used++;
-        gemv_rows_prepare_launch(l, s, x, sc[l], k, rows);
-    }
+    for (int l = 0, used = 0; l < GR_LAYOUTS; ++l)
+        if (need[l]) sc[l] = (uint8_t *)scratch + one * used++;
+    gemv_rows_prepare_launch(s, x, swiglu_up, (void *const *)sc, k, rows);
     for (int i = 0; i < count; ++i)
         gemv_rows_main_launch(ws[i]->fmt, (unsigned)g.cus, s, ws[i]->dev, sc[gemv_rows_layout(ws[i]->fmt)], bias, residual, ys[i], ws[i]->n, k, rows);
     HIP_TRY(hipGetLastError());
@@ -1471,6 +1472,10 @@ int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, co
     if (many && (!up || (g.prefill_fuse_swiglu && prefill_prepare_fuses_norm(w->k)))) {
         return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp, up, SCRATCH_THREAD, g.prefill_defer_join ? part : nullptr,
                                     g.prefill_defer_join ? defer : nullptr);
+    }
+    if (up && g.rows_prepare_fused && rows_path(w, rows)) {  // silu(x) * up is formed by the preparation of the one-pass kernel
+        count_op(ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n));
+        return launch_rows_group(&w, &y, 1, x, rows, nullptr, res, st, SCRATCH_THREAD, up);
     }
     if (up) {
         const long long count = (long long)rows * w->k;

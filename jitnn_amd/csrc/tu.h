@@ -86,7 +86,9 @@ bool gemv_rows_supported(int fmt);
 int gemv_rows_layout(int fmt);                     // GR_LAYOUT_* of the format, -1: the kernel is not built for it
 size_t gemv_rows_scratch_bytes(int rows, int k);   // operands + scales of `rows` activation rows of k values
 KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blocks);  // the variant gemv_rows_main_launch picks for this shape
-void gemv_rows_prepare_launch(int layout, hipStream_t s, const float *x, void *scratch, int k, int rows);
+// every layout with a scratch (scratch[GR_LAYOUTS], nullptr: not wanted) in one launch; swiglu_up != nullptr: the rows are
+// silu(x) * swiglu_up, both [rows, k]
+void gemv_rows_prepare_launch(hipStream_t s, const float *x, const float *swiglu_up, void *const *scratch, int k, int rows);
 // y = x W^T (+ bias [n]) (+ res [rows, n])
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,
                            int n, int k, int rows);
