@@ -422,7 +422,8 @@ __host__ __device__ constexpr size_t gemv_rows_stage_bytes(int tiles_per_wave) {
 
 // y[b, row] = sum_k W[row, k] x[b, k] (+ bias[row]) (+ res[b, row]) for b < rows <= 8 * groups; k a multiple of 256, n >= 16.
 //   ops / inv: the output of rows_prepare_kernel<RTile<FMT>::SUMS> for the same x.  grid: up to one workgroup per batch of T tiles of 16
-//   weight rows (the host caps it at one per compute unit); GR_THREADS threads; gemv_rows_lds_bytes() of dynamic LDS.
+//   weight rows (the host caps it at one per compute unit) x shares of the groups of activation rows; GR_THREADS threads;
+//   gemv_rows_lds_bytes() + gemv_rows_stage_bytes() of dynamic LDS.
 // T = 2 halves the activation-operand traffic per weight byte; T = 1 is for matrices with too few tiles to give every CU a
 // workgroup otherwise.
 template <int FMT, int T>
@@ -440,6 +441,18 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
     uint8_t *stage = gr_smem + gemv_rows_lds_bytes(T) + gemv_rows_stage_bytes<FMT>(T) / GR_WAVES * wave;
     const int ncol = k >> 8, ntiles = (n + 15) >> 4, nbatch = (ntiles + T - 1) / T;
     const size_t rowbytes = (size_t)ncol * R::BYTES;
+    // gridDim.y > 1 (matrices with few tiles): workgroup y takes the groups [gper y, gper y + gper) of activation rows - it
+    // decodes the same weights as its neighbours and writes whole outputs of its own rows, nothing meets across workgroups
+    if (gridDim.y > 1) {
+        const int gper = (groups + (int)gridDim.y - 1) / (int)gridDim.y, g0 = (int)blockIdx.y * gper;
+        if (g0 >= groups) return;
+        ops += (size_t)g0 * ncol * GR_OP_HALVES;
+        inv += (size_t)g0 * ncol * 8;
+        y += (size_t)8 * g0 * n;
+        if (res) res += (size_t)8 * g0 * n;
+        rows -= 8 * g0;
+        groups = min(gper, groups - g0);
+    }
 
     for (int tb = blockIdx.x; tb < nbatch; tb += gridDim.x) {
         // this lane's row of each tile of the batch (the last tile of a ragged matrix is the last 16 rows: in bounds, its

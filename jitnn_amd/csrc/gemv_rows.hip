@@ -11,13 +11,21 @@ size_t gemv_rows_scratch_bytes(int rows, int k) {
     return gemv_rows_ops_bytes(groups, k) + gemv_rows_inv_bytes(groups, k);
 }
 
-// Two tiles per wave where that still gives every CU a workgroup, else one - but Q6_K with long rows (a wave then walks
-// many columns) and three groups of activation rows or more keeps two even if only every other CU gets a workgroup: its
-// sixteen operands per tile make the activation operands what the launch waits for, and two tiles share them (4096 x 14336
-// at 40 rows: 64.9 against 81.1 us; Q4_K on the same shape 47.0 against 41.5, Q8_0 58.5 against 46.0 - so not for those).
+static bool group_split = true;
+void gemv_rows_configure(bool split_groups) { group_split = split_groups; }
+
+// Two tiles per wave where that still gives every CU a workgroup - and, for many groups of activation rows, where it gives
+// every other CU one: two tiles share the activation operands, which are what the launch waits for, and the idle half of the
+// device takes a share of the groups (below).  4096 x 14336 at 40 rows, one tile against two: Q6_K 81.1 / 53.9 us, Q4_K 42.4 /
+// 35.7, Q5_K 44.3 / 40.6, Q4_1 42.4 / 38.1; 4096 x 4096 Q4_K 18.9 / 17.3 - at 24 rows they are level or the single tile ahead
+// (Q5_K 33.1 / 35.0), and Q4_0 and Q8_0 lose up to 40 rows (Q8_0 4096 x 4096 18.8 / 21.1) and gain little at 64: not for those.
+// Without the sharing of groups only Q6_K, with its sixteen operands per tile, gains from two tiles on half the CUs (64.9;
+// Q4_K 47.0, Q8_0 58.5 against 46.0).
 static int tiles_per_wave(int fmt, int n, int k, int rows, unsigned max_blocks) {
     const unsigned pairs = (unsigned)(((n + 15) / 16 + 1) / 2);
-    return pairs >= max_blocks || (fmt == F_Q6_K && rows > 16 && k >= 8192 && 2 * pairs >= max_blocks) ? 2 : 1;
+    bool half = fmt == F_Q6_K && rows > 16 && k >= 8192;
+    if (group_split && rows > 32 && k >= 4096 && (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K || fmt == F_Q4_1)) half = true;
+    return pairs >= max_blocks || (half && 2 * pairs >= max_blocks) ? 2 : 1;
 }
 
 template <int FMT>
@@ -80,8 +88,16 @@ static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const v
     const float *inv = reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(scratch) + gemv_rows_ops_bytes(groups, k));
     const int T = tiles_per_wave(FMT, n, k, rows, max_blocks), nbatch = ((n + 15) / 16 + T - 1) / T;
     const unsigned blocks = (unsigned)nbatch < max_blocks ? (unsigned)nbatch : max_blocks;
-    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, bias, res, y, n, k, rows, groups);
-    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, bias, res, y, n, k, rows, groups);
+    // Few tiles: the groups of activation rows are shared out over as many workgroups per tile as the device has room for -
+    // each decodes the tile's weights again (the device would idle otherwise) and writes whole outputs of its own rows.
+    // 1024 x 4096 at 40 rows: Q6_K 30.0 -> 19.4 us, Q4_K 17.5 -> 13.5; twice as many workgroups as CUs: 23.4, 13.9.
+    int gy = 1;
+    if (group_split && (unsigned)nbatch * 2 <= max_blocks) {
+        const int cap = (int)(max_blocks / (unsigned)nbatch), gper = (groups + cap - 1) / cap;
+        gy = (groups + gper - 1) / gper;
+    }
+    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, bias, res, y, n, k, rows, groups);
+    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, bias, res, y, n, k, rows, groups);
 }
 
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,

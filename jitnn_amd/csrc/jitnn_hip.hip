@@ -887,6 +887,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_PREFILL_DUAL")) g.prefill_dual = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ROPE_JOIN")) g.prefill_rope_join = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_ROWS_PREPARE_FUSED")) g.rows_prepare_fused = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_ROWS_GROUP_SPLIT")) gemv_rows_configure(atoi(e) != 0);
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
     g.ready = true;
