@@ -454,29 +454,39 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
         groups = min(gper, groups - g0);
     }
 
+    // this lane's row of each tile of a batch (the last tile of a ragged matrix is the last 16 rows: in bounds, its first
+    // rows computed twice, stored once)
+    typename R::Ptr sp[T];
+    typename R::Raw raw[T];
+    auto point = [&](int tb) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) sp[t] = R::ptr(W, min(min(tb * T + t, ntiles - 1) * 16, n - 16), rowbytes, lane);
+    };
+    auto fetch = [&](int col) {
+#pragma unroll
+        for (int t = 0; t < T; ++t) R::load(raw[t], sp[t], col);
+    };
+    // The bytes of a wave's next column are always on their way while it works on the current one - also across the end
+    // of a batch, under the reduction of its sums (128256 x 4096 Q6_K at 9 rows: 215 -> 202 us; a few per cent on matrices
+    // of two batches per workgroup).  Not for two tiles of Q6_K, whose 256 registers have no room for the second set of
+    // row pointers (4096 x 14336 at 40 rows: 55.1 against 53.3 us with the spills).
+    constexpr bool ACROSS = !(FMT == F_Q6_K && T == 2);
+    if (ACROSS && (int)blockIdx.x < nbatch && wave < ncol) {
+        point(blockIdx.x);
+        fetch(wave);
+    }
     for (int tb = blockIdx.x; tb < nbatch; tb += gridDim.x) {
-        // this lane's row of each tile of the batch (the last tile of a ragged matrix is the last 16 rows: in bounds, its
-        // first rows computed twice, stored once)
-        typename R::Ptr sp[T];
+        if (!ACROSS) {
+            point(tb);
+            if (wave < ncol) fetch(wave);
+        }
         bool live[T];
 #pragma unroll
-        for (int t = 0; t < T; ++t) {
-            const int tile = tb * T + t;
-            live[t] = tile < ntiles;  // workgroup-uniform
-            const int r0 = min((live[t] ? tile : ntiles - 1) * 16, n - 16);
-            sp[t] = R::ptr(W, r0, rowbytes, lane);
-        }
+        for (int t = 0; t < T; ++t) live[t] = tb * T + t < ntiles;  // workgroup-uniform
         for (int i = tid; i < T * groups * GR_THREADS; i += GR_THREADS) accl[i] = make_float2(0.f, 0.f);
         // (each thread only ever touches its own slots of accl until the final reduction: no barrier needed here)
 
-        typename R::Raw raw[T];
-        auto fetch = [&](int col) {
-#pragma unroll
-            for (int t = 0; t < T; ++t) R::load(raw[t], sp[t], col);
-        };
-        int c = wave;
-        if (c < ncol) fetch(c);
-        for (; c < ncol; c += GR_WAVES) {
+        for (int c = wave; c < ncol; c += GR_WAVES) {
             f16x8 B[T][NOPS], Bm[T];
             float d[T], dmin64[T];
             float dblk[R::BLOCK_SCALES ? T : 1][8];
@@ -490,7 +500,12 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
                     dmin64[t] = dm * 64.f;
                 }
             }
-            if (c + GR_WAVES < ncol) fetch(c + GR_WAVES);  // the next column's bytes are on their way while this one meets the activations
+            if (c + GR_WAVES < ncol) {
+                fetch(c + GR_WAVES);
+            } else if (ACROSS && tb + (int)gridDim.x < nbatch) {  // this batch's last column: the first of the next batch
+                point(tb + gridDim.x);
+                fetch(wave);
+            }
             for (int g = 0; g < groups; ++g) {
                 const _Float16 *op = ops + ((size_t)g * ncol + c) * GR_OP_HALVES + lane * 8;
                 f16x8 A[9];
