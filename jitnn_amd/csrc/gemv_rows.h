@@ -14,13 +14,14 @@
 //     eight sub-blocks of a super-block in one FP32 chain; only the super-block's d and dmin (and the activation scale)
 //     meet the sums in FP32, once per 16 x 256 tile instead of once per block.  The conversion costs what the plain one
 //     did: (1024 + q) * sc - 1024 * sc is one packed FMA on the pattern 0x6400 | q.  Q6_K's int8 scale times 6-bit quant
-//     is not an FP16 integer, but its two parts are (RTile<F_Q6_K>): two operands per 32-value step.
+//     is not an FP16 integer, but its two parts are (RTile<F_Q6_K>): two operands per 32-value step.  The 32-value formats
+//     have FP16 block scales, nothing folds: their operands are the quants, and each block's sum meets its d in FP32.
 // A workgroup of eight waves owns tiles of 16 weight rows; wave w walks the 256-value columns w, w + 8, ... of K for the
-// workgroup's tiles, T tiles at a time: every lane fetches the bytes of its own weight row straight from global memory
-// (the four 8-byte pieces of a row's 128 quant bytes share a cache line, so the line is used whole), turns them into
-// operands once, and runs them against every group of eight activation rows.  Partial sums live in LDS per lane (the
-// group index is a run-time value) and are added across the eight waves in wave order at the end of a tile batch: a
-// fixed summation order, no atomics.
+// workgroup's tiles, T tiles at a time: it fetches the tiles' bytes of a column sixteen bytes a lane, parts them through
+// a stage of its own in LDS (RStaged), turns them into operands once, and runs them against every group of eight
+// activation rows.  Partial sums live in LDS per lane (the group index is a run-time value) and are added across the
+// eight waves in wave order at the end of a tile batch: a fixed summation order, no atomics.  A launch with few tiles
+// puts several workgroups on a batch, each with a share of the groups (gridDim.y).
 #pragma once
 #include "common.h"
 #include "gemv_mfma.h"
