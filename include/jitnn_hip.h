@@ -86,7 +86,10 @@ JITNN_HIP_API long long jitnn_hip_weight_nbytes(int fmt, long long n, long long 
 
 /* Copies raw blocks from host memory to HBM unchanged.  Stands in for the upload of a persistent
  * block-quantised storage (Tensor.quantized / Tensor.persistent, core/Tensor.java:249-278; the bytes come
- * from GgufFile.tensor / raw, gguf/GgufFile.java:329-366).  nbytes must equal jitnn_hip_weight_nbytes. */
+ * from GgufFile.tensor / raw, gguf/GgufFile.java:329-366).  nbytes must equal jitnn_hip_weight_nbytes.
+ * Two formats without kernels of their own are rewritten on the way, block by block, into a format that holds exactly
+ * the same values - Q5_0 into Q8_0, Q3_K into Q6_K (every dequantised value keeps its bits) - and run on that format's
+ * kernels; jitnn_hip_weight_info still reports what was uploaded.  JITNN_HIP_TRANSCODE=0 keeps them as they are. */
 JITNN_HIP_API int jitnn_hip_weight_upload(int fmt, const void *blocks_host, long long nbytes, int n, int k, jitnn_hip_weight **out);
 
 /* Wraps blocks that are already in device memory (not copied, not owned: the caller keeps them alive).

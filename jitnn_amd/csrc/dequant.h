@@ -179,6 +179,49 @@ __global__ void __launch_bounds__(256) gemv_plain_kernel(const uint8_t *__restri
     }
 }
 
+// Two of the formats without kernels of their own hold exactly the values of a format that has them, block by block and
+// element by element, and are rewritten into it once, when the weight is uploaded:
+//   Q5_0 (q - 16) d, q of five bits (kernels/GgufKernels.java:147-153)  ->  Q8_0 with the same d and the int8 quant q - 16;
+//   Q3_K d (sc - 32) (q - 4 or q), sc of six bits per 16 values, q of two bits (kernels/GgufKernels.java:185-198)  ->  Q6_K
+//   with the same d, the int8 scale sc - 32 and the 6-bit quant q' + 32, q' = q - 4 or q: Q6_K's element order, its scale
+//   index 8 n + 2 k + l / 16 and its product d * sc * q (kernels/GgufKernels.java:126-138) are Q3_K's own.
+// The same floats multiply in the same order, so every value - and the dequantiser's output - keeps its bits.
+// One thread per block.
+static __global__ void __launch_bounds__(256) transcode_q5_0_to_q8_0_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, size_t blocks) {
+    for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < blocks; b += (size_t)gridDim.x * blockDim.x) {
+        const uint8_t *s = src + b * 22;
+        uint8_t *d = dst + b * 34;
+        d[0] = s[0];
+        d[1] = s[1];
+        const uint32_t qh = (uint32_t)s[2] | ((uint32_t)s[3] << 8) | ((uint32_t)s[4] << 16) | ((uint32_t)s[5] << 24);
+        for (int e = 0; e < 32; ++e) {
+            const int byte = s[6 + (e & 15)], q = (e < 16 ? byte & 15 : byte >> 4) + 16 * (int)((qh >> e) & 1u);
+            d[2 + e] = (uint8_t)(int8_t)(q - 16);
+        }
+    }
+}
+
+static __global__ void __launch_bounds__(256) transcode_q3_k_to_q6_k_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst, size_t blocks) {
+    for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < blocks; b += (size_t)gridDim.x * blockDim.x) {
+        const uint8_t *s = src + b * 110;  // hmask[32], qs[64], scales[12], d
+        uint8_t *d = dst + b * 210;        // ql[128], qh[64], scales[16], d
+        for (int i = 0; i < 192; ++i) d[i] = 0;
+        for (int e = 0; e < 256; ++e) {
+            const int n = e >> 7, j = (e & 127) >> 5, l = e & 31;
+            const int q = (s[32 + n * 32 + l] >> (2 * j)) & 3, high = (s[l] >> (4 * n + j)) & 1;
+            const int q6 = q - (high ? 0 : 4) + 32;  // 28 .. 35
+            d[64 * n + l + (j & 1) * 32] |= (uint8_t)((q6 & 15) << (j < 2 ? 0 : 4));
+            d[128 + 32 * n + l] |= (uint8_t)((q6 >> 4) << (2 * j));
+        }
+        for (int is = 0; is < 16; ++is) {  // the 6-bit scale `is`: low four bits from bytes 0..7, high two from bytes 8..11
+            const int low = is < 8 ? s[96 + is] & 15 : s[96 + is - 8] >> 4, hi2 = (s[96 + 8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+            d[192 + is] = (uint8_t)(int8_t)(low + 16 * hi2 - 32);
+        }
+        d[208] = s[108];
+        d[209] = s[109];
+    }
+}
+
 // FP32 -> Q8_0, one thread per block of 32 values, in the reference quantiser's arithmetic
 // (core/ops/Quant.java:102-118): amax in double, d = (float)(amax / 127.0) stored as binary16 (round to
 // nearest even), quants = round-half-away(x / (double)d) with the unrounded float d, clamped to +-127.

@@ -31,11 +31,13 @@
 using namespace jitnn;
 
 struct jitnn_hip_weight {
-    int fmt;
+    int fmt;  // of the blocks at dev: the caller's format, or the one an uploaded weight was rewritten into (below)
     int n, k;
     long long nbytes;
     uint8_t *dev;
     bool owned;
+    int file_fmt = 0;  // != 0: what the caller uploaded, when that was another format of exactly the same values
+    long long file_nbytes = 0;
 };
 
 // Scratch of the entry point that allocates nothing (jitnn_hip_linear_noalloc_dev): FP16 activations in operand order,
@@ -89,6 +91,7 @@ struct State {
     int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
     int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
     bool rows_prepare_fused = true;   // JITNN_HIP_ROWS_PREPARE_FUSED=0: the SwiGLU in front of a one-pass ffn_down by a kernel of its own
+    bool transcode = true;            // JITNN_HIP_TRANSCODE=0: uploaded Q5_0 / Q3_K blocks stay as they are (plain kernels)
     bool prefill_rope_join = true;    // JITNN_HIP_PREFILL_ROPE_JOIN=0: the K slices of q, k and v of a prefill step joined by a kernel of its own
     bool prefill_dual = true;         // JITNN_HIP_PREFILL_DUAL=0: gate and up of a prefill step as two products, SwiGLU by the next preparation
     bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
@@ -886,6 +889,7 @@ int jitnn_hip_init(int device_ordinal) {
     if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_DUAL")) g.prefill_dual = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_PREFILL_ROPE_JOIN")) g.prefill_rope_join = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_TRANSCODE")) g.transcode = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_ROWS_PREPARE_FUSED")) g.rows_prepare_fused = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_ROWS_GROUP_SPLIT")) gemv_rows_configure(atoi(e) != 0);
     if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
@@ -940,10 +944,40 @@ int jitnn_hip_weight_upload(int fmt, const void *blocks_host, long long nbytes, 
         (void)hipFree(dev);
         return fail(JITNN_HIP_EDEVICE, "hipMemcpy of %lld bytes: %s", nbytes, hipGetErrorString(e));
     }
-    jitnn_hip_weight *w = new (std::nothrow) jitnn_hip_weight{fmt, n, k, nbytes, dev, true};
+    // Q5_0 and Q3_K have no kernels of their own but hold exactly the values of Q8_0 / Q6_K blocks (dequant.h): rewritten
+    // once, here, they run on those formats' kernels with the same results, bit for bit where the dequantiser is concerned
+    int dev_fmt = fmt;
+    long long dev_nbytes = nbytes;
+    if (g.transcode && (fmt == F_Q5_0 || fmt == F_Q3_K)) {
+        dev_fmt = fmt == F_Q5_0 ? F_Q8_0 : F_Q6_K;
+        dev_nbytes = jitnn_hip_weight_nbytes(dev_fmt, n, k);
+        uint8_t *dev2 = nullptr;
+        e = hipMalloc(&dev2, (size_t)dev_nbytes);
+        if (e != hipSuccess) {
+            (void)hipFree(dev);
+            return fail(JITNN_HIP_ENOMEM, "hipMalloc of %lld bytes: %s", dev_nbytes, hipGetErrorString(e));
+        }
+        const size_t blocks = (size_t)n * k / block_values(fmt);
+        const unsigned grid = (unsigned)std::min<size_t>((blocks + 255) / 256, (size_t)g.cus * 16);
+        if (fmt == F_Q5_0) hipLaunchKernelGGL(transcode_q5_0_to_q8_0_kernel, dim3(grid), dim3(256), 0, nullptr, dev, dev2, blocks);
+        else hipLaunchKernelGGL(transcode_q3_k_to_q6_k_kernel, dim3(grid), dim3(256), 0, nullptr, dev, dev2, blocks);
+        e = hipGetLastError();
+        if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+        (void)hipFree(dev);
+        dev = dev2;
+        if (e != hipSuccess) {
+            (void)hipFree(dev);
+            return fail(JITNN_HIP_EDEVICE, "rewriting the blocks: %s", hipGetErrorString(e));
+        }
+    }
+    jitnn_hip_weight *w = new (std::nothrow) jitnn_hip_weight{dev_fmt, n, k, dev_nbytes, dev, true};
     if (!w) {
         (void)hipFree(dev);
         return fail(JITNN_HIP_ENOMEM, "out of host memory");
+    }
+    if (dev_fmt != fmt) {
+        w->file_fmt = fmt;
+        w->file_nbytes = nbytes;
     }
     *out = w;
     return JITNN_HIP_OK;
@@ -971,10 +1005,10 @@ int jitnn_hip_weight_free(jitnn_hip_weight *w) {
 
 int jitnn_hip_weight_info(const jitnn_hip_weight *w, int *fmt, int *n, int *k, long long *nbytes) {
     if (!w) return fail(JITNN_HIP_EINVAL, "weight is NULL");
-    if (fmt) *fmt = w->fmt;
+    if (fmt) *fmt = w->file_fmt ? w->file_fmt : w->fmt;  // (the caller's format and byte count, also where the device copy is another)
     if (n) *n = w->n;
     if (k) *k = w->k;
-    if (nbytes) *nbytes = w->nbytes;
+    if (nbytes) *nbytes = w->file_fmt ? w->file_nbytes : w->nbytes;
     return JITNN_HIP_OK;
 }
 
