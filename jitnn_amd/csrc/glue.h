@@ -140,30 +140,31 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
     }
 }
 
-// Merge of the key chunks of attn_decode_kernel: one workgroup per query head, two threads per value - one takes the
-// even chunks, one the odd ones, each with a running maximum over its chunks in order, then the two meet in LDS (a
-// fixed summation order).  A thread issues the loads of 16 chunks before it uses the first, so a context of up to
-// 1024 keys costs one round trip to memory.
+// Merge of the key chunks of attn_decode_kernel: one workgroup per query head, NP threads per value - thread p of a value
+// takes the chunks p, p + NP, ..., each with a running maximum over its chunks in order, then the NP partial results meet
+// in LDS and are combined in the order of p (a fixed summation order).  A thread issues the loads of 16 chunks before
+// it uses the first: NP = 2 covers a context of 1024 keys in one round trip to memory; long contexts take NP = 8 (a
+// context of 8192 keys: 256 chunks, two round trips instead of eight).
 // A separate launch on purpose: publishing the partial results to another workgroup inside one kernel needs
 // device-scope fences, which cost several times this kernel on a part with one L2 per XCD.
-template <int D>
+template <int D, int NP>
 __device__ __forceinline__ void attn_merge_body(const float *__restrict__ p, float *__restrict__ out, int chunks) {
     constexpr int U = 16;
-    __shared__ float sm[3][D];
-    const int d = threadIdx.x % D, half = threadIdx.x / D;
+    __shared__ float sm[NP - 1][3][D];
+    const int d = threadIdx.x % D, part = threadIdx.x / D;
     float m = -INFINITY, l = 0.f, acc = 0.f;
-    for (int c0 = half; c0 < chunks; c0 += 2 * U) {
+    for (int c0 = part; c0 < chunks; c0 += NP * U) {
         float mm[U], ll[U], aa[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const float *pc = p + (size_t)min(c0 + 2 * u, chunks - 1) * (D + 2);
+            const float *pc = p + (size_t)min(c0 + NP * u, chunks - 1) * (D + 2);
             mm[u] = pc[D];
             ll[u] = pc[D + 1];
             aa[u] = pc[d];
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            if (c0 + 2 * u < chunks) {
+            if (c0 + NP * u < chunks) {
                 const float mn = fmaxf(m, mm[u]);
                 const float a = __expf(m - mn), b = __expf(mm[u] - mn);
                 l = l * a + ll[u] * b;
@@ -172,28 +173,32 @@ __device__ __forceinline__ void attn_merge_body(const float *__restrict__ p, flo
             }
         }
     }
-    if (half == 1) {
-        sm[0][d] = m;
-        sm[1][d] = l;
-        sm[2][d] = acc;
+    if (part > 0) {
+        sm[part - 1][0][d] = m;
+        sm[part - 1][1][d] = l;
+        sm[part - 1][2][d] = acc;
     }
     __syncthreads();
-    if (half == 0) {
-        const float m1 = sm[0][d], l1 = sm[1][d], a1 = sm[2][d];
-        if (m1 > -INFINITY) {  // the odd half saw at least one chunk
-            const float mn = fmaxf(m, m1);
-            const float a = __expf(m - mn), b = __expf(m1 - mn);
-            l = l * a + l1 * b;
-            acc = acc * a + a1 * b;
+    if (part == 0) {
+#pragma unroll
+        for (int q = 0; q < NP - 1; ++q) {
+            const float m1 = sm[q][0][d], l1 = sm[q][1][d], a1 = sm[q][2][d];
+            if (m1 > -INFINITY) {  // that part saw at least one chunk
+                const float mn = fmaxf(m, m1);
+                const float a = __expf(m - mn), b = __expf(m1 - mn);
+                l = l * a + l1 * b;
+                acc = acc * a + a1 * b;
+                m = mn;
+            }
         }
         out[d] = acc / l;
     }
 }
 
-template <int D>
-__global__ void __launch_bounds__(2 * D) attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int chunks) {
+template <int D, int NP>
+__global__ void __launch_bounds__(NP * D) attn_merge_kernel(const float *__restrict__ part, float *__restrict__ out, int chunks) {
     const int h = blockIdx.x;
-    attn_merge_body<D>(part + (size_t)h * chunks * (D + 2), out + (size_t)h * D, chunks);
+    attn_merge_body<D, NP>(part + (size_t)h * chunks * (D + 2), out + (size_t)h * D, chunks);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -1398,7 +1398,9 @@ void launch_attention(const jitnn_hip_llama *m, int layer, int pos, hipStream_t 
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
     hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->k, m->v, m->kc + lo, m->vc + lo, m->cosv, m->sinv,
                        m->part, m->heads, m->kv, pos, 1.0f / sqrtf((float)D), m->rope_interleaved);
-    hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(m->heads), dim3(2 * D), 0, st, m->part, m->att, chunks);
+    constexpr int NPL = 1024 / D < 8 ? 1024 / D : 8;  // long contexts: more threads per value share the chunks
+    if (chunks > 32) hipLaunchKernelGGL((attn_merge_kernel<D, NPL>), dim3(m->heads), dim3(NPL * D), 0, st, m->part, m->att, chunks);
+    else hipLaunchKernelGGL((attn_merge_kernel<D, 2>), dim3(m->heads), dim3(2 * D), 0, st, m->part, m->att, chunks);
 }
 
 bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !g.force_lds && !is_extra_format(w->fmt); }

@@ -93,6 +93,27 @@ def test_decode_8b_shaped_layer(jn):
     dec.close()
 
 
+@pytest.mark.parametrize("heads,kv_heads,head_dim,ctx", [(4, 2, 64, 1500), (4, 1, 128, 2077), (2, 2, 192, 700), (2, 1, 256, 1111)])
+def test_decode_long_context(jn, heads, kv_heads, head_dim, ctx):
+    """One token over a long cache: more than 32 key chunks per head, so the merge of the chunks runs with eight (five,
+    four) threads per value instead of two; the last chunk is partly filled."""
+    cfg = dict(layers=1, d_model=256, heads=heads, kv_heads=kv_heads, head_dim=head_dim, ffn=256, vocab=100, max_ctx=ctx + 2, rms_eps=1e-5,
+               rope_theta=5e5)
+    dec, layers, out_norm, out_w = build(jn, cfg, 31, {s: "Q8_0" for s in SLOTS}, "Q8_0")
+    rng = np.random.default_rng(7)
+    kc = np.zeros((1, cfg["max_ctx"], kv_heads, head_dim), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :ctx] = rng.standard_normal(kc[:, :ctx].shape)
+    vc[:, :ctx] = rng.standard_normal(vc[:, :ctx].shape)
+    dec.kv_write(0, 0, kc[0, :ctx], vc[0, :ctx])
+    for step in range(2):
+        x = rng.standard_normal(cfg["d_model"]).astype(np.float32)
+        ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x, ctx + step)
+        y = dec.decode(x, ctx + step)
+        assert norm_err(y, ref) <= 1e-4, (head_dim, step, norm_err(y, ref))
+    dec.close()
+
+
 def test_decode_argument_checks(jn):
     cfg = dict(layers=1, d_model=256, heads=4, kv_heads=2, head_dim=64, ffn=512, vocab=64, max_ctx=8, rms_eps=1e-5, rope_theta=1e4)
     dec = jn.LlamaDecoder(**cfg)
