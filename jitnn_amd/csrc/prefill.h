@@ -24,6 +24,7 @@ namespace jitnn {
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int PF_BN = 128, PF_BM = 256, PF_BK = 64, PF_LD = PF_BK + 8;  // LDS row pitch in halves: 144 bytes, conflict-free 16-byte reads
+constexpr int PF_NARROW_ROWS = 128;  // calls of at most this many rows: two 32-row blocks per wave instead of four (prefill_mfma_body, RT)
 
 // position of value i (0..3) of a group of four in the FP16 operands: 0, 2, 1, 3
 __host__ __device__ constexpr int pf_perm4(int i) { return ((i & 1) << 1) | (i >> 1); }
@@ -499,7 +500,10 @@ __device__ __forceinline__ void pf_load_lds(PfRaw<FMT> &r, const uint8_t *b, int
 // its first two 32-row blocks and the same rows of W2 [n, k] in the other two, so that a lane holds the gate and the up
 // product of one output in the same element of two accumulators, and y [m, n] = silu(x W^T) * (x W2^T) - the two products
 // never go to memory.  No K slices, no bias.
-template <int FMT, bool DUAL = false>
+// RT = 4: wave w owns all four 32-row blocks of the tile x tokens [64 w, +64).  RT = 2, for calls of at most 128 rows (the
+// token slices of waves 2 and 3 would be empty, half the matrix cores would multiply zeros): wave w owns the row blocks
+// w % 2 and w % 2 + 2 - a gate and its up block when DUAL - x tokens [64 (w / 2), +64): half the products per wave and step.
+template <int FMT, bool DUAL = false, int RT = 4>
 __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W, const _Float16 *__restrict__ xo, const float *__restrict__ inv_scale,
                                                   const float *__restrict__ bias, float *__restrict__ y, const int m, const int n, const int k,
                                                   const int split_steps, const int tile, const int slice, const uint8_t *__restrict__ W2 = nullptr) {
@@ -519,10 +523,12 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
     const int ksteps = pf_ksteps(k);
     // B operands of token blocks m0/32 + 2 w + {0, 1}: 16 bytes per lane, consecutive K steps 1 KiB apart (the operand
     // array is padded to whole tiles of PF_BM tokens, so both blocks exist)
-    const f16x8 *xb = reinterpret_cast<const f16x8 *>(xo) + ((size_t)(m0 / 32 + 2 * wave) * ksteps) * 64 + lane;
-    f32x16 acc[4][2];
+    const int tslice = RT == 4 ? wave : wave >> 1;                    // this wave's 64 tokens of the tile
+    auto rblock = [&](int i) { return RT == 4 ? i : (wave & 1) + 2 * i; };  // the 32-row block of acc[i]
+    const f16x8 *xb = reinterpret_cast<const f16x8 *>(xo) + ((size_t)(m0 / 32 + 2 * tslice) * ksteps) * 64 + lane;
+    f32x16 acc[RT][2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -623,17 +629,17 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
         // of a substep are read from LDS while the MFMAs of the one before run (one wave per SIMD: nobody else hides
         // the LDS latency).
         const _Float16 *ap = &As[buf][(lane & 31) * PF_LD + 8 * (lane >> 5)];
-        f16x8 a[2][4];
+        f16x8 a[2][RT];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a[0][i] = *reinterpret_cast<const f16x8 *>(ap + 32 * i * PF_LD);
+        for (int i = 0; i < RT; ++i) a[0][i] = *reinterpret_cast<const f16x8 *>(ap + 32 * rblock(i) * PF_LD);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             if (ks < 3) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) a[(ks + 1) & 1][i] = *reinterpret_cast<const f16x8 *>(ap + 32 * i * PF_LD + 16 * (ks + 1));
+                for (int i = 0; i < RT; ++i) a[(ks + 1) & 1][i] = *reinterpret_cast<const f16x8 *>(ap + 32 * rblock(i) * PF_LD + 16 * (ks + 1));
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < RT; ++i)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bcur[j][ks], a[ks & 1][i], acc[i][j], 0, 0, 0);
         }
@@ -644,13 +650,13 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
         // time also one LDS operand read and one of the step's global loads.  The loads are spread over the step on
         // purpose: issued in one burst after the barrier, the four waves' requests queue up at the CU's one
         // address unit and the waves stall at the issue while the matrix pipe idles.
-        __builtin_amdgcn_sched_group_barrier(0x100, 4 + Stage::NRAW, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, RT + Stage::NRAW, 0);
 #pragma unroll
-        for (int i = 0; i < 32; ++i) {
+        for (int i = 0; i < 8 * RT; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-            if (i % 2 == 0 && i < 24) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, RT == 4 ? 4 : 8, 0);  // (the decode of a step is as long whatever RT is)
+            if (i % 2 == 0 && i < 6 * RT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (RT == 2 || i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
     };
     if constexpr (STAGED) {
@@ -682,7 +688,7 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
     // half wave store 32 consecutive floats of one token's output row.  The 32 token scales of the lane are read
     // first, in one batch (index clamped, so the loads are unconditional): a load between the stores would make
     // every store wait for the one before it, stores and loads being counted by the same counter.
-    const int tok0 = m0 + 64 * wave + 4 * (lane >> 5);
+    const int tok0 = m0 + 64 * tslice + 4 * (lane >> 5);
     float isc[2][16];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
@@ -693,31 +699,31 @@ __device__ __forceinline__ void prefill_mfma_body(const uint8_t *__restrict__ W,
         // stored products: XP_SWIGLU)
         auto sw = [](float g, float u) { return (g / (1.f + __expf(-g))) * u; };
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int row = n0 + 32 * i + (lane & 31);
+        for (int i = 0; i < RT / 2; ++i) {  // accumulators i (gate) and i + RT / 2 (up): row blocks rblock(i) and rblock(i) + 2
+            const int row = n0 + 32 * rblock(i) + (lane & 31);
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int tok = tok0 + 32 * j + 8 * (r >> 2) + (r & 3);
-                    if (row < n && tok < m) y[(size_t)tok * n + row] = sw(acc[i][j][r] * isc[j][r], acc[i + 2][j][r] * isc[j][r]);
+                    if (row < n && tok < m) y[(size_t)tok * n + row] = sw(acc[i][j][r] * isc[j][r], acc[i + RT / 2][j][r] * isc[j][r]);
                 }
             }
         }
         return;
     }
-    float bv[4];
+    float bv[RT];
     {
         const float *bp = bias ? bias : inv_scale;  // some readable address when there is no bias: the value is dropped
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float b = bp[bias ? min(n0 + 32 * i + (lane & 31), n - 1) : 0];
+        for (int i = 0; i < RT; ++i) {
+            const float b = bp[bias ? min(n0 + 32 * rblock(i) + (lane & 31), n - 1) : 0];
             bv[i] = bias ? b : 0.f;
         }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = n0 + 32 * i + (lane & 31);
+    for (int i = 0; i < RT; ++i) {
+        const int row = n0 + 32 * rblock(i) + (lane & 31);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -755,7 +761,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                                                             int m, int k) {
     int seg, tile, slice;
     pf_locate(sg, seg, tile, slice);
-    prefill_mfma_body<FMT>(sg.W[seg], xo, inv_scale, bias, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+    if (m <= PF_NARROW_ROWS) prefill_mfma_body<FMT, false, 2>(sg.W[seg], xo, inv_scale, bias, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+    else prefill_mfma_body<FMT>(sg.W[seg], xo, inv_scale, bias, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
 }
 
 // The same for weights of two formats (a Q4_K_M layer keeps q and k as Q4_K and v as Q6_K): segments below first_b are
@@ -766,8 +773,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                                                             int m, int k) {
     int seg, tile, slice;
     pf_locate(sg, seg, tile, slice);
-    if (seg < first_b) prefill_mfma_body<FA>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
-    else prefill_mfma_body<FB>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+    if (m <= PF_NARROW_ROWS) {
+        if (seg < first_b) prefill_mfma_body<FA, false, 2>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+        else prefill_mfma_body<FB, false, 2>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+    } else if (seg < first_b) {
+        prefill_mfma_body<FA>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+    } else {
+        prefill_mfma_body<FB>(sg.W[seg], xo, inv_scale, nullptr, sg.y[seg], m, sg.n[seg], k, sg.split_steps[seg], tile, slice);
+    }
 }
 
 // y [m, n] = silu(x W^T) * (x W2^T) for two weights [n, k] of one format: grid (ceil(n / 64), token tiles).
@@ -777,7 +790,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))
                                                                                                             const _Float16 *__restrict__ xo,
                                                                                                             const float *__restrict__ inv_scale,
                                                                                                             float *__restrict__ y, int m, int n, int k) {
-    prefill_mfma_body<FMT, true>(W, xo, inv_scale, nullptr, y, m, n, k, (k + PF_BK - 1) / PF_BK, blockIdx.x, 0, W2);
+    if (m <= PF_NARROW_ROWS) prefill_mfma_body<FMT, true, 2>(W, xo, inv_scale, nullptr, y, m, n, k, (k + PF_BK - 1) / PF_BK, blockIdx.x, 0, W2);
+    else prefill_mfma_body<FMT, true>(W, xo, inv_scale, nullptr, y, m, n, k, (k + PF_BK - 1) / PF_BK, blockIdx.x, 0, W2);
 }
 
 // y[tok, row] = sum over the K slices of part[z][tok, row] (+ bias[row]) (+ res[tok, row]), slices in order: the second half of a
