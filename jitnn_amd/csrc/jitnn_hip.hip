@@ -273,10 +273,14 @@ int launch_xreg(const XregCall &c, hipStream_t stream) {
     // Two workgroups (eight waves) per CU measured best for streaming: fewer, longer row streams keep HBM pages
     // open.  A wave that sees many rows needs one row of prefetch; when it sees only a handful (a 14336-row
     // matrix gives a wave seven rows) a second row in flight covers the start-up latency.
-    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : 2);
+    // Matrices of few rows (a wave sees two to four of them: attn_o, a 4096 x 4096 weight) do better with three
+    // workgroups per CU and one row of prefetch: Q8_0 4096 x 4096 6.9 -> 6.5 us, attn_o of the 8B step 5.34 -> 5.25; from
+    // 11008 rows on the two-workgroup shape is level or ahead (Q4_0 11008 x 4096 7.56 against 7.78 us).
+    const bool few = n <= 8192 && !c.w2;
+    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : few ? 3 : 2);
     if (blocks > cap) blocks = cap;
     const int rows_per_wave = (n + blocks * waves - 1) / (blocks * waves);
-    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
+    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (few || rows_per_wave >= 16 ? 1 : 2);
     a.rpw = g.xreg_priority ? rows_per_wave : 0;
     const int mode = c.w2 ? 3 : c.norm_w ? 2 : c.bias ? 1 : 0;
     xreg_fn fn = pick_xreg(c.w[0]->fmt, a.k % 64 == 0, mode, pf);
@@ -322,7 +326,8 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
     if (blocks_a > (na + waves - 1) / waves) blocks_a = (na + waves - 1) / waves;
     if (blocks_b > (nb + waves - 1) / waves) blocks_b = (nb + waves - 1) / waves;
     const int rpw_a = (na + blocks_a * waves - 1) / (blocks_a * waves), rpw_b = (nb + blocks_b * waves - 1) / (blocks_b * waves);
-    const int pf = g.xreg_pf > 0 ? g.xreg_pf : ((rpw_a > rpw_b ? rpw_a : rpw_b) >= 16 ? 1 : 2);
+    // (one row of prefetch: the q, k | v launch of an 8B layer - 6144 rows, three per wave - 8.1 -> 7.7 us against two)
+    const int pf = g.xreg_pf > 0 ? g.xreg_pf : 1;
     a.rpw = g.xreg_priority ? rpw_a : 0;
     b.rpw = g.xreg_priority ? rpw_b : 0;
     xreg2_fn fn = pf == 1 ? pick_xreg2_pf<1>(ca.w[0]->fmt, cb.w[0]->fmt) : pick_xreg2_pf<2>(ca.w[0]->fmt, cb.w[0]->fmt);
@@ -366,10 +371,14 @@ int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *b
     if (per_cu < 1) per_cu = 1;
     const int waves_cap = 16 / slices > 0 ? 16 / slices : 1;  // at most 16 waves (4 per SIMD: the kernels use ~128 VGPRs)
     if (per_cu > waves_cap) per_cu = waves_cap;
+    // One row of prefetch, and for matrices of few rows at most three workgroups per CU: the ffn_down of an 8B layer (Q6_K
+    // 4096 x 14336, four waves per workgroup) 14.6 -> 14.2 us against four workgroups with two rows in flight each, Q5_K
+    // 14.0 -> 13.0, Q4_K 4096 x 8192 8.45 -> 8.2; with many rows per workgroup more of them are better (Q4_K 14336 x 8192
+    // 15.4 against 16.8 us with three).
+    if (w->n <= 8192 && per_cu > 3) per_cu = 3;
     if (g.xreg_blocks_per_cu > 0 && per_cu > g.xreg_blocks_per_cu) per_cu = g.xreg_blocks_per_cu;
     int blocks = w->n < g.cus * per_cu ? w->n : g.cus * per_cu;
-    const int rows_per_block = (w->n + blocks - 1) / blocks;
-    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_block >= 16 ? 1 : 2);
+    const int pf = g.xreg_pf > 0 ? g.xreg_pf : 1;
     gemv1_fn fn = pf == 1 ? pick_ksplit_pf<1>(w->fmt, w->k % 64 == 0) : pick_ksplit_pf<2>(w->fmt, w->k % 64 == 0);
     if (int rc = allow_lds((const void *)fn, lds)) return rc;
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(64 * slices), lds, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
