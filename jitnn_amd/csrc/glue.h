@@ -3,6 +3,7 @@
 // bandwidth story of the step (the weights are) and are written plainly in FP32; each follows the reference
 // operator it stands for (paths below are under jitnn-core/src/main/java/ai/beestream/jitnn/).
 #pragma once
+#include <type_traits>
 #include "common.h"
 
 namespace jitnn {
@@ -259,47 +260,56 @@ __global__ void __launch_bounds__(256) rope_append_rows_join_kernel(const float 
                                                                      float *__restrict__ kcache, float *__restrict__ vcache,
                                                                      const float *__restrict__ cosv, const float *__restrict__ sinv, int heads,
                                                                      int kv_heads, int D, int pos0, int interleaved) {
-    constexpr int ZMAX = 8;  // most K slices of a many-row launch
     const int t = blockIdx.x, pos = pos0 + t, half = D / 2;
     const int nq = heads * D, nk = kv_heads * D;
     const size_t zq = (size_t)T * nq, zk = (size_t)T * nk;  // floats per slice
     const float *pq = part + (size_t)t * nq, *pk = part + zq * s0 + (size_t)t * nk, *pv = part + zq * s0 + zk * s1 + (size_t)t * nk;
     const float *cp = cosv + (size_t)pos * half, *sp = sinv + (size_t)pos * half;
-    // four values at a time, every slice's load issued before the first sum (slices past the last repeat it and are not
-    // added): the sum runs in slice order
-    auto joined = [&](const float *p, size_t zs, int splits, int i) {
-        float4 v[ZMAX];
+    // four values at a time, the loads of all Z >= splits slices issued before the first sum (slices past the last repeat
+    // it and are not added; Z is the power of two at or above the launch's slices, at most the eight a many-row launch
+    // makes): the sum runs in slice order
+    auto joined = [&](auto zc, const float *p, size_t zs, int splits, int i) {
+        constexpr int Z = decltype(zc)::value;
+        float4 v[Z];
 #pragma unroll
-        for (int z = 0; z < ZMAX; ++z) v[z] = *reinterpret_cast<const float4 *>(p + (size_t)min(z, splits - 1) * zs + i);
+        for (int z = 0; z < Z; ++z) v[z] = *reinterpret_cast<const float4 *>(p + (size_t)min(z, splits - 1) * zs + i);
         float4 a = v[0];
 #pragma unroll
-        for (int z = 1; z < ZMAX; ++z)
+        for (int z = 1; z < Z; ++z)
             if (z < splits) a = make_float4(a.x + v[z].x, a.y + v[z].y, a.z + v[z].z, a.w + v[z].w);
         return a;
     };
     // a rotation item: four angles p .. p + 3 of one head - values (p .. p + 3, p + half .. p + half + 3), or 2 p .. 2 p + 7 in pairs
-    auto rotate = [&](const float *src, size_t zs, int splits, float *dst, int nheads) {
+    auto rotate = [&](auto zc, const float *src, size_t zs, int splits, float *dst, int nheads) {
         for (int i = threadIdx.x; i < nheads * (half / 4); i += 256) {
             const int h = i / (half / 4), p = 4 * (i - h * (half / 4));
             const float4 cs = *reinterpret_cast<const float4 *>(cp + p), sn = *reinterpret_cast<const float4 *>(sp + p);
             if (interleaved) {
                 const int i0 = h * D + 2 * p;
-                const float4 u = joined(src, zs, splits, i0), w = joined(src, zs, splits, i0 + 4);
+                const float4 u = joined(zc, src, zs, splits, i0), w = joined(zc, src, zs, splits, i0 + 4);
                 *reinterpret_cast<float4 *>(dst + i0) = make_float4(u.x * cs.x - u.y * sn.x, u.x * sn.x + u.y * cs.x, u.z * cs.y - u.w * sn.y, u.z * sn.y + u.w * cs.y);
                 *reinterpret_cast<float4 *>(dst + i0 + 4) =
                     make_float4(w.x * cs.z - w.y * sn.z, w.x * sn.z + w.y * cs.z, w.z * cs.w - w.w * sn.w, w.z * sn.w + w.w * cs.w);
             } else {
                 const int i0 = h * D + p, i1 = i0 + half;
-                const float4 a = joined(src, zs, splits, i0), b = joined(src, zs, splits, i1);
+                const float4 a = joined(zc, src, zs, splits, i0), b = joined(zc, src, zs, splits, i1);
                 *reinterpret_cast<float4 *>(dst + i0) = make_float4(a.x * cs.x - b.x * sn.x, a.y * cs.y - b.y * sn.y, a.z * cs.z - b.z * sn.z, a.w * cs.w - b.w * sn.w);
                 *reinterpret_cast<float4 *>(dst + i1) = make_float4(a.x * sn.x + b.x * cs.x, a.y * sn.y + b.y * cs.y, a.z * sn.z + b.z * cs.z, a.w * sn.w + b.w * cs.w);
             }
         }
     };
-    rotate(pq, zq, s0, q + (size_t)t * nq, heads);
-    rotate(pk, zk, s1, kcache + (size_t)pos * nk, kv_heads);
+    auto with_slices = [&](int splits, auto &&f) {  // f(the power of two at or above splits, as a type)
+        if (splits <= 1) f(std::integral_constant<int, 1>{});
+        else if (splits <= 2) f(std::integral_constant<int, 2>{});
+        else if (splits <= 4) f(std::integral_constant<int, 4>{});
+        else f(std::integral_constant<int, 8>{});
+    };
+    with_slices(s0, [&](auto zc) { rotate(zc, pq, zq, s0, q + (size_t)t * nq, heads); });
+    with_slices(s1, [&](auto zc) { rotate(zc, pk, zk, s1, kcache + (size_t)pos * nk, kv_heads); });
     float *vc = vcache + (size_t)pos * nk;
-    for (int i = 4 * threadIdx.x; i < nk; i += 1024) *reinterpret_cast<float4 *>(vc + i) = joined(pv, zk, s2, i);
+    with_slices(s2, [&](auto zc) {
+        for (int i = 4 * threadIdx.x; i < nk; i += 1024) *reinterpret_cast<float4 *>(vc + i) = joined(zc, pv, zk, s2, i);
+    });
 }
 
 // Causal attention of a block of consecutive tokens: the (token, query head) pairs of one key/value head - ATT_ROWS
