@@ -12,4 +12,4 @@ from .llama import LlamaDecoder  # noqa: F401
 from .gguf_file import GgufFile, GgufTensorInfo  # noqa: F401
 from ._lib import UnsupportedTypeError  # noqa: F401
 from .tokenizer import Tokenizer  # noqa: F401
-from .llm import Llm, ModelInfo  # noqa: F401
+from .llm import GenerationRequest, GenerationResult, Llm, ModelInfo  # noqa: F401

@@ -87,6 +87,56 @@ def test_bpe_tokenizer_round_trip():
     assert tk.decode([len(toks) - 1]) == ""          # control tokens print nothing
 
 
+def test_sample_token_limits_and_distribution():
+    """The sampler of generate(request): its limits are the greedy choice, its draws follow the renormalised softmax of the
+    candidates that top_k and top_p leave, and a seed fixes them."""
+    from jitnn_amd.llm import sample_token
+    rng = np.random.default_rng(0)
+    logits = rng.standard_normal(50).astype(np.float32) * 2
+    logits[[7, 31]] = logits.max() + 1.0  # two equal maxima: the lower index
+    logits[3] = np.nan
+    for kw in (dict(temperature=0.0, top_k=0, top_p=1.0), dict(temperature=1.0, top_k=1, top_p=1.0), dict(temperature=1e-4, top_k=0, top_p=1.0)):
+        picks = {sample_token(logits, rng=np.random.default_rng(s), **kw) for s in range(20)}
+        assert picks <= {7, 31}
+    assert sample_token(logits, 0.0, 0, 1.0, rng) == 7 and sample_token(logits, 1.0, 1, 1.0, rng) == 7
+    assert sample_token(logits, 1.0, 0, 1e-9, np.random.default_rng(1)) == 7  # a nucleus of one token
+    # frequencies over many draws against the closed form, with and without the limits
+    clean = np.where(np.isnan(logits), -np.inf, logits).astype(np.float64)
+    for temperature, top_k, top_p in ((1.0, 0, 1.0), (0.7, 5, 1.0), (1.5, 0, 0.6), (1.0, 8, 0.9)):
+        order = np.argsort(-clean, kind="stable")
+        if top_k:
+            order = order[:top_k]
+        p = np.exp((clean[order] - clean[order[0]]) / temperature)
+        p /= p.sum()
+        if top_p < 1.0:
+            keep = int(np.argmax(np.cumsum(p) >= top_p)) + 1
+            order, p = order[:keep], p[:keep] / p[:keep].sum()
+        want = np.zeros(50)
+        want[order] = p
+        g = np.random.default_rng(11)
+        n = 40000
+        got = np.bincount([sample_token(logits, temperature, top_k, top_p, g) for _ in range(n)], minlength=50) / n
+        assert got[want == 0].sum() == 0 and np.abs(got - want).max() < 4 * np.sqrt(0.25 / n), (temperature, top_k, top_p)
+    a = [sample_token(logits, 1.0, 0, 1.0, np.random.default_rng(5)) for _ in range(3)]
+    assert len(set(a)) == 1  # same seed, same draw
+
+
+def test_stop_filter_holds_back_what_may_become_a_stop_sequence():
+    from jitnn_amd.llm import GenerationRequest, StopFilter
+    f = StopFilter(["END", "\n\n"])
+    out = [f.push(p) for p in ["abc E", "N", "x \n", "y EN", "D tail", "more"]]
+    assert out == [("abc ", False), ("", False), ("ENx ", False), ("\ny ", False), ("", True), ("", True)]
+    assert f.flush() == "" and f.stopped
+    f = StopFilter(["END"])
+    assert f.push("so it E") == ("so it ", False) and f.flush() == "E"  # what was held back comes out at the end
+    f = StopFilter([])
+    assert f.push("anything") == ("anything", False)
+    assert GenerationRequest("p", stop="x").stop == ("x",) and GenerationRequest("p", stop=["a", ""]).stop == ("a",)
+    for bad in (dict(max_new_tokens=-1), dict(temperature=-0.1), dict(top_p=0.0), dict(top_p=1.5), dict(top_k=-2)):
+        with pytest.raises(ValueError):
+            GenerationRequest("p", **bad)
+
+
 # ------------------------------------------------------------------------------------------------ on the GPU
 
 CFG = dict(layers=2, d_model=256, heads=4, kv_heads=2, head_dim=64, ffn=512, max_ctx=64, rms_eps=1e-5, rope_theta=10000.0)
@@ -196,6 +246,39 @@ def test_generate_from_a_gguf_file(tmp_path, arch, embd_fmt, tied):
         # stops at the end-of-sequence token: make it the most likely continuation by asking for it as the eos id
         first = out[0]
         assert llm.model().generate(ids, 5, eos_token=first) == []
+
+
+@pytest.mark.gpu
+def test_generate_request_sampling_and_stop(tmp_path):
+    """generate(request) (Llm.java:84-93): temperature 0 is the greedy loop of the library token for token; a seed fixes a
+    sampled continuation; a stop sequence ends the text in front of itself; the length limit and the end-of-sequence token
+    are told apart; the streamed pieces add up to the text."""
+    import jitnn_amd
+    from jitnn_amd import GenerationRequest
+    path = tmp_path / "tiny.gguf"
+    write_model(path, "llama", 7)
+    with jitnn_amd.Llm.load(path) as llm:
+        prompt = "the cat sat on the"
+        ids = llm.tokenizer().encode(prompt)
+        greedy_ids, greedy = llm.generate_tokens(ids, 12), llm.generate(prompt, 12)
+        streamed = []
+        r = llm.generate(GenerationRequest(prompt, 12, on_token=streamed.append))
+        assert r.tokens == greedy_ids and r.text == greedy == "".join(streamed) and r.prompt_tokens == len(ids)
+        assert r.finish_reason == ("length" if len(greedy_ids) == 12 else "eos")
+        a = llm.generate(GenerationRequest(prompt, 16, temperature=0.9, top_k=40, top_p=0.95, seed=3))
+        b = llm.generate(GenerationRequest(prompt, 16, temperature=0.9, top_k=40, top_p=0.95, seed=3))
+        others = [llm.generate(GenerationRequest(prompt, 16, temperature=0.9, seed=s)).tokens for s in range(4, 10)]
+        assert a.tokens == b.tokens and a.text == b.text and any(t != a.tokens for t in others)
+        assert llm.generate(GenerationRequest(prompt, 16, temperature=5.0, top_k=1, seed=1)).tokens == llm.generate_tokens(ids, 16)
+        # a stop sequence taken from the middle of the greedy text: the text ends in front of it
+        if len(greedy) >= 6:
+            stop = greedy[len(greedy) // 2:len(greedy) // 2 + 3]
+            streamed = []
+            s = llm.generate(GenerationRequest(prompt, 12, stop=[stop], on_token=streamed.append))
+            assert s.finish_reason == "stop" and s.text == greedy[:greedy.find(stop)] == "".join(streamed)
+        assert llm.generate(GenerationRequest(prompt, 0)).tokens == []
+        with pytest.raises(ValueError):
+            llm.generate(GenerationRequest(prompt, 10 ** 6))
 
 
 @pytest.mark.gpu
