@@ -496,6 +496,75 @@ def bench_prefill(torch, lib, steps=20, with_cpu=True):
     return res
 
 
+def bench_codec(torch, lib, with_cpu):
+    """The dequantiser and the Q8_0 quantiser (ops gguf_dequantize, dequantize_q8_0, quantize_q8_0) on whole weights: HIP-event
+    time per call, algorithmic bytes (blocks + 4 bytes per value, read or written), bit-exactness against the oracle on the
+    first rows, and the oracle's own one-thread time for the whole call (what the reference's host loop does)."""
+    import numpy as np
+    from oracle import oracle
+    out = {}
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def timed(fn, steps=50, warmup=5):
+        for _ in range(warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / steps
+
+    for name, fmt, n, k, seed in (("dequantize_q4_k_14336x4096", "Q4_K", 14336, 4096, 1030), ("dequantize_q6_k_4096x14336", "Q6_K", 4096, 14336, 1045),
+                                  ("dequantize_q8_0_4096x4096", "Q8_0", 4096, 4096, 1010)):
+        fid, qk, nb = BLOCK[fmt]
+        t = quantized_device_weight(torch, lib, fmt, n, k, seed)
+        h = C.c_void_p()
+        lib.check(lib.lib.jitnn_hip_weight_wrap_dev(fid, C.c_void_p(t.data_ptr()), t.numel(), n, k, C.byref(h)), "wrap")
+        y = torch.empty(n * k, dtype=torch.float32, device="cuda")
+        yp = C.c_void_p(y.data_ptr())
+        sec = timed(lambda: lib.check(lib.lib.jitnn_hip_dequantize_dev(h, yp, stream), "dequantize"))
+        nbytes = t.numel() + 4 * n * k
+        rows = min(n, 64)
+        raw = t[:rows * (k // qk) * nb].cpu().numpy()
+        e = {"workload": f"{fmt} [{n}, {k}] blocks -> FP32", "us": sec * 1e6, "bytes_per_call": nbytes, "GBps": nbytes / sec / 1e9,
+             "pct_of_peak": nbytes / sec / 1e9 / PEAK_HBM_GBPS * 100,
+             "bit_exact_first_rows": bool(np.array_equal(y[:rows * k].cpu().numpy().view(np.uint32), oracle.dequantize(fid, raw, rows * k).view(np.uint32)))}
+        if with_cpu:
+            sample = min(n, 2048)
+            rs = t[:sample * (k // qk) * nb].cpu().numpy()
+            t0 = time.perf_counter()
+            oracle.dequantize(fid, rs, sample * k)
+            e["cpu_baseline"] = {"ms": (time.perf_counter() - t0) * (n / sample) * 1e3, "cores": 1, "kind": "port",
+                                 "sample": f"the first {sample} of {n} rows through the C restatement of the per-value decode, one thread, time scaled"}
+        lib.lib.jitnn_hip_weight_free(h)
+        out[name] = e
+        del t, y
+    for name, rows, k in (("quantize_q8_0_512x14336", 512, 14336), ("quantize_q8_0_14336x4096", 14336, 4096)):
+        g = torch.Generator(device="cuda").manual_seed(77)
+        x = torch.randn(rows, k, generator=g, device="cuda")
+        q = torch.empty(rows * k // 32 * 34, dtype=torch.uint8, device="cuda")
+        xp, qp = C.c_void_p(x.data_ptr()), C.c_void_p(q.data_ptr())
+        sec = timed(lambda: lib.check(lib.lib.jitnn_hip_quantize_q8_0_dev(xp, rows * k, qp, stream), "quantize"))
+        nbytes = 4 * rows * k + q.numel()
+        sample = min(rows, 64)
+        e = {"workload": f"FP32 [{rows}, {k}] -> Q8_0 blocks", "us": sec * 1e6, "bytes_per_call": nbytes, "GBps": nbytes / sec / 1e9,
+             "pct_of_peak": nbytes / sec / 1e9 / PEAK_HBM_GBPS * 100,
+             "bit_exact_first_rows": bool(np.array_equal(q[:sample * k // 32 * 34].cpu().numpy(), oracle.quantize_q8_0(x[:sample].cpu().numpy())))}
+        if with_cpu:
+            cs = min(rows, 1024)
+            xs = x[:cs].cpu().numpy()
+            t0 = time.perf_counter()
+            oracle.quantize_q8_0(xs)
+            e["cpu_baseline"] = {"ms": (time.perf_counter() - t0) * (rows / cs) * 1e3, "cores": 1, "kind": "port",
+                                 "sample": f"the first {cs} of {rows} rows through the C restatement of Quant.quantize, one thread, time scaled"}
+        out[name] = e
+        del x, q
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -566,12 +635,14 @@ def main() -> int:
             w2.close()
             configs[name] = out
 
-    decode = prefill = None
+    decode = prefill = codec = None
     if not a.quick or a.decode:
         if not only or "decode" in only:
             decode = bench_decode(torch, lib, steps=30, warmup=3)
         if (not only or "prefill" in only) and not a.quick:
             prefill = bench_prefill(torch, lib, with_cpu=not a.no_cpu)
+        if (not only or "codec" in only) and not a.quick:
+            codec = bench_codec(torch, lib, with_cpu=not a.no_cpu)
 
     ms = head["us_per_step_wall"] / 1e3
     line = {
@@ -602,6 +673,7 @@ def main() -> int:
         "configs": configs,
         "decode": decode,
         "prefill": prefill,
+        "codec": codec,
     }
     print(json.dumps(line))
     return 0

@@ -222,34 +222,111 @@ static __global__ void __launch_bounds__(256) transcode_q3_k_to_q6_k_kernel(cons
     }
 }
 
-// FP32 -> Q8_0, one thread per block of 32 values, in the reference quantiser's arithmetic
-// (core/ops/Quant.java:102-118): amax in double, d = (float)(amax / 127.0) stored as binary16 (round to
-// nearest even), quants = round-half-away(x / (double)d) with the unrounded float d, clamped to +-127.
+// FP32 -> Q8_0 in the reference quantiser's arithmetic (core/ops/Quant.java:102-118): amax in double, d = (float)(amax / 127.0)
+// stored as binary16 (round to nearest even), quants = round-half-away(x / (double)d) with the unrounded float d, clamped
+// to +-127.  One block of 32 values, the reference's expressions as they stand:
+__device__ __forceinline__ void quantize_q8_0_block(const float *__restrict__ xb, uint8_t *__restrict__ o) {
+    double amax = 0;
+#pragma unroll 1  // (rolled: this is the rare path of the kernel below, and must not cost it registers)
+    for (int l = 0; l < 32; ++l) {
+        double a = fabs((double)xb[l]);
+        amax = a > amax ? a : amax;
+    }
+    const float d = (float)(amax / 127.0);
+    o[0] = (uint8_t)(__half_as_ushort(__float2half_rn(d)) & 0xff);
+    o[1] = (uint8_t)(__half_as_ushort(__float2half_rn(d)) >> 8);
+#pragma unroll 1
+    for (int l = 0; l < 32; ++l) {
+        double s = d > 0 ? (double)xb[l] / (double)d : 0.0;
+        long long r = s >= 0 ? (long long)(s + 0.5) : -(long long)(-s + 0.5);
+        r = r < -127 ? -127 : (r > 127 ? 127 : r);
+        o[2 + l] = (uint8_t)(int8_t)r;
+    }
+}
+
+// The kernel: a wave takes Q8Q_BLOCKS consecutive blocks per turn with coalesced 16-byte loads - eight lanes share a
+// block -, finds the block maxima with three lane exchanges, lets one lane per block do the one FP64
+// division of d, and writes the blocks through its own LDS region as whole dwords.  The 32 FP64 divisions per block of
+// the reference's expression are not needed for its bits: with q = |x| / d the exact quotient of two floats and
+// 0.5 <= q < 128, 2 q - (2 k + 1) is either zero or at least 2^-24 in magnitude (numerator and denominator are 24-bit
+// integers times a power of two that leaves the difference of the cross products an integer), while the division, and
+// the addition of 0.5 after it, each err by at most 2^-46: the reference's result IS the exact quotient rounded half
+// away from zero.  So: a candidate from one FP32 multiplication (off by one at most), set right by the signs of
+// fma(r + 1/2, d, -|x|) and fma(r - 1/2, d, -|x|) - an FMA rounds the exact value once, its sign is the exact sign.
+// Blocks with a value that is not finite or beyond 2^100, or a maximum below 2^-100 (d near or in the subnormals), take
+// the reference's expression itself.  grid: any; 256 threads.
+constexpr int Q8Q_NI = 4, Q8Q_BLOCKS = 8 * Q8Q_NI;  // 16-byte loads per lane and blocks per wave and turn
 static __global__ void __launch_bounds__(256) quantize_q8_0_kernel(const float *__restrict__ x, uint8_t *__restrict__ q, size_t blocks) {
-    for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < blocks; b += (size_t)gridDim.x * blockDim.x) {
-        const float *xb = x + b * 32;
-        float v[32];
+    constexpr int NI = Q8Q_NI, NB = Q8Q_BLOCKS;
+    __shared__ __align__(16) uint8_t out_s[4][NB * 34];
+    __shared__ float amax_s[4][NB], d_s[4][NB];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane >> 3, part = lane & 7;
+    auto wave_sync = [] {  // the lanes of a wave run in step and LDS serves them in order: a fence for the compiler
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    for (size_t w0 = ((size_t)blockIdx.x * 4 + wave) * NB; w0 < blocks; w0 += (size_t)gridDim.x * 4 * NB) {
+        const int nb = (int)(blocks - w0 < NB ? blocks - w0 : NB);
+        const float *xw = x + w0 * 32;
+        float4 v[NI];
+        bool odd = false;  // a value outside the range the short form is proven for
 #pragma unroll
-        for (int l = 0; l < 8; ++l) {
-            float4 t = reinterpret_cast<const float4 *>(xb)[l];
-            v[4 * l] = t.x; v[4 * l + 1] = t.y; v[4 * l + 2] = t.z; v[4 * l + 3] = t.w;
-        }
-        double amax = 0;
+        for (int i = 0; i < NI; ++i)  // block 8 i + sub of the wave's, values 4 part .. 4 part + 3; all requests before the first use,
+            v[i] = *reinterpret_cast<const float4 *>(xw + (8 * i + sub < nb ? 256 * i + 4 * lane : 4 * part));  // none conditional
 #pragma unroll
-        for (int l = 0; l < 32; ++l) {
-            double a = fabs((double)v[l]);
-            amax = a > amax ? a : amax;
+        for (int i = 0; i < NI; ++i) {
+            if (8 * i + sub >= nb) v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            const float a0 = fabsf(v[i].x), a1 = fabsf(v[i].y), a2 = fabsf(v[i].z), a3 = fabsf(v[i].w);
+            odd |= !(a0 <= 0x1p100f) | !(a1 <= 0x1p100f) | !(a2 <= 0x1p100f) | !(a3 <= 0x1p100f);
+            float m = fmaxf(fmaxf(a0, a1), fmaxf(a2, a3));
+            m = fmaxf(m, __shfl_xor(m, 1));
+            m = fmaxf(m, __shfl_xor(m, 2));
+            m = fmaxf(m, __shfl_xor(m, 4));
+            if (part == 0) amax_s[wave][8 * i + sub] = m;
         }
-        const float d = (float)(amax / 127.0);
-        uint8_t *o = q + b * 34;
-        *reinterpret_cast<uint16_t *>(o) = __half_as_ushort(__float2half_rn(d));
+        wave_sync();
+        if (lane < NB) {  // one lane per block: the scale
+            const float am = amax_s[wave][lane];
+            odd |= am > 0.f && am < 0x1p-100f;
+            const float d = (float)((double)am / 127.0);
+            d_s[wave][lane] = d;
+            *reinterpret_cast<uint16_t *>(&out_s[wave][34 * lane]) = __half_as_ushort(__float2half_rn(d));
+        }
+        if (__any(odd)) {  // (wave-uniform) the reference's expression, a block per lane, straight to memory
+            if (lane < nb) quantize_q8_0_block(xw + 32 * lane, q + (w0 + lane) * 34);
+            wave_sync();
+            continue;
+        }
+        wave_sync();
 #pragma unroll
-        for (int l = 0; l < 32; ++l) {
-            double s = d > 0 ? (double)v[l] / (double)d : 0.0;
-            long long r = s >= 0 ? (long long)(s + 0.5) : -(long long)(-s + 0.5);
-            r = r < -127 ? -127 : (r > 127 ? 127 : r);
-            o[2 + l] = (uint8_t)(int8_t)r;
+        for (int i = 0; i < NI; ++i) {
+            const int blk = 8 * i + sub;
+            const float d0 = d_s[wave][blk], d = d0 > 0.f ? d0 : 1.f, inv = 1.0f / d;  // (a block of zeros: any scale gives zeros)
+            const float xs[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+            uint32_t packed = 0;  // bytes q + 128, by the float -> byte converter that also places the byte
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float a = fabsf(xs[e]);
+                float r = rintf(a * inv);
+                // |x| / d >= r + 1/2: one more; |x| / d < r - 1/2: one less (never both).  No clamp: |x| <= amax and d is
+                // amax / 127 rounded to float, so the quotient stays below 127.5.
+                const float step = __builtin_fmaf(r + 0.5f, d, -a) <= 0.f ? 1.f : (__builtin_fmaf(r - 0.5f, d, -a) > 0.f ? -1.f : 0.f);
+                packed = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_copysignf(r + step, xs[e]) + 128.f, e, packed);
+            }
+            packed ^= 0x80808080u;  // q + 128 -> the two's complement byte of q
+            uint16_t *o = reinterpret_cast<uint16_t *>(&out_s[wave][34 * blk + 2 + 4 * part]);  // 2-byte aligned
+            o[0] = (uint16_t)packed;
+            o[1] = (uint16_t)(packed >> 16);
         }
+        wave_sync();
+        uint8_t *qw = q + w0 * 34;  // a multiple of NB blocks: 4-byte aligned whenever q is
+        if (nb == NB && (reinterpret_cast<uintptr_t>(qw) & 3) == 0) {
+            for (int j = lane; j < NB * 34 / 4; j += 64) reinterpret_cast<uint32_t *>(qw)[j] = reinterpret_cast<const uint32_t *>(out_s[wave])[j];
+        } else {
+            for (int j = lane; j < nb * 34; j += 64) qw[j] = out_s[wave][j];
+        }
+        wave_sync();  // the next round's writes wait for these reads
     }
 }
 

@@ -1196,8 +1196,8 @@ int jitnn_hip_quantize_q8_0_dev(const float *x_dev, long long numel, void *block
     if (numel == 0) return JITNN_HIP_OK;
     count_op(ST_QUANT, 4ll * numel + numel / 32 * 34);
     const size_t blocks = (size_t)numel / 32;
-    size_t grid = (blocks + 255) / 256;
-    if (grid > (size_t)g.cus * 16) grid = (size_t)g.cus * 16;
+    size_t grid = (blocks + 4 * Q8Q_BLOCKS - 1) / (4 * Q8Q_BLOCKS);
+    if (grid > (size_t)g.cus * 32) grid = (size_t)g.cus * 32;
     hipLaunchKernelGGL(quantize_q8_0_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, x_dev, (uint8_t *)blocks_dev, blocks);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;

@@ -346,6 +346,36 @@ def test_quantize_q8_0_bit_exact_vs_oracle(jn):
     assert norm_err(y, oracle.gguf_linear(8, xin, exp, b, 64, 256)) <= 1e-5
 
 
+def test_quantize_q8_0_bytes_on_ties_extremes_and_ragged_sizes(jn):
+    """The quantiser's bytes against the oracle's on what its short form must get right: values on and one float either
+    side of every half-integer multiple of the block's scale, blocks whose scale is huge, tiny, subnormal or zero, and
+    sizes that are not whole groups of 64 blocks.  (Values that are not finite are outside the reference's tests, and the C
+    oracle's cast of NaN to an integer is not Java's.)"""
+    import ctypes as C
+    from jitnn_amd import _lib
+    from oracle import oracle
+    rng = np.random.default_rng(33)
+    rows = []
+    for amax in (127.0, 1.0, 3.1415927, 1e-3, 6.5e4, 1e20, 1e-20, 2.0 ** -99, 2.0 ** -101, 1e-38, 1e-42, 3e38):
+        d = np.float32(np.float64(np.float32(amax)) / 127.0)
+        for _ in range(3):
+            ks = rng.integers(0, 127, size=31)
+            ties = ((ks + 0.5) * np.float64(d)).astype(np.float32)
+            ties = np.nextafter(ties, np.float32(rng.choice([-np.inf, np.inf])) if rng.integers(3) else ties).astype(np.float32)
+            blk = np.concatenate([[np.float32(amax)], ties * rng.choice([-1, 1], size=31).astype(np.float32)])
+            rows.append(rng.permutation(blk).astype(np.float32))
+    rows.append(np.zeros(32, dtype=np.float32))
+    rows.append(np.full(32, -0.0, dtype=np.float32))
+    special = np.stack(rows)
+    bulk = (rng.standard_normal((64 * 5 + 37, 32)) * 10.0 ** rng.uniform(-6, 6, size=(64 * 5 + 37, 1))).astype(np.float32)
+    x = np.concatenate([special, bulk])
+    for count in (x.shape[0], 64, 65, 1, 200):
+        xs = np.ascontiguousarray(x[:count])
+        got = np.empty(xs.size // 32 * 34, dtype=np.uint8)
+        rc = _lib.lib.jitnn_hip_quantize_q8_0(xs.ctypes.data_as(C.c_void_p), xs.size, got.ctypes.data_as(C.c_void_p))
+        assert rc == 0 and np.array_equal(got, oracle.quantize_q8_0(xs)), count
+
+
 # ------------------------------------------------------------------------------------------ the other dequantisable formats
 
 # Q5_1, Q2_K: bit-exact dequantiser + plain GEMV, no tuned kernels.  Q5_0, Q3_K: rewritten at upload into Q8_0 / Q6_K blocks
