@@ -10,13 +10,6 @@
 
 namespace jitnn {
 
-// 6-bit scale (part 0) or min (part 1) of sub-block j from the 12 scale bytes at s (GgufKernels.java:74-83).
-__device__ __forceinline__ int k4_scale_min(const uint8_t *s, int j, int part) {
-    if (j < 4) return s[j + 4 * part] & 63;
-    int low = part == 0 ? (s[j + 4] & 15) : (s[j + 4] >> 4);
-    return low | ((s[j - 4 + 4 * part] >> 6) << 4);
-}
-
 // Four consecutive values i..i+3 (i % 4 == 0) of a tensor: they share block, sub-block, nibble half and scale.
 template <int FMT>
 __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
@@ -25,9 +18,10 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
         const uint8_t *b = w + (i >> 5) * 18;
         const int e = (int)(i & 31);
         const float d = h2f(ld16(b));
+        const uint32_t vs = ld32<2>(b + 2 + (e & 15));  // the four bytes of the quad at once
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            int v = b[2 + ((e + t) & 15)];
+            int v = (vs >> (8 * t)) & 255;
             int q = e < 16 ? (v & 15) : (v >> 4);
             o[t] = (float)(q - 8) * d;
         }
@@ -35,9 +29,10 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
         const uint8_t *b = w + (i >> 5) * 20;
         const int e = (int)(i & 31);
         const float d = h2f(ld16(b)), m = h2f(ld16(b + 2));
+        const uint32_t vs = ld32<4>(b + 4 + (e & 15));
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            int v = b[4 + ((e + t) & 15)];
+            int v = (vs >> (8 * t)) & 255;
             int q = e < 16 ? (v & 15) : (v >> 4);
             float p = (float)q * d;
             o[t] = p + m;
@@ -46,20 +41,30 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
         const uint8_t *b = w + (i >> 5) * 34;
         const int e = (int)(i & 31);
         const float d = h2f(ld16(b));
+        const uint32_t vs = ld32<2>(b + 2 + e);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) o[t] = d * (float)(int)(int8_t)b[2 + e + t];
+        for (int t = 0; t < 4; ++t) o[t] = d * (float)(int)(int8_t)(uint8_t)(vs >> (8 * t));
     } else if constexpr (FMT == F_Q4_K || FMT == F_Q5_K) {
         constexpr int NB = FMT == F_Q4_K ? 144 : 176, QS = FMT == F_Q4_K ? 16 : 48;
         const uint8_t *b = w + (i >> 8) * NB;
         const int e = (int)(i & 255);
         const int j = e >> 6, half = (e & 63) >> 5, l = e & 31, sub = 2 * j + half;
-        const float ds = h2f(ld16(b)) * (float)k4_scale_min(b + 4, sub, 0);
-        const float m = h2f(ld16(b + 2)) * (float)k4_scale_min(b + 4, sub, 1);
+        // d, dmin and the twelve scale bytes as four dwords; the 6-bit scale and min of sub-block `sub` (GgufKernels.java:74-83):
+        // bytes sub and sub + 4 for sub < 4, else a nibble of byte sub + 4 with the top two bits of byte sub - 4 or sub
+        const uint32_t dm = ld32<4>(b), s0 = ld32<4>(b + 4), s1 = ld32<4>(b + 8), s2 = ld32<4>(b + 12);
+        const int sh = 8 * (sub & 3);
+        const int sc = sub < 4 ? (s0 >> sh) & 63 : ((s2 >> sh) & 15) | (((s0 >> (sh + 6)) & 3) << 4);
+        const int mn = sub < 4 ? (s1 >> sh) & 63 : ((s2 >> (sh + 4)) & 15) | (((s1 >> (sh + 6)) & 3) << 4);
+        const float ds = h2f(dm) * (float)sc;
+        const float m = h2f(dm >> 16) * (float)mn;
+        const uint32_t vs = ld32<4>(b + QS + 32 * j + l);
+        uint32_t hs = 0;
+        if constexpr (FMT == F_Q5_K) hs = ld32<4>(b + 16 + l);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            int v = b[QS + 32 * j + l + t];
+            int v = (vs >> (8 * t)) & 255;
             int q = half == 0 ? (v & 15) : (v >> 4);
-            if constexpr (FMT == F_Q5_K) q += 16 * ((b[16 + l + t] >> sub) & 1);
+            if constexpr (FMT == F_Q5_K) q += 16 * ((((hs >> (8 * t)) & 255) >> sub) & 1);
             float a = ds * (float)q;
             o[t] = a - m;
         }
@@ -118,11 +123,12 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
         const int n = e >> 7, k = (e & 127) >> 5, l = e & 31;
         const int sc = (int)(int8_t)b[192 + 8 * n + (l >> 4) + 2 * k];
         const float a = h2f(ld16(b + 208)) * (float)sc;
+        const uint32_t ls = ld32<2>(b + 64 * n + l + (k & 1) * 32), hs = ld32<2>(b + 128 + 32 * n + l);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            int lb = b[64 * n + l + t + (k & 1) * 32];
+            int lb = (ls >> (8 * t)) & 255;
             int low = k < 2 ? (lb & 15) : (lb >> 4);
-            int hb = (b[128 + 32 * n + l + t] >> (2 * k)) & 3;
+            int hb = (((hs >> (8 * t)) & 255) >> (2 * k)) & 3;
             o[t] = a * (float)(low + 16 * hb - 32);
         }
     }
