@@ -75,10 +75,12 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
         const uint8_t *b = w + (i >> 5) * NB;
         const int e = (int)(i & 31);
         const float d = h2f(ld16(b));
+        constexpr int AL = FMT == F_Q5_0 ? 2 : 4;
+        const uint32_t vs = ld32<AL>(b + QS + (e & 15)), qh = ld32<AL>(b + QH);  // the quad's nibble bytes; bit e of qh is value e's
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const int v = b[QS + ((e + t) & 15)];
-            const int q = (e < 16 ? (v & 15) : (v >> 4)) + 16 * ((b[QH + ((e + t) >> 3)] >> ((e + t) & 7)) & 1);
+            const int v = (vs >> (8 * t)) & 255;
+            const int q = (e < 16 ? (v & 15) : (v >> 4)) + 16 * ((qh >> (e + t)) & 1);
             if constexpr (FMT == F_Q5_0) {
                 o[t] = (float)(q - 16) * d;
             } else {
@@ -95,9 +97,10 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
         const int sc = b[n * 8 + j * 2 + (l >> 4)];
         const float ds = h2f(ld16(b + 80)) * (float)(sc & 15);
         const float m = h2f(ld16(b + 82)) * (float)(sc >> 4);
+        const uint32_t vs = ld32<4>(b + 16 + n * 32 + l);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const int q = (b[16 + n * 32 + l + t] >> (2 * j)) & 3;
+            const int q = (vs >> (8 * t + 2 * j)) & 3;
             const float a = ds * (float)q;
             o[t] = a - m;
         }
@@ -111,10 +114,11 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
         const int low = is < 8 ? (b[96 + is] & 15) : (b[96 + is - 8] >> 4);
         const int high = (b[96 + 8 + (is & 3)] >> (2 * (is >> 2))) & 3;
         const float a = h2f(ld16(b + 108)) * (float)(low + 16 * high - 32);
+        const uint32_t vs = ld32<2>(b + 32 + n * 32 + l), hs = ld32<2>(b + l);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const int q = (b[32 + n * 32 + l + t] >> (2 * j)) & 3;
-            const int hb = (b[l + t] >> (4 * n + j)) & 1;
+            const int q = (vs >> (8 * t + 2 * j)) & 3;
+            const int hb = (hs >> (8 * t + 4 * n + j)) & 1;
             o[t] = a * (float)(q - (hb == 1 ? 0 : 4));
         }
     } else {  // F_Q6_K
