@@ -14,6 +14,8 @@ namespace jitnn {
 enum : int { F_Q4_0 = 2, F_Q4_1 = 3, F_Q8_0 = 8, F_Q4_K = 12, F_Q5_K = 13, F_Q6_K = 14, F_Q5_0 = 6, F_Q5_1 = 7, F_Q2_K = 10, F_Q3_K = 11 };
 
 __host__ __device__ constexpr bool is_extra_format(int fmt) { return fmt == F_Q5_0 || fmt == F_Q5_1 || fmt == F_Q2_K || fmt == F_Q3_K; }
+// (of these, Q5_1 and Q2_K have a decoder in the many-row kernel; Q5_0 and Q3_K reach it rewritten as Q8_0 and Q6_K)
+__host__ __device__ constexpr bool has_many_row_kernel(int fmt) { return !is_extra_format(fmt) || fmt == F_Q5_1 || fmt == F_Q2_K; }
 
 __host__ __device__ constexpr int block_values(int fmt) {
     return (fmt == F_Q4_0 || fmt == F_Q4_1 || fmt == F_Q8_0 || fmt == F_Q5_0 || fmt == F_Q5_1) ? 32

@@ -1116,7 +1116,7 @@ int linear_dev(const jitnn_hip_weight *w, const float *x_dev, int rows, const fl
     if (!w || !x_dev || !y_dev) return fail(JITNN_HIP_EINVAL, "weight, input or output is NULL");
     if (rows < 1) return fail(JITNN_HIP_EINVAL, "rows = %d", rows);
     if (int rc = check_ready()) return rc;
-    const bool many = rows > g.gemv_max_rows && !is_extra_format(w->fmt);
+    const bool many = rows > g.gemv_max_rows && has_many_row_kernel(w->fmt);
     count_op(many ? ST_MFMA : ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n) + (bias_dev ? 4ll * w->n : 0));
     if (many) return launch_prefill(w, x_dev, rows, bias_dev, y_dev, s, src);
     // several rows, rows of whole 256-value columns: every row meets the weights in one pass over them (gemv_rows.h)
@@ -1485,7 +1485,7 @@ void flush_pending(PfPending &p, int rows, hipStream_t st) {
 int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const *ws, float *const *ys, int count, const float *x, int rows,
                         const float *nw, float *xn, hipStream_t st, PfPending *pend = nullptr, PfGroupPending *gdefer = nullptr) {
     bool group = rows > g.gemv_max_rows && prefill_prepare_fuses_norm(m->d);
-    for (int i = 0; i < count; ++i) group = group && !is_extra_format(ws[i]->fmt);
+    for (int i = 0; i < count; ++i) group = group && has_many_row_kernel(ws[i]->fmt);
     if (group) {
         const bool fused = pend && pend->part && pend->out == x && pend->n == m->d;
         const int rc = launch_prefill_group(ws, ys, count, x, rows, nullptr, nw, m->eps, st, nullptr, nullptr, nullptr, SCRATCH_THREAD, nullptr, nullptr,
@@ -1514,7 +1514,7 @@ int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const 
 // part / defer: see launch_prefill_group - the join of the K slices may be left to the caller.
 int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, const float *res, float *tmp, float *y, hipStream_t st,
                          const float *up = nullptr, float *h = nullptr, float *part = nullptr, PfPending *defer = nullptr) {
-    const bool many = rows > g.gemv_max_rows && !is_extra_format(w->fmt) && w->n % 4 == 0;
+    const bool many = rows > g.gemv_max_rows && has_many_row_kernel(w->fmt) && w->n % 4 == 0;
     if (many && (!up || (g.prefill_fuse_swiglu && prefill_prepare_fuses_norm(w->k)))) {
         return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp, up, SCRATCH_THREAD, g.prefill_defer_join ? part : nullptr,
                                     g.prefill_defer_join ? defer : nullptr);

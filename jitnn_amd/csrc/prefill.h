@@ -228,6 +228,10 @@ template <>
 struct PfRaw<F_Q5_K> { u32x4 h, q0, q1, qh0, qh1; };
 template <>
 struct PfRaw<F_Q6_K> { u32x4 l0, l1, h0, h1; uint32_t sc, d; };
+template <>
+struct PfRaw<F_Q5_1> { u32x4 q; uint32_t dm, qh; };
+template <>
+struct PfRaw<F_Q2_K> { u32x4 q0, q1; uint32_t sc, dd; };
 
 template <int FMT>
 __device__ __forceinline__ void pf_load(PfRaw<FMT> &r, const uint8_t *row, int k0) {
@@ -239,6 +243,18 @@ __device__ __forceinline__ void pf_load(PfRaw<FMT> &r, const uint8_t *row, int k
         const uint8_t *b = row + (size_t)(k0 >> 5) * 20;
         r.dm = ld32<4>(b);
         r.q = ld128<4>(b + 4);
+    } else if constexpr (FMT == F_Q5_1) {  // 24 bytes: d, m, 32 fifth bits, 16 bytes of nibbles
+        const uint8_t *b = row + (size_t)(k0 >> 5) * 24;
+        r.dm = ld32<4>(b);
+        r.qh = ld32<4>(b + 4);
+        r.q = ld128<4>(b + 8);
+    } else if constexpr (FMT == F_Q2_K) {  // 84 bytes: 16 scale bytes, 64 bytes of 2-bit quants, d, dmin
+        const uint8_t *b = row + (size_t)(k0 >> 8) * 84;
+        const int e = k0 & 255, n = e >> 7, j = (e & 127) >> 5;
+        r.q0 = ld128<4>(b + 16 + 32 * n);
+        r.q1 = ld128<4>(b + 16 + 32 * n + 16);
+        r.sc = ld16(b + 8 * n + 2 * j);
+        r.dd = ld32<4>(b + 80);
     } else if constexpr (FMT == F_Q8_0) {
         const uint8_t *b = row + (size_t)(k0 >> 5) * 34;
         r.d = ld16(b);
@@ -287,6 +303,26 @@ __device__ __forceinline__ void pf_decode(const PfRaw<FMT> &r, int k0, float (&o
                 o[i] = (float)(byte & 15u) * d + m;
                 o[16 + i] = (float)(byte >> 4) * d + m;
             }
+        }
+    } else if constexpr (FMT == F_Q5_1) {  // (q_low + 16 bit e of qh) d + m (GgufKernels.java:155-163)
+        const float d = h2f(r.dm), m = h2f(r.dm >> 16);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const uint32_t byte = (r.q[i >> 2] >> (8 * (i & 3))) & 0xffu;
+            const float lo = (float)((byte & 15u) + 16u * ((r.qh >> i) & 1u)) * d, hi = (float)((byte >> 4) + 16u * ((r.qh >> (16 + i)) & 1u)) * d;
+            o[i] = lo + m;
+            o[16 + i] = hi + m;
+        }
+    } else if constexpr (FMT == F_Q2_K) {  // d (scale nibble) q - dmin (min nibble), a scale byte per 16 values (GgufKernels.java:166-175)
+        const int j = ((k0 & 127) >> 5);
+        const float d = h2f(r.dd), dmin = h2f(r.dd >> 16);
+        const float ds0 = d * (float)(r.sc & 15u), m0 = dmin * (float)((r.sc >> 4) & 15u);
+        const float ds1 = d * (float)((r.sc >> 8) & 15u), m1 = dmin * (float)((r.sc >> 12) & 15u);
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+            const uint32_t w = i < 16 ? r.q0[i >> 2] : r.q1[(i - 16) >> 2];
+            const float a = (i < 16 ? ds0 : ds1) * (float)((w >> (8 * (i & 3) + 2 * j)) & 3u);
+            o[i] = a - (i < 16 ? m0 : m1);
         }
     } else if constexpr (FMT == F_Q8_0) {
         const float d = h2f(r.d);

@@ -1,4 +1,4 @@
-// prefill_mfma_kernel for the 32-value formats, the activation preparation and the join of K slices.
+// prefill_mfma_kernel for the 32-value formats (Q5_1 among them), the activation preparation and the join of K slices.
 #include "prefill.h"
 #include "tu.h"
 
@@ -9,6 +9,7 @@ KernelRef prefill_kernel_q32(int fmt) {
     case F_Q4_0: return {(const void *)prefill_mfma_kernel<F_Q4_0>, pf_lds_bytes<F_Q4_0>()};
     case F_Q4_1: return {(const void *)prefill_mfma_kernel<F_Q4_1>, pf_lds_bytes<F_Q4_1>()};
     case F_Q8_0: return {(const void *)prefill_mfma_kernel<F_Q8_0>, pf_lds_bytes<F_Q8_0>()};
+    case F_Q5_1: return {(const void *)prefill_mfma_kernel<F_Q5_1>, pf_lds_bytes<F_Q5_1>()};
     default: return {nullptr, 0};
     }
 }
@@ -18,6 +19,7 @@ void prefill_launch_q32(int fmt, dim3 grid, hipStream_t s, const PfSegments &sg,
     case F_Q4_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_0>, grid, dim3(256), pf_lds_bytes<F_Q4_0>(), s, sg, xo, inv_scale, bias, m, k); break;
     case F_Q4_1: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q4_1>, grid, dim3(256), pf_lds_bytes<F_Q4_1>(), s, sg, xo, inv_scale, bias, m, k); break;
     case F_Q8_0: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q8_0>, grid, dim3(256), pf_lds_bytes<F_Q8_0>(), s, sg, xo, inv_scale, bias, m, k); break;
+    case F_Q5_1: hipLaunchKernelGGL(prefill_mfma_kernel<F_Q5_1>, grid, dim3(256), pf_lds_bytes<F_Q5_1>(), s, sg, xo, inv_scale, bias, m, k); break;
     default: break;
     }
 }
