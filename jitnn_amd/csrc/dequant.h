@@ -139,10 +139,36 @@ __device__ __forceinline__ float4 dequant4(const uint8_t *w, size_t i) {
     return make_float4(o[0], o[1], o[2], o[3]);
 }
 
+// Q6_K: a lane's four values need bytes from four fields of the block, and four narrow load instructions per wave and
+// 1 KiB of output keep the CU's one address unit busier than the memory behind it.  A wave takes a whole block - 64
+// quads - instead: thirteen lanes fetch its 208 bytes as 16-byte pieces and a fourteenth its last 16 bytes for the two of d
+// (one load instruction, nothing read past the block), the pieces are parted through the wave's own LDS region, and every lane
+// decodes its quad from there with the same expressions.
 template <int FMT>
 __global__ void __launch_bounds__(256) dequant_kernel(const uint8_t *__restrict__ w, float *__restrict__ y, size_t quads) {
-    for (size_t f = (size_t)blockIdx.x * blockDim.x + threadIdx.x; f < quads; f += (size_t)gridDim.x * blockDim.x) {
-        reinterpret_cast<float4 *>(y)[f] = dequant4<FMT>(w, f * 4);
+    if constexpr (FMT == F_Q6_K) {
+        __shared__ __align__(16) uint8_t stage[4][224];
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const size_t nblk = quads / 64, nwaves = (size_t)gridDim.x * 4;
+        for (size_t blk = (size_t)blockIdx.x * 4 + wave; blk < nblk; blk += nwaves) {
+            const uint8_t *b = w + blk * 210;
+            if (lane < 14) {  // (the fourteenth lane: the block's last 16 bytes, d in the top half-word)
+                const u32x4 c = ld128<2>(b + (lane < 13 ? 16 * lane : 194));
+                if (lane < 13) *reinterpret_cast<u32x4 *>(&stage[wave][16 * lane]) = c;
+                else *reinterpret_cast<uint16_t *>(&stage[wave][208]) = (uint16_t)(c.w >> 16);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // (the lanes of a wave run in step, LDS serves them in order)
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            reinterpret_cast<float4 *>(y)[blk * 64 + lane] = dequant4<FMT>(stage[wave], (size_t)lane * 4);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+    } else {
+        for (size_t f = (size_t)blockIdx.x * blockDim.x + threadIdx.x; f < quads; f += (size_t)gridDim.x * blockDim.x) {
+            reinterpret_cast<float4 *>(y)[f] = dequant4<FMT>(w, f * 4);
+        }
     }
 }
 
