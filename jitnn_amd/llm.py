@@ -1,4 +1,4 @@
-"""Host mirror of jitnn-llm's Llm (jitnn-llm/src/main/java/ai/beestream/jitnn/llm/Llm.java:47-120): a GGUF language model
+"""Host mirror of jitnn-llm's Llm (jitnn-llm/src/main/java/ai/beestream/jitnn/llm/Llm.java:48-120): a GGUF language model
 that generates text.  The reference hands generation to the third-party jitllm engine; here the file's quantised weights
 are attached to the decode step of libjitnn_hip.so (jitnn_hip_llama_*), the token loop runs in the library
 (jitnn_hip_llama_generate: embedding lookup, prompt pass, greedy choice, token-by-token decode over the KV cache) and the
