@@ -1,0 +1,438 @@
+// Batch-1 GEMV on raw K-quant blocks with the dot products on the matrix cores in INT8 (gfx950, wave64).
+//
+// The quants of a K-quant block are small integers (4, 5 or 6 bits) and sit in memory as nibbles and bit fields: two or
+// three mask / shift instructions turn a dword of them into four INT8 values - an operand of v_mfma_i32_4x4x4_16b_i8 as
+// it stands.  The activations are turned once per workgroup into 22-bit fixed point per 64-value chunk (a power-of-two
+// step from the chunk's largest magnitude, rounding by one FMA with 1.5 * 2^23) and cut into three signed byte digits,
+// v = d0 + 256 d1 + 65536 d2: three of the four operand rows of the 4x4x4 product.  The instruction multiplies sixteen
+// independent 4x4 blocks, each with its own activations: lane 4 b + j feeds the quants of weight row j (of four rows) for
+// chunk b (of sixteen) of the row, lane 4 b + i the digit plane i of chunk b's activations, and the three digit sums of
+// (row j, chunk b) come back to lane 4 b + j - the lane that loaded that row's bytes and decodes its scales.  So the
+// sums are exact integers, nothing crosses lanes between load and scale, and per 64 weights a lane issues 16 matrix
+// instructions and about 24 mask / shift instructions where the FP32 kernel issues 32 conversions and 64 multiply-adds.
+// Error against the FP64 reference: the rounding of x to 2^-22 of its chunk's largest magnitude (about 3e-7 of max|y|).
+//
+// Work decomposition: a workgroup has one wave per 1024 values of the row (four for K = 4096); a turn of the
+// workgroup is a group of four consecutive weight rows, wave w multiplying its 1024-value slice of them.  The slice's
+// partial sums of a turn leave the wave through a two-step DPP fold (16 floats to LDS); every I8_FLUSH turns the
+// workgroup meets at a barrier and one thread per output adds the partial sums in a fixed order - no atomics, the
+// result does not depend on the launch shape.  Weight bytes are prefetched PF turns ahead through a register ring with
+// unconditional loads (turns past the end read one 16-byte piece) so the hardware's in-order load counter is waited on
+// exactly.
+//
+// A slice that holds an activation that is not finite takes a slow path (every weight decoded by the bit-exact
+// expression of the dequantiser and multiplied in FP32) so that +-Inf and NaN come out as the reference's FP64 sum
+// gives them (core/ops/Gguf.java:187-205).
+#pragma once
+#include "common.h"
+#include "dequant.h"
+#include "tu.h"
+
+namespace jitnn {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int I8_FLUSH = 24;   // turns between two joins of the waves' partial sums (a multiple of every ring length)
+constexpr int I8_MAX_WAVES = 16;
+constexpr size_t I8_LDS_PER_WAVE = 3072;  // 16 chunks x 3 planes x 64 bytes; afterwards the wave's partial sums (2 x 24 turns x 16 floats)
+
+__host__ __device__ constexpr size_t gemv_i8_lds_bytes(int waves) { return (size_t)waves * I8_LDS_PER_WAVE; }
+
+// The three digit sums of a block as one number.  With quants of at most five bits the whole sum fits 32 bits
+// (31 * 16 * 2^22 < 2^31); six-bit quants (63 * 16 * 2^22) need the last step in floating point.
+__device__ __forceinline__ int i8_combine(const i32x4 &d) { return (((d[2] << 8) + d[1]) << 8) + d[0]; }
+__device__ __forceinline__ float i8_combine_wide(const i32x4 &d) { return __builtin_fmaf((float)((d[2] << 8) + d[1]), 256.f, (float)d[0]); }
+
+// Weight bytes come through buffer loads: the descriptor (base of the matrix, extent) and the byte offset of the turn's
+// row group sit in scalar registers, the lane's own offsets in vector registers computed once - a load costs no vector
+// arithmetic, and a descriptor of extent zero makes the loads of a turn past the end return zeros without touching memory.
+__device__ __forceinline__ u32x4 i8_ld128(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b128(rs, (int)voff, (int)soff, 0);
+}
+
+template <int FMT>
+struct U8;
+
+// scale and min of sub-blocks 2j and 2j+1 of a Q4_K / Q5_K super-block as packed byte pairs (h = the block's first 16
+// bytes; reference: core/kernels/GgufKernels.java:74-83)
+__device__ __forceinline__ void i8_scale_min(const u32x4 &h, int j, uint32_t &sc2, uint32_t &mn2) {
+    const int sh = (j & 1) * 16;
+    const uint32_t m1 = j < 2 ? 0x3f3fu : 0u, m2 = j < 2 ? 0u : 0x0f0fu, m3 = j < 2 ? 0u : 0x3030u;
+    const uint32_t a = h.y >> sh, b = h.z >> sh, c = h.w >> sh;
+    sc2 = (a & m1) | (c & m2) | ((a >> 2) & m3);
+    mn2 = (b & m1) | ((c >> 4) & m2) | ((b >> 2) & m3);
+}
+
+// ---------------------------------------------------------------------------------------------- Q4_K
+// Chunk c of a row = values [64 c, 64 c + 64): group c % 4 of super-block c / 4, 32 qs bytes whose low nibbles are the
+// first 32 values (sub-block 2j) and whose high nibbles the last 32 (sub-block 2j + 1).
+template <>
+struct U8<F_Q4_K> {
+    static constexpr int FMT = F_Q4_K, NSUM = 2;
+    struct Raw { u32x4 h, q0, q1; };
+    struct Off { uint32_t h, q; };  // byte offsets of the lane's fields from the first row of its row group
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) {
+        Off o;
+        o.h = row_off + (uint32_t)(c >> 2) * 144u;
+        o.q = o.h + 16u + (uint32_t)(c & 3) * 32u;
+        return o;
+    }
+    __device__ static __forceinline__ int x_first(int c, int j) { return c * 64 + j * 16; }  // the 16 values lane (c, j) stages
+    __device__ static __forceinline__ int x_pos(int c, int e) { return c * 64 + e; }         // value e of the chunk in operand order
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.h = i8_ld128(rs, o.h, soff);
+        r.q0 = i8_ld128(rs, o.q, soff);
+        r.q1 = i8_ld128(rs, o.q + 16u, soff);
+    }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
+        s[0] = s4[0] + s4[1];
+        s[1] = s4[2] + s4[3];
+    }
+    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
+        i32x4 dl = {0, 0, 0, 0}, dh = {0, 0, 0, 0};
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const uint32_t v = m < 4 ? r.q0[m & 3] : r.q1[m & 3];
+            dl = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[m], (int)(v & 0x0f0f0f0fu), dl, 0, 0, 0);
+            dh = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + m], (int)((v >> 4) & 0x0f0f0f0fu), dh, 0, 0, 0);
+        }
+        uint32_t sc2, mn2;
+        i8_scale_min(r.h, c & 3, sc2, mn2);
+        const float d = h2f(r.h.x) * sinv, dmin = h2f(r.h.x >> 16);
+        const float t = __builtin_fmaf(d * ub0(sc2), (float)i8_combine(dl), (d * ub1(sc2)) * (float)i8_combine(dh));
+        const float m = __builtin_fmaf(dmin * ub0(mn2), s[0], (dmin * ub1(mn2)) * s[1]);
+        return t - m;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------- Q5_K
+// As Q4_K with a fifth bit: bit (2j + half) of qh[l] (core/kernels/GgufKernels.java:113-125); block 176 bytes:
+// d, dmin, scales[12], qh[32], qs[128].
+template <>
+struct U8<F_Q5_K> {
+    static constexpr int FMT = F_Q5_K, NSUM = 2;
+    struct Raw { u32x4 h, h0, h1, q0, q1; };
+    struct Off { uint32_t h, q; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) {
+        Off o;
+        o.h = row_off + (uint32_t)(c >> 2) * 176u;
+        o.q = o.h + 48u + (uint32_t)(c & 3) * 32u;
+        return o;
+    }
+    __device__ static __forceinline__ int x_first(int c, int j) { return c * 64 + j * 16; }
+    __device__ static __forceinline__ int x_pos(int c, int e) { return c * 64 + e; }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.h = i8_ld128(rs, o.h, soff);
+        r.h0 = i8_ld128(rs, o.h + 16u, soff);
+        r.h1 = i8_ld128(rs, o.h + 32u, soff);
+        r.q0 = i8_ld128(rs, o.q, soff);
+        r.q1 = i8_ld128(rs, o.q + 16u, soff);
+    }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
+        s[0] = s4[0] + s4[1];
+        s[1] = s4[2] + s4[3];
+    }
+    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
+        i32x4 dl = {0, 0, 0, 0}, dh = {0, 0, 0, 0};
+        const int sh = 2 * (c & 3);
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            const uint32_t v = m < 4 ? r.q0[m & 3] : r.q1[m & 3];
+            const uint32_t hb = (m < 4 ? r.h0[m & 3] : r.h1[m & 3]) >> sh;  // bit 0 of every byte: sub-block 2j, bit 1: 2j + 1
+            const uint32_t lo = (v & 0x0f0f0f0fu) | ((hb << 4) & 0x10101010u);
+            const uint32_t hi = ((v >> 4) & 0x0f0f0f0fu) | ((hb << 3) & 0x10101010u);
+            dl = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[m], (int)lo, dl, 0, 0, 0);
+            dh = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + m], (int)hi, dh, 0, 0, 0);
+        }
+        uint32_t sc2, mn2;
+        i8_scale_min(r.h, c & 3, sc2, mn2);
+        const float d = h2f(r.h.x) * sinv, dmin = h2f(r.h.x >> 16);
+        const float t = __builtin_fmaf(d * ub0(sc2), (float)i8_combine(dl), (d * ub1(sc2)) * (float)i8_combine(dh));
+        const float m = __builtin_fmaf(dmin * ub0(mn2), s[0], (dmin * ub1(mn2)) * s[1]);
+        return t - m;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------- Q6_K
+// block_q6_K, 210 bytes: ql[128], qh[64], i8 scales[16], f16 d (core/kernels/GgufKernels.java:127-140).  Chunk
+// c = 4 sb + 2 n + r covers l in [16 r, 16 r + 16) of half n of super-block sb for the four k: four runs of 16 values,
+// run k at x[256 sb + 128 n + 32 k + 16 r ..], each with its own int8 scale (index 8 n + 2 k + r).  The quants come out
+// as q in 0..63; the -32 of the format meets the sums of x over the runs.
+template <>
+struct U8<F_Q6_K> {
+    static constexpr int FMT = F_Q6_K, NSUM = 4;
+    struct Raw { u32x4 la, lb, qh; u32x2 sc; uint32_t d; };
+    struct Off { uint32_t la, qh, sc, d; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) {
+        Off o;
+        const uint32_t blk = row_off + (uint32_t)(c >> 2) * 210u, n = (uint32_t)(c >> 1) & 1u, r = (uint32_t)c & 1u;
+        o.la = blk + 64u * n + 16u * r;
+        o.qh = blk + 128u + 32u * n + 16u * r;
+        o.sc = blk + 192u + 8u * n;
+        o.d = blk + 208u;
+        return o;
+    }
+    __device__ static __forceinline__ int x_first(int c, int j) { return (c >> 2) * 256 + ((c >> 1) & 1) * 128 + 32 * j + 16 * (c & 1); }
+    __device__ static __forceinline__ int x_pos(int c, int e) { return x_first(c, e >> 4) + (e & 15); }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.la = i8_ld128(rs, o.la, soff);   // (fields on 2-byte boundaries: buffer loads take them like the global ones)
+        r.lb = i8_ld128(rs, o.la + 32u, soff);
+        r.qh = i8_ld128(rs, o.qh, soff);
+        r.sc = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)o.sc, (int)soff, 0);
+        r.d = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)o.d, (int)soff, 0);
+    }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] = -32.f * s4[i];
+    }
+    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
+        i32x4 d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0}, d2 = {0, 0, 0, 0}, d3 = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t a = r.la[i], b = r.lb[i], h = r.qh[i];
+            const uint32_t v0 = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
+            const uint32_t v1 = (b & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
+            const uint32_t v2 = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
+            const uint32_t v3 = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
+            d0 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[i], (int)v0, d0, 0, 0, 0);
+            d1 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[4 + i], (int)v1, d1, 0, 0, 0);
+            d2 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + i], (int)v2, d2, 0, 0, 0);
+            d3 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[12 + i], (int)v3, d3, 0, 0, 0);
+        }
+        const int sh = (c & 1) * 8;
+        const uint32_t sa = r.sc.x >> sh, sb = r.sc.y >> sh;  // bytes 0 and 2: the scales of runs 0, 1 | 2, 3
+        float acc = (float)(int)(int8_t)sa * __builtin_fmaf(i8_combine_wide(d0), sinv, s[0]);
+        acc = __builtin_fmaf((float)(int)(int8_t)(sa >> 16), __builtin_fmaf(i8_combine_wide(d1), sinv, s[1]), acc);
+        acc = __builtin_fmaf((float)(int)(int8_t)sb, __builtin_fmaf(i8_combine_wide(d2), sinv, s[2]), acc);
+        acc = __builtin_fmaf((float)(int)(int8_t)(sb >> 16), __builtin_fmaf(i8_combine_wide(d3), sinv, s[3]), acc);
+        return acc * h2f(r.d);
+    }
+};
+
+// -------------------------------------------------------------------------------------------------- the kernel body
+template <class U, int PF, bool BIAS, bool NORM, bool DUAL>
+__device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, const int nblocks) {
+    constexpr int FMT = U::FMT, NB = PF + 1, FL = I8_FLUSH;
+    static_assert(FL % NB == 0 && FL % 2 == 0, "whole rings (and gate/up pairs) per flush window");
+    extern __shared__ __align__(16) uint8_t i8_smem[];
+    __shared__ float red[I8_MAX_WAVES];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
+    u32x4 *const planes = reinterpret_cast<u32x4 *>(i8_smem + (size_t)wave * I8_LDS_PER_WAVE);
+    float *const mypart = reinterpret_cast<float *>(planes);  // after the staging: [2][FL][4 dpp rows][4 rows] partial sums of this wave
+    const int b = lane >> 2, j = lane & 3;
+    const int k = a.k, chunks = k >> 6;
+    const int n = a.n[0] + a.n[1] + a.n[2];
+    const int groups = (n + 3) >> 2;
+    const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
+    const bool inrow = wave * 16 + b < chunks;      // lanes past the end of the row: zero activations
+    const int c = inrow ? wave * 16 + b : chunks - 1;
+    const typename U::Off off = U::offsets(c, (uint32_t)j * (uint32_t)rowbytes);
+    const int turns = (groups + nblocks - 1) / nblocks;  // row groups this workgroup takes (the last may be missing)
+    const int vturns = DUAL ? 2 * turns : turns;         // DUAL: a group's gate rows, then its up rows
+
+    // ---- the activations this lane stages: 16 values of chunk c
+    const int xf = U::x_first(c, j);
+    float4 xv[4], nv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        xv[i] = inrow ? reinterpret_cast<const float4 *>(a.x + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (NORM) nv[i] = inrow ? reinterpret_cast<const float4 *>(a.nw + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    // ---- the ring of weight bytes
+    typename U::Raw buf[NB];
+    // A turn's row group g holds the rows min(4 g, n - 4) ... + 3 (the last group of a row count that is no multiple of four
+    // overlaps its neighbour; the flush skips the rows it shares).  Group, segment and byte offset are wave-uniform: scalar
+    // arithmetic, and no branch - with conditional loads the compiler cannot count the loads in flight.
+    // (the segment's matrix by differences: a choice among three pointers by two conditions gets compiled into a table in
+    // private memory)
+    const uint8_t *const w0 = a.w[0], *const wd = a.w2;
+    const ptrdiff_t d01 = a.w[1] - a.w[0], d12 = a.w[2] - a.w[1];
+    const int n0 = a.n[0], n01 = a.n[0] + a.n[1];
+    auto fill = [&](typename U::Raw &dst, int t) {
+        const int g = bid + (DUAL ? t >> 1 : t) * nblocks;
+        // extent of the descriptor: everything for a group that exists, nothing past the last group (turns at or past
+        // vturns are past it too) - by arithmetic, so that the descriptor stays in scalar registers
+        // (read back through a scalar lane: as a plain select feeding the descriptor it is built in vector registers, and every
+        // load then runs in a loop over the descriptor values the lanes hold)
+        const int extent = __builtin_amdgcn_readfirstlane((g - groups) >> 31);
+        const int r0 = min(4 * g, n - 4);
+        const bool in1 = r0 >= n0, in2 = r0 >= n01;
+        const uint8_t *base = w0 + (in1 ? d01 : 0) + (in2 ? d12 : 0);
+        if (DUAL) base = (t & 1) ? wd : w0;
+        const int local = r0 - (in1 ? n0 : 0) - (in2 ? n01 - n0 : 0);
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, extent, 0x00020000);
+        U::load(dst, rs, off, (uint32_t)local * (uint32_t)rowbytes);
+    };
+#pragma unroll
+    for (int i = 0; i < NB; ++i) fill(buf[i], i);
+    __builtin_amdgcn_sched_barrier(0);  // the weight loads leave before anything waits for the activations
+
+    float nscale = 1.f;
+    if (NORM) {  // x <- x * nw / sqrt(mean(x^2) + eps) (ops/RowNorm.java:286-306)
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+        for (int w = 0; w < waves; ++w) tot += red[w];
+        nscale = 1.f / sqrtf(tot / (float)k + a.eps);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            xv[i] = make_float4(xv[i].x * nscale * nv[i].x, xv[i].y * nscale * nv[i].y, xv[i].z * nscale * nv[i].z, xv[i].w * nscale * nv[i].w);
+    }
+
+    // ---- fixed point: v = rint(x * s), |v| < 2^22, s a power of two from the chunk's largest magnitude
+    uint32_t am = 0u;
+    float sm = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        am = max(max(am, max(__float_as_uint(xv[i].x) & 0x7fffffffu, __float_as_uint(xv[i].y) & 0x7fffffffu)),
+                 max(__float_as_uint(xv[i].z) & 0x7fffffffu, __float_as_uint(xv[i].w) & 0x7fffffffu));
+        sm += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+    }
+    am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+    am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+    const bool slow = __builtin_amdgcn_ballot_w64(am >= 0x7f800000u) != 0;                  // an Inf or NaN in this wave's slice
+    const uint32_t eb = max(am >> 23, 22u);
+    const float s = __uint_as_float((275u - min(eb, 254u)) << 23), sinv = __uint_as_float((min(eb, 254u) - 21u) << 23);
+    float s4[4], sums[U::NSUM];
+    s4[0] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x00, 0xF, 0xF, true));  // quad_perm [0,0,0,0]
+    s4[1] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x55, 0xF, 0xF, true));
+    s4[2] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xAA, 0xF, 0xF, true));
+    s4[3] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xFF, 0xF, 0xF, true));
+    U::sums(s4, sums);
+    uint32_t xa[16];
+    if (!slow) {
+        uint32_t pl[3][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float f[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+            uint32_t u[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) u[e] = __float_as_uint(__builtin_fmaf(f[e], s, 12582912.f)) + (0x00808080u - 0x4B400000u);
+            // bytes 0..2 of u are the digits + 128; gather byte p of the four values into one dword, then flip the top bits
+            const uint32_t t01 = __builtin_amdgcn_perm(u[1], u[0], 0x05010400u), t23 = __builtin_amdgcn_perm(u[3], u[2], 0x05010400u);
+            pl[0][i] = __builtin_amdgcn_perm(t23, t01, 0x05040100u) ^ 0x80808080u;
+            pl[1][i] = __builtin_amdgcn_perm(t23, t01, 0x07060302u) ^ 0x80808080u;
+            const uint32_t w01 = __builtin_amdgcn_perm(u[1], u[0], 0x00000602u), w23 = __builtin_amdgcn_perm(u[3], u[2], 0x00000602u);
+            pl[2][i] = __builtin_amdgcn_perm(w23, w01, 0x05040100u) ^ 0x80808080u;
+        }
+#pragma unroll
+        for (int p = 0; p < 3; ++p) planes[(b * 3 + p) * 4 + j] = u32x4{pl[p][0], pl[p][1], pl[p][2], pl[p][3]};
+        // (the LDS accesses of a wave complete in order: its reads below see its writes above without a barrier)
+        __builtin_amdgcn_wave_barrier();
+        const int p = min(j, 2);  // operand row 3 of the product is not used: lane 4b + 3 feeds plane 2 again
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            const u32x4 v = planes[(b * 3 + p) * 4 + qd];
+            xa[qd * 4 + 0] = v.x; xa[qd * 4 + 1] = v.y; xa[qd * 4 + 2] = v.z; xa[qd * 4 + 3] = v.w;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    auto group_of = [&](int t) { return bid + (DUAL ? t >> 1 : t) * nblocks; };
+    // one output of the window that started at turn t0: the partial sums of all waves in wave order
+    auto joined = [&](int half, int tt, int jj) {
+        float sum = 0.f;
+        for (int w = 0; w < waves; ++w) {
+            const float *p = reinterpret_cast<const float *>(i8_smem + (size_t)w * I8_LDS_PER_WAVE) + (half * FL + tt) * 16 + jj;
+            sum += (p[0] + p[4]) + (p[8] + p[12]);
+        }
+        return sum;
+    };
+
+    // a turn's partial sums of this wave: fold the sixteen chunks of every row (lanes 4b + j, b = 0..15) to four per row
+    auto emit = [&](float acc, int half, int tt) {
+        if (!inrow) acc = 0.f;
+        acc += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc), 0x114, 0xF, 0xF, true));  // row_shr:4
+        acc += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc), 0x118, 0xF, 0xF, true));  // row_shr:8
+        if ((lane & 15) >= 12) mypart[(half * FL + tt) * 16 + (lane >> 4) * 4 + j] = acc;
+    };
+
+    for (int t0 = 0, half = 0; t0 < vturns; t0 += FL, half ^= 1) {
+        const int tend = min(t0 + FL, vturns);
+        if (!slow) {
+#pragma unroll 1
+            for (int tb = t0; tb < tend; tb += NB) {
+#pragma unroll
+                for (int i = 0; i < NB; ++i) {
+                    const int t = tb + i;
+                    if (t < tend && group_of(t) < groups) emit(U::dot(buf[i], c, xa, sinv, sums), half, t - t0);  // wave-uniform
+                    fill(buf[i], t + NB);
+                }
+            }
+        } else {
+            // an activation of this slice is not finite: every weight by the dequantiser's own code, FP32 products, straight
+            // from memory (four values at a time, in the order the operands have them)
+#pragma unroll 1
+            for (int t = t0; t < tend; ++t) {
+                const int g = group_of(t);
+                if (g >= groups) continue;
+                const int row = min(4 * g, n - 4) + j;
+                const bool in1 = row >= n0, in2 = row >= n01;
+                const uint8_t *rp = (DUAL ? ((t & 1) ? wd : w0) : w0 + (in1 ? d01 : 0) + (in2 ? d12 : 0)) +
+                                    (size_t)(row - (in1 ? n0 : 0) - (in2 ? n01 - n0 : 0)) * rowbytes;
+                float acc = 0.f;
+#pragma unroll 1
+                for (int e = 0; e < 64; e += 4) {
+                    const int p = U::x_pos(c, e);
+                    const float4 w4 = dequant4<FMT>(rp, (size_t)p);
+                    float4 x4 = *reinterpret_cast<const float4 *>(a.x + p);
+                    if (NORM) {
+                        const float4 n4 = *reinterpret_cast<const float4 *>(a.nw + p);
+                        x4 = make_float4(x4.x * nscale * n4.x, x4.y * nscale * n4.y, x4.z * nscale * n4.z, x4.w * nscale * n4.w);
+                    }
+                    acc = __builtin_fmaf(w4.x, x4.x, acc);
+                    acc = __builtin_fmaf(w4.y, x4.y, acc);
+                    acc = __builtin_fmaf(w4.z, x4.z, acc);
+                    acc = __builtin_fmaf(w4.w, x4.w, acc);
+                }
+                emit(acc, half, t - t0);
+            }
+        }
+        __syncthreads();  // (one barrier per window: the next window writes the other half of the partial-sum area)
+        const int outs = DUAL ? 2 * (tend - t0) : 4 * (tend - t0);
+        for (int o = tid; o < outs; o += (int)blockDim.x) {  // (a one-wave workgroup has fewer threads than a window has outputs)
+            if (DUAL) {
+                const int pr = o >> 2, jj = o & 3;
+                const int g = group_of(t0 + 2 * pr), row = min(4 * g, n - 4) + jj;
+                if (g < groups && row >= 4 * g) {
+                    const float gate = joined(half, 2 * pr, jj), up = joined(half, 2 * pr + 1, jj);
+                    a.y[0][row] = (gate / (1.f + __expf(-gate))) * up;
+                }
+            } else {
+                const int tt = o >> 2, jj = o & 3;
+                const int g = group_of(t0 + tt), row = min(4 * g, n - 4) + jj;
+                if (g < groups && row >= 4 * g) {
+                    // (segment pointers by differences, as in fill: no dependent load from the argument block on the way out)
+                    const bool in1 = row >= a.n[0], in2 = row >= a.n[0] + a.n[1];
+                    const int local = row - (in1 ? a.n[0] : 0) - (in2 ? a.n[1] : 0);
+                    float *const yp = a.y[0] + (in1 ? a.y[1] - a.y[0] : 0) + (in2 ? a.y[2] - a.y[1] : 0);
+                    float bias = 0.f;
+                    if (BIAS) bias = (a.bias[0] + (in1 ? a.bias[1] - a.bias[0] : 0) + (in2 ? a.bias[2] - a.bias[1] : 0))[local];
+                    const float sum = joined(half, tt, jj);
+                    yp[local] = BIAS ? sum + bias : sum;
+                }
+            }
+        }
+    }
+}
+
+template <class U, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
+__global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_kernel(const I8Args a) {
+    gemv_i8_body<U, PF, BIAS, NORM, DUAL>(a, blockIdx.x, gridDim.x);
+}
+
+// Two sets of matrices in two formats over the same (normalised) activations in one launch - the q / k and the v
+// projections of a Q4_K_M layer: workgroups below `split` run the first set, the others the second.
+template <class UA, class UB, int PF, int MAXW>
+__global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_pair_kernel(const I8Args a, const I8Args b, const int split) {
+    if ((int)blockIdx.x < split) gemv_i8_body<UA, PF, false, true, false>(a, blockIdx.x, split);
+    else gemv_i8_body<UB, PF, false, true, false>(b, blockIdx.x - split, gridDim.x - split);
+}
+
+}  // namespace jitnn

@@ -98,6 +98,8 @@ struct State {
     bool prefill_attn_mfma = true;  // JITNN_HIP_PREFILL_ATTN_MFMA=0: the FP16 attention of long prompts on v_dot2 instead of the matrix cores
     bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
     void *scratch_ptr = nullptr;    // device address of `scratch` on g.device (hipGetSymbolAddress at init)
+    bool gemv_i8 = true;            // JITNN_HIP_GEMV_I8=0: batch-1 K-quant GEMV on the FP32 register kernels instead of the INT8 matrix-core one
+    int i8_pf = 0, i8_blocks_per_cu = 0;  // JITNN_HIP_I8_PF / JITNN_HIP_I8_BLOCKS: overrides for measurements (0 = built-in choice)
 };
 State g;
 std::mutex g_mu;
@@ -265,7 +267,65 @@ int xreg_args(const XregCall &c, XregArgs &a) {
     return n;
 }
 
+// The INT8 matrix-core kernel (gemv_i8.h) takes what the register-resident kernels take of the K-quants, and rows of up
+// to 16384 values.
+// Its row groups are four rows: at least four rows in all, and the segments of a shared launch whole groups; its buffer
+// loads address a matrix with 32 bits.
+bool i8_ok(const XregCall &c) {
+    if (!g.gemv_i8 || !gemv_i8_supported(c.w[0]->fmt, c.w[0]->k)) return false;
+    int n = 0;
+    for (int i = 0; i < 3; ++i) {
+        if (!c.w[i]) continue;
+        n += c.w[i]->n;
+        if (c.w[i]->nbytes >= (1ll << 32) || (c.w[1] && c.w[i]->n % 4 != 0)) return false;
+    }
+    if (c.w2 && c.w2->nbytes >= (1ll << 32)) return false;
+    return n >= 4;
+}
+
+int i8_args(const XregCall &c, I8Args &a) {
+    int n = 0;
+    for (int i = 0; i < 3; ++i) {
+        a.w[i] = c.w[i] ? c.w[i]->dev : c.w[0]->dev;
+        a.y[i] = c.y[i] ? c.y[i] : c.y[0];
+        a.bias[i] = c.bias;
+        a.n[i] = c.w[i] ? c.w[i]->n : 0;
+        n += a.n[i];
+    }
+    a.w2 = c.w2 ? c.w2->dev : nullptr;
+    a.x = c.x;
+    a.nw = c.norm_w;
+    a.eps = c.eps;
+    a.k = c.w[0]->k;
+    return n;
+}
+
+// workgroups and turns in flight for a launch of `groups` row groups (four rows each) of `waves`-wave workgroups
+void i8_shape(int groups, int waves, bool dual, int &blocks, int &pf) {
+    // One workgroup per CU with three turns in flight, or two with one turn in flight, measured level on 14336 x 4096
+    // (7.7 against 8.0 us); matrices of few rows want more, shorter workgroups.
+    int per_cu = waves > 8 ? 1 : waves > 4 ? 2 : groups <= 4 * g.cus ? 4 : groups <= 8 * g.cus ? 2 : 1;
+    if (g.i8_blocks_per_cu > 0) per_cu = g.i8_blocks_per_cu;
+    blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
+    const int turns = (groups + blocks - 1) / blocks * (dual ? 2 : 1);
+    pf = turns >= 8 ? 3 : turns >= 4 ? 2 : 1;
+    if (g.i8_pf > 0) pf = g.i8_pf;
+}
+
+int launch_i8(const XregCall &c, hipStream_t stream) {
+    I8Args a{};
+    const int n = i8_args(c, a);
+    const int mode = c.w2 ? I8_DUAL : c.norm_w ? I8_NORM : c.bias ? I8_BIAS : I8_PLAIN;
+    int blocks, pf;
+    i8_shape((n + 3) / 4, (a.k + 1023) / 1024, c.w2 != nullptr, blocks, pf);
+    if (c.w[0]->fmt == F_Q5_K && pf > 2) pf = 2;  // (five loads per turn: a fourth buffer does not fit 128 registers)
+    gemv_i8_launch(c.w[0]->fmt, mode, pf, (unsigned)blocks, stream, a);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
 int launch_xreg(const XregCall &c, hipStream_t stream) {
+    if (i8_ok(c) && !(c.norm_w && c.bias)) return launch_i8(c, stream);
     XregArgs a{};
     const int n = xreg_args(c, a);
     const int threads = XREG_THREADS, waves = threads / 64;
@@ -314,6 +374,23 @@ bool xreg2_ok(int fa, int fb) { return pick_xreg2_pf<1>(fa < fb ? fa : fb, fa < 
 int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
     const bool swap = c0.w[0]->fmt > c1.w[0]->fmt;
     const XregCall &ca = swap ? c1 : c0, &cb = swap ? c0 : c1;
+    if (i8_ok(ca) && i8_ok(cb) && ca.w[0]->k <= 4096 && gemv_i8_pair_supported(ca.w[0]->fmt, cb.w[0]->fmt)) {
+        I8Args a{}, b{};
+        const int ga = (i8_args(ca, a) + 3) / 4, gb = (i8_args(cb, b) + 3) / 4;
+        const double ba = (double)ga * ca.w[0]->nbytes / ca.w[0]->n, bb = (double)gb * cb.w[0]->nbytes / cb.w[0]->n;
+        int total, pf;
+        i8_shape(ga + gb, (a.k + 1023) / 1024, false, total, pf);
+        if (total < 2) total = 2;
+        int blocks_a = (int)(total * ba / (ba + bb) + 0.5);
+        if (blocks_a < 1) blocks_a = 1;
+        if (blocks_a > total - 1) blocks_a = total - 1;
+        if (blocks_a > ga) blocks_a = ga;
+        int blocks_b = total - blocks_a;
+        if (blocks_b > gb) blocks_b = gb;
+        gemv_i8_pair_launch(ca.w[0]->fmt, cb.w[0]->fmt, pf > 2 ? 2 : pf, (unsigned)blocks_a, (unsigned)blocks_b, stream, a, b);
+        HIP_TRY(hipGetLastError());
+        return JITNN_HIP_OK;
+    }
     XregArgs a{}, b{};
     const int na = xreg_args(ca, a), nb = xreg_args(cb, b);
     const int waves = XREG_THREADS / 64;
@@ -365,6 +442,14 @@ size_t ksplit_lds(int fmt, int slices) {  // the single-block units need the mos
 
 // Batch 1, rows of 4097..32768 values: one wave per 4096-value slice of the row, partial sums joined in LDS.
 int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *bias, float *y, hipStream_t stream) {
+    {
+        XregCall c;
+        c.w[0] = w;
+        c.y[0] = y;
+        c.bias = bias;
+        c.x = x;
+        if (i8_ok(c)) return launch_i8(c, stream);
+    }
     const int slices = (w->k + 4095) / 4096;
     const size_t lds = ksplit_lds(w->fmt, slices);
     int per_cu = (int)((g.lds_per_cu - 4096) / lds);  // workgroups of one CU by LDS
@@ -884,6 +969,9 @@ int jitnn_hip_init(int device_ordinal) {
         int v = atoi(e);
         if (v >= 1) g.gemv_max_rows = v;
     }
+    if (const char *e = getenv("JITNN_HIP_GEMV_I8")) g.gemv_i8 = atoi(e) != 0;
+    if (const char *e = getenv("JITNN_HIP_I8_PF")) g.i8_pf = atoi(e);
+    if (const char *e = getenv("JITNN_HIP_I8_BLOCKS")) g.i8_blocks_per_cu = atoi(e);
     if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
