@@ -158,9 +158,52 @@ struct U8<F_Q5_K> {
 // c = 4 sb + 2 n + r covers l in [16 r, 16 r + 16) of half n of super-block sb for the four k: four runs of 16 values,
 // run k at x[256 sb + 128 n + 32 k + 16 r ..], each with its own int8 scale (index 8 n + 2 k + r).  The quants come out
 // as q in 0..63; the -32 of the format meets the sums of x over the runs.
-template <>
-struct U8<F_Q6_K> {
+//
+// Blocks are 210 bytes long, so every other block of a row starts two bytes past a dword boundary - and a 16-byte load
+// from such an address runs at 70 % of the rate of a dword-aligned one (4.6 against 6.5 TB/s streaming, measured; loads of
+// 8 and 2 bytes cost more still).  U8Q6<true> (rows a multiple of 4 bytes long, i.e. K a multiple of 512, and matrices on
+// dword boundaries) therefore fetches dword-aligned windows - the lane's field minus the block's two-byte shift - and
+// shifts the fields into place with v_alignbit: the two bytes a window misses are the first two of the window that
+// follows it in memory, which a neighbouring lane of the same block holds (the fields of the four chunks of a block tile
+// ql and qh without gaps) and hands over with one DPP rotation.  U8Q6<false> loads the fields where they are.
+template <bool ALIGNED>
+struct U8Q6;
+
+struct U8Q6Base {
     static constexpr int FMT = F_Q6_K, NSUM = 4;
+    __device__ static __forceinline__ int x_first(int c, int j) { return (c >> 2) * 256 + ((c >> 1) & 1) * 128 + 32 * j + 16 * (c & 1); }
+    __device__ static __forceinline__ int x_pos(int c, int e) { return x_first(c, e >> 4) + (e & 15); }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] = -32.f * s4[i];
+    }
+    // la, lb: the lane's 16 bytes of ql at 64 n + 16 r and 32 further on; qh: its 16 bytes of qh; sa, sb: dwords whose bytes 0 and
+    // 2 are the scales of runs 0, 1 | 2, 3; d: the block scale's bits
+    __device__ static __forceinline__ float dot_fields(const u32x4 &la, const u32x4 &lb, const u32x4 &qh, uint32_t sa, uint32_t sb, uint32_t d,
+                                                       const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
+        i32x4 d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0}, d2 = {0, 0, 0, 0}, d3 = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t a = la[i], b = lb[i], h = qh[i];
+            const uint32_t v0 = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
+            const uint32_t v1 = (b & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
+            const uint32_t v2 = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
+            const uint32_t v3 = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
+            d0 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[i], (int)v0, d0, 0, 0, 0);
+            d1 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[4 + i], (int)v1, d1, 0, 0, 0);
+            d2 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + i], (int)v2, d2, 0, 0, 0);
+            d3 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[12 + i], (int)v3, d3, 0, 0, 0);
+        }
+        float acc = (float)(int)(int8_t)sa * __builtin_fmaf(i8_combine_wide(d0), sinv, s[0]);
+        acc = __builtin_fmaf((float)(int)(int8_t)(sa >> 16), __builtin_fmaf(i8_combine_wide(d1), sinv, s[1]), acc);
+        acc = __builtin_fmaf((float)(int)(int8_t)sb, __builtin_fmaf(i8_combine_wide(d2), sinv, s[2]), acc);
+        acc = __builtin_fmaf((float)(int)(int8_t)(sb >> 16), __builtin_fmaf(i8_combine_wide(d3), sinv, s[3]), acc);
+        return acc * h2f(d);
+    }
+};
+
+template <>
+struct U8Q6<false> : U8Q6Base {
     struct Raw { u32x4 la, lb, qh; u32x2 sc; uint32_t d; };
     struct Off { uint32_t la, qh, sc, d; };
     __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) {
@@ -172,8 +215,6 @@ struct U8<F_Q6_K> {
         o.d = blk + 208u;
         return o;
     }
-    __device__ static __forceinline__ int x_first(int c, int j) { return (c >> 2) * 256 + ((c >> 1) & 1) * 128 + 32 * j + 16 * (c & 1); }
-    __device__ static __forceinline__ int x_pos(int c, int e) { return x_first(c, e >> 4) + (e & 15); }
     __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
         r.la = i8_ld128(rs, o.la, soff);   // (fields on 2-byte boundaries: buffer loads take them like the global ones)
         r.lb = i8_ld128(rs, o.la + 32u, soff);
@@ -181,33 +222,59 @@ struct U8<F_Q6_K> {
         r.sc = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)o.sc, (int)soff, 0);
         r.d = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)o.d, (int)soff, 0);
     }
-    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) s[i] = -32.f * s4[i];
-    }
     __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
-        i32x4 d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0}, d2 = {0, 0, 0, 0}, d3 = {0, 0, 0, 0};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t a = r.la[i], b = r.lb[i], h = r.qh[i];
-            const uint32_t v0 = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
-            const uint32_t v1 = (b & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
-            const uint32_t v2 = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
-            const uint32_t v3 = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
-            d0 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[i], (int)v0, d0, 0, 0, 0);
-            d1 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[4 + i], (int)v1, d1, 0, 0, 0);
-            d2 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + i], (int)v2, d2, 0, 0, 0);
-            d3 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[12 + i], (int)v3, d3, 0, 0, 0);
-        }
         const int sh = (c & 1) * 8;
-        const uint32_t sa = r.sc.x >> sh, sb = r.sc.y >> sh;  // bytes 0 and 2: the scales of runs 0, 1 | 2, 3
-        float acc = (float)(int)(int8_t)sa * __builtin_fmaf(i8_combine_wide(d0), sinv, s[0]);
-        acc = __builtin_fmaf((float)(int)(int8_t)(sa >> 16), __builtin_fmaf(i8_combine_wide(d1), sinv, s[1]), acc);
-        acc = __builtin_fmaf((float)(int)(int8_t)sb, __builtin_fmaf(i8_combine_wide(d2), sinv, s[2]), acc);
-        acc = __builtin_fmaf((float)(int)(int8_t)(sb >> 16), __builtin_fmaf(i8_combine_wide(d3), sinv, s[3]), acc);
-        return acc * h2f(r.d);
+        return dot_fields(r.la, r.lb, r.qh, r.sc.x >> sh, r.sc.y >> sh, r.d, xa, sinv, s);
     }
 };
+
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+
+template <>
+struct U8Q6<true> : U8Q6Base {
+    struct Raw { u32x4 la, lb, qh; u32x3 sc; uint32_t d; };  // dword-aligned windows: the fields start `shift` bytes into them
+    struct Off { uint32_t la, qh, sc, d; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) {
+        Off o;
+        const uint32_t blk = row_off + (uint32_t)(c >> 2) * 210u, n = (uint32_t)(c >> 1) & 1u, r = (uint32_t)c & 1u;
+        const uint32_t base = blk & ~3u;  // (row_off is a multiple of 4: the shift of a block is 2 for odd sb)
+        o.la = base + 64u * n + 16u * r;
+        o.qh = base + 128u + 32u * n + 16u * r;
+        o.sc = base + 192u + 8u * n;
+        o.d = base + 208u;
+        return o;
+    }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.la = i8_ld128(rs, o.la, soff);
+        r.lb = i8_ld128(rs, o.la + 32u, soff);
+        r.qh = i8_ld128(rs, o.qh, soff);
+        r.sc = __builtin_amdgcn_raw_buffer_load_b96(rs, (int)o.sc, (int)soff, 0);
+        r.d = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, (int)o.d, (int)soff, 0);
+    }
+    // the first dword of the lane 4 further on / 4 back in its row of 16 lanes (the next / previous chunk of the block, same weight row)
+    __device__ static __forceinline__ uint32_t next4(uint32_t v) { return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x12C, 0xF, 0xF, false); }  // row_ror:12
+    __device__ static __forceinline__ uint32_t prev4(uint32_t v) { return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x124, 0xF, 0xF, false); }  // row_ror:4
+    __device__ static __forceinline__ u32x4 shifted(const u32x4 &w, uint32_t after, uint32_t sh) {
+        return u32x4{__builtin_amdgcn_alignbit(w.y, w.x, sh), __builtin_amdgcn_alignbit(w.z, w.y, sh), __builtin_amdgcn_alignbit(w.w, w.z, sh),
+                     __builtin_amdgcn_alignbit(after, w.w, sh)};
+    }
+    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
+        const uint32_t sh = (uint32_t)((c >> 2) & 1) * 16u;  // bits the block's fields sit past their windows' starts
+        const bool r0 = (c & 1) == 0, n0 = (c & 2) == 0, last = (c & 3) == 3;
+        // In memory the windows of a block follow one another as la(b0) la(b1) lb(b0) lb(b1) la(b2) la(b3) lb(b2) lb(b3) qh(b0..b3)
+        // scales (b = chunk of the block): the dword after a window is the first dword of the next one.
+        const uint32_t nla = next4(r.la.x), nlb = next4(r.lb.x), nqh = next4(r.qh.x), nsc = next4(r.sc.x), plb = prev4(r.lb.x);
+        const u32x4 la = shifted(r.la, r0 ? nla : plb, sh);
+        const u32x4 lb = shifted(r.lb, r0 ? nlb : n0 ? nla : nqh, sh);
+        const u32x4 qh = shifted(r.qh, last ? nsc : nqh, sh);
+        const uint32_t sx = __builtin_amdgcn_alignbit(r.sc.y, r.sc.x, sh), sy = __builtin_amdgcn_alignbit(r.sc.z, r.sc.y, sh);
+        const int s8 = (c & 1) * 8;
+        return dot_fields(la, lb, qh, sx >> s8, sy >> s8, r.d >> sh, xa, sinv, s);
+    }
+};
+
+template <>
+struct U8<F_Q6_K> : U8Q6<false> {};
 
 // -------------------------------------------------------------------------------------------------- the kernel body
 template <class U, int PF, bool BIAS, bool NORM, bool DUAL>
@@ -269,20 +336,18 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
     for (int i = 0; i < NB; ++i) fill(buf[i], i);
     __builtin_amdgcn_sched_barrier(0);  // the weight loads leave before anything waits for the activations
 
-    float nscale = 1.f;
-    if (NORM) {  // x <- x * nw / sqrt(mean(x^2) + eps) (ops/RowNorm.java:286-306)
+    if (NORM) {
+        // RMSNorm (ops/RowNorm.java:286-306): y = W (x * nw / sqrt(mean(x^2) + eps)).  The factor 1 / sqrt(...) is one number for the
+        // whole vector, so it multiplies the outputs instead of the inputs: the activations go to fixed point as x * nw without
+        // waiting for a workgroup-wide reduction, and the sum of squares (one partial per wave, in LDS) is only read after the
+        // barrier that precedes the first outputs anyway.
         float ss = 0.f;
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
         ss = wave_sum(ss);
         if (lane == 0) red[wave] = ss;
-        __syncthreads();
-        float tot = 0.f;
-        for (int w = 0; w < waves; ++w) tot += red[w];
-        nscale = 1.f / sqrtf(tot / (float)k + a.eps);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            xv[i] = make_float4(xv[i].x * nscale * nv[i].x, xv[i].y * nscale * nv[i].y, xv[i].z * nscale * nv[i].z, xv[i].w * nscale * nv[i].w);
+        for (int i = 0; i < 4; ++i) xv[i] = make_float4(xv[i].x * nv[i].x, xv[i].y * nv[i].y, xv[i].z * nv[i].z, xv[i].w * nv[i].w);
     }
 
     // ---- fixed point: v = rint(x * s), |v| < 2^22, s a power of two from the chunk's largest magnitude
@@ -384,7 +449,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
                     float4 x4 = *reinterpret_cast<const float4 *>(a.x + p);
                     if (NORM) {
                         const float4 n4 = *reinterpret_cast<const float4 *>(a.nw + p);
-                        x4 = make_float4(x4.x * nscale * n4.x, x4.y * nscale * n4.y, x4.z * nscale * n4.z, x4.w * nscale * n4.w);
+                        x4 = make_float4(x4.x * n4.x, x4.y * n4.y, x4.z * n4.z, x4.w * n4.w);
                     }
                     acc = __builtin_fmaf(w4.x, x4.x, acc);
                     acc = __builtin_fmaf(w4.y, x4.y, acc);
@@ -395,13 +460,19 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
             }
         }
         __syncthreads();  // (one barrier per window: the next window writes the other half of the partial-sum area)
+        float nscale = 1.f;
+        if (NORM) {
+            float tot = 0.f;
+            for (int w = 0; w < waves; ++w) tot += red[w];
+            nscale = 1.f / sqrtf(tot / (float)k + a.eps);
+        }
         const int outs = DUAL ? 2 * (tend - t0) : 4 * (tend - t0);
         for (int o = tid; o < outs; o += (int)blockDim.x) {  // (a one-wave workgroup has fewer threads than a window has outputs)
             if (DUAL) {
                 const int pr = o >> 2, jj = o & 3;
                 const int g = group_of(t0 + 2 * pr), row = min(4 * g, n - 4) + jj;
                 if (g < groups && row >= 4 * g) {
-                    const float gate = joined(half, 2 * pr, jj), up = joined(half, 2 * pr + 1, jj);
+                    const float gate = joined(half, 2 * pr, jj) * nscale, up = joined(half, 2 * pr + 1, jj) * nscale;
                     a.y[0][row] = (gate / (1.f + __expf(-gate))) * up;
                 }
             } else {
@@ -414,7 +485,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
                     float *const yp = a.y[0] + (in1 ? a.y[1] - a.y[0] : 0) + (in2 ? a.y[2] - a.y[1] : 0);
                     float bias = 0.f;
                     if (BIAS) bias = (a.bias[0] + (in1 ? a.bias[1] - a.bias[0] : 0) + (in2 ? a.bias[2] - a.bias[1] : 0))[local];
-                    const float sum = joined(half, tt, jj);
+                    const float sum = NORM ? joined(half, tt, jj) * nscale : joined(half, tt, jj);
                     yp[local] = BIAS ? sum + bias : sum;
                 }
             }

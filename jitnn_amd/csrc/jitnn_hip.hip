@@ -302,14 +302,16 @@ int i8_args(const XregCall &c, I8Args &a) {
 
 // workgroups and turns in flight for a launch of `groups` row groups (four rows each) of `waves`-wave workgroups
 void i8_shape(int groups, int waves, bool dual, int &blocks, int &pf) {
-    // One workgroup per CU with three turns in flight, or two with one turn in flight, measured level on 14336 x 4096
-    // (7.7 against 8.0 us); matrices of few rows want more, shorter workgroups.
-    int per_cu = waves > 8 ? 1 : waves > 4 ? 2 : groups <= 4 * g.cus ? 4 : groups <= 8 * g.cus ? 2 : 1;
+    // Measured (us, pf / workgroups per CU): Q4_K 14336 x 4096 8.40 (1/2) 8.44 (2/1) 8.48 (3/1) 9.54 (1/4); Q4_K 4096 x 4096 4.75 (1/2)
+    // 4.93 (1/1) 5.82 (1/4); Q6_K 128256 x 4096 71.9 (2/1) 72.9 (3/1) 73.6 (1/1) 74.5 (1/2); Q6_K 4096 x 14336 (14 waves) 12.9
+    // (1/1) 14.3 (2/1) 16.2 (1/2).  Tall matrices: one workgroup per CU with two turns in flight behind the one being
+    // multiplied; short ones: two workgroups with one; long rows: one with one.
+    const int turns1 = (groups + g.cus - 1) / g.cus;
+    int per_cu = waves > 4 ? 1 : turns1 >= 8 ? 1 : 2;
+    pf = waves > 4 ? 1 : turns1 >= 8 ? (dual ? 3 : 2) : 1;  // (gate + up of an 8B layer: 14.4 us with three turns in flight, 15.1 with two)
     if (g.i8_blocks_per_cu > 0) per_cu = g.i8_blocks_per_cu;
-    blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
-    const int turns = (groups + blocks - 1) / blocks * (dual ? 2 : 1);
-    pf = turns >= 8 ? 3 : turns >= 4 ? 2 : 1;
     if (g.i8_pf > 0) pf = g.i8_pf;
+    blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
 }
 
 int launch_i8(const XregCall &c, hipStream_t stream) {
