@@ -280,7 +280,8 @@ JITNN_HIP_API int jitnn_hip_llama_set_rope_interleaved(jitnn_hip_llama *m, int i
  * to HBM as it is; a token's embedding is its row, dequantised bit-exactly (F.embedding on the dequantised table). */
 JITNN_HIP_API int jitnn_hip_llama_set_embedding(jitnn_hip_llama *m, int ggml_type, const void *table_host, long long nbytes);
 
-/* x [count, d_model] = embedding rows of `count` token ids in device memory. */
+/* x [count, d_model] = embedding rows of `count` token ids in device memory.  The ids are the caller's: one outside
+ * [0, vocab) reads nothing and gives a row of NaN. */
 JITNN_HIP_API int jitnn_hip_llama_embed_dev(jitnn_hip_llama *m, const int *tokens_dev, int count, float *x_dev, void *stream);
 
 /* *token_dev = index of the largest of the model's `vocab` logits (the lowest index among equal ones). */

@@ -173,12 +173,19 @@ __global__ void __launch_bounds__(256) dequant_kernel(const uint8_t *__restrict_
 }
 
 // Rows token[t] of a block-quantised table [vocab, k], dequantised bit-exactly into x [tokens, k] (the embedding lookup of
-// a model whose token table is quantised).  grid = tokens.
+// a model whose token table is quantised).  grid = tokens.  An id outside [0, vocab) reads nothing: its row is NaN.
 template <int FMT>
-__global__ void __launch_bounds__(256) dequant_rows_kernel(const uint8_t *__restrict__ w, const int *__restrict__ tokens, float *__restrict__ x, int k) {
+__global__ void __launch_bounds__(256) dequant_rows_kernel(const uint8_t *__restrict__ w, const int *__restrict__ tokens, float *__restrict__ x, int k,
+                                                            int vocab) {
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
-    const uint8_t *wr = w + (size_t)tokens[blockIdx.x] * rowbytes;
+    const int id = tokens[blockIdx.x];
     float4 *xr = reinterpret_cast<float4 *>(x + (size_t)blockIdx.x * k);
+    if (id < 0 || id >= vocab) {
+        const float nan = __builtin_nanf("");
+        for (int f = threadIdx.x; f < (k >> 2); f += 256) xr[f] = make_float4(nan, nan, nan, nan);
+        return;
+    }
+    const uint8_t *wr = w + (size_t)id * rowbytes;
     for (int f = threadIdx.x; f < (k >> 2); f += 256) xr[f] = dequant4<FMT>(wr, (size_t)f * 4);
 }
 

@@ -921,11 +921,16 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const float *__restrict__ 
 }
 
 // x[t, :] = row token[t] of an unquantised embedding table [vocab, d] (F32: fmt 0, F16: fmt 1); block-quantised tables go
-// through dequant_rows_kernel.  grid = tokens.
+// through dequant_rows_kernel.  grid = tokens.  An id outside [0, vocab) reads nothing: its row is NaN.
 __global__ void __launch_bounds__(256) embed_plain_rows_kernel(const void *__restrict__ table, int fmt, const int *__restrict__ tokens, float *__restrict__ x,
-                                                                int d) {
+                                                                int d, int vocab) {
     const int t = blockIdx.x;
-    const size_t row = (size_t)tokens[t] * d;
+    const int id = tokens[t];
+    if (id < 0 || id >= vocab) {
+        for (int i = threadIdx.x; i < d; i += 256) x[(size_t)t * d + i] = __builtin_nanf("");
+        return;
+    }
+    const size_t row = (size_t)id * d;
     for (int i = threadIdx.x; i < d; i += 256)
         x[(size_t)t * d + i] = fmt == 0 ? reinterpret_cast<const float *>(table)[row + i]
                                         : __half2float(reinterpret_cast<const __half *>(table)[row + i]);

@@ -576,6 +576,7 @@ thread_local Workspace g_ws;
 // Where a many-row launch takes its scratch from: the calling thread's grow-only buffer (may allocate), or the
 // library's static array (never allocates; the caller keeps calls on one GPU from overlapping).
 enum ScratchSource { SCRATCH_THREAD, SCRATCH_STATIC };
+void touch_thread_state();  // registers the calling thread's clean-up (defined below ThreadState)
 
 int workspace(size_t bytes, hipStream_t stream, void **out, ScratchSource src = SCRATCH_THREAD) {
     if (src == SCRATCH_STATIC) {
@@ -586,6 +587,7 @@ int workspace(size_t bytes, hipStream_t stream, void **out, ScratchSource src = 
         return JITNN_HIP_OK;
     }
     Workspace &w = g_ws;
+    touch_thread_state();  // a thread that only ever calls the device-pointer entry points must give its scratch back too
     if (!w.ev) HIP_TRY(hipEventCreateWithFlags(&w.ev, hipEventDisableTiming));
     if (bytes > w.cap) {
         if (w.ptr) HIP_TRY(hipFree(w.ptr));  // waits for the device: nobody is still reading the old block
@@ -655,6 +657,7 @@ struct ThreadState {
 };
 thread_local ThreadState g_thread;
 bool calling_thread_is_main();
+void touch_thread_state() { g_thread.is_main = calling_thread_is_main(); }
 
 int stage_reserve(size_t pinned_bytes, size_t dev_bytes) {
     HostStage &st = g_thread.stage;
@@ -1982,17 +1985,17 @@ int jitnn_hip_llama_embed_dev(jitnn_hip_llama *m, const int *tokens_dev, int cou
     const dim3 grid((unsigned)count), block(256);
     switch (m->embd_fmt) {
     case 0:
-    case 1: hipLaunchKernelGGL(embed_plain_rows_kernel, grid, block, 0, st, (const void *)m->embd, m->embd_fmt, tokens_dev, x_dev, m->d); break;
-    case F_Q4_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q4_1: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_1>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q5_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q5_1: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_1>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q8_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q8_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q2_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q2_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q3_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q3_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q4_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    case F_Q5_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
-    default: hipLaunchKernelGGL(dequant_rows_kernel<F_Q6_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d); break;
+    case 1: hipLaunchKernelGGL(embed_plain_rows_kernel, grid, block, 0, st, (const void *)m->embd, m->embd_fmt, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q4_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q4_1: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_1>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q5_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q5_1: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_1>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q8_0: hipLaunchKernelGGL(dequant_rows_kernel<F_Q8_0>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q2_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q2_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q3_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q3_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q4_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q4_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    case F_Q5_K: hipLaunchKernelGGL(dequant_rows_kernel<F_Q5_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
+    default: hipLaunchKernelGGL(dequant_rows_kernel<F_Q6_K>, grid, block, 0, st, m->embd, tokens_dev, x_dev, m->d, m->vocab); break;
     }
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;

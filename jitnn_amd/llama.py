@@ -95,6 +95,8 @@ class LlamaDecoder:
     def embed(self, tokens) -> np.ndarray:
         """Embedding rows [count, d_model] of token ids (through device memory; for tests)."""
         ids = np.ascontiguousarray(tokens, dtype=np.int32).reshape(-1)
+        if ids.size and (ids.min() < 0 or ids.max() >= self.cfg["vocab"]):
+            raise ValueError(f"token id outside [0, {self.cfg['vocab']})")
         n, d = ids.size, self.cfg["d_model"]
         dev_ids, dev_x = C.c_void_p(), C.c_void_p()
         _lib.check(_lib.lib.jitnn_hip_malloc(ids.nbytes, C.byref(dev_ids)), "jitnn_hip_malloc")

@@ -131,6 +131,38 @@ def test_two_host_threads_two_streams(jn, rows):
         assert torch.equal(got[t], alone[t]), t
 
 
+def test_worker_thread_gives_its_scratch_back(jn):
+    """A thread that only ever calls a device-pointer entry point (here one 512-row linear, which takes the thread's
+    many-row scratch: 16 MiB of FP16 operands and more) returns that scratch when it ends: six such threads one after the
+    other leave the free device memory where the first left it - a thread that kept its scratch would cost 16 MiB each.
+    (The bar leaves room for one pool block the HIP runtime may take for itself along the way.)"""
+    rng = np.random.default_rng(21)
+    n, k, rows = 64, 16384, 512
+    w = jn.Tensor.quantized(jn.DType.Q4_K, random_valid_blocks(rng, "Q4_K", n, k), n, k)
+    x = torch.randn(rows, k, device="cuda", generator=torch.Generator(device="cuda").manual_seed(4))
+    y = torch.empty(rows, n, device="cuda")
+    s = torch.cuda.Stream()
+    errors = []
+
+    def work():
+        try:
+            linear_dev(jn, w, x, y, s)
+            s.synchronize()
+        except Exception as e:  # surfaced below
+            errors.append(e)
+
+    def once():
+        th = threading.Thread(target=work)
+        th.start()
+        th.join()
+        torch.cuda.synchronize()
+        return torch.cuda.mem_get_info()[0]
+
+    free = [once() for _ in range(7)]   # (one-off allocations of the runtime happen in the first)
+    assert not errors, errors
+    assert free[1] - free[6] < (12 << 20), free
+
+
 def test_one_thread_alternating_streams_many_rows(jn):
     """One host thread feeding the many-row path from two streams in turn: the second stream's call waits for the first
     one's use of the thread's scratch instead of overwriting it."""
@@ -171,6 +203,11 @@ def test_non_finite_activations(jn, fmt, rows):
         ref = oracle.gguf_linear(GGML_ID[fmt], bad, raw, None, n, k)
     y = jn.Gguf.linear(jn.Tensor.of(bad), w, None).numpy()
     assert not np.isfinite(ref[0]).any() and not np.isfinite(y[0]).any()
+    if rows == 1 and fmt in ("Q4_K", "Q5_K", "Q6_K"):
+        # the batch-1 kernel of the K-quants multiplies a slice that holds a non-finite activation weight by weight in FP32:
+        # +Inf, -Inf and NaN fall where the reference's FP64 sum has them
+        assert np.array_equal(np.isnan(y[0]), np.isnan(ref[0])), fmt
+        assert np.array_equal(np.isposinf(y[0]), np.isposinf(ref[0])) and np.array_equal(np.isneginf(y[0]), np.isneginf(ref[0])), fmt
     if rows > 1:
         assert np.isnan(ref[rows - 1]).all() and np.isnan(y[rows - 1]).all()
     bar = 1e-4 if rows <= 64 else 2e-3

@@ -298,6 +298,44 @@ def test_argmax_kernel_ties_and_nan():
     dec.close()
 
 
+@pytest.mark.gpu
+def test_embedding_ids_outside_the_vocabulary():
+    """jitnn_hip_llama_embed_dev takes its ids from the caller's device memory: an id below 0 or at / past the vocabulary reads
+    nothing and gives a row of NaN (both table kinds), the rows of the valid ids beside it are right; the host mirror
+    refuses such ids before anything is launched."""
+    import ctypes as C
+    import jitnn_amd
+    from jitnn_amd import _lib
+    vocab, d = 300, 256
+    rng = np.random.default_rng(8)
+    table = rng.standard_normal((vocab, d)).astype(np.float32)
+    for fmt in ("F32", "Q8_0"):
+        dec = jitnn_amd.LlamaDecoder(1, d, 4, 2, 64, 512, vocab, 8)
+        if fmt == "F32":
+            dec.set_embedding(0, table)
+            want = table
+        else:
+            from oracle import oracle
+            raw = oracle.quantize_q8_0(table.reshape(-1))
+            dec.set_embedding(GGML_ID["Q8_0"], raw)
+            want = oracle.dequantize(GGML_ID["Q8_0"], raw, vocab * d).reshape(vocab, d)
+        with pytest.raises(ValueError):
+            dec.embed([0, -1])
+        with pytest.raises(ValueError):
+            dec.embed([vocab])
+        ids = torch.tensor([5, -1, vocab - 1, vocab, 2 ** 31 - 1, 0], dtype=torch.int32, device="cuda")
+        x = torch.zeros(ids.numel(), d, device="cuda")
+        _lib.check(_lib.lib.jitnn_hip_llama_embed_dev(dec.handle, C.c_void_p(ids.data_ptr()), ids.numel(), C.c_void_p(x.data_ptr()), None), "embed")
+        torch.cuda.synchronize()
+        got = x.cpu().numpy()
+        for row, i in enumerate(ids.tolist()):
+            if 0 <= i < vocab:
+                assert np.array_equal(got[row], want[i]), (fmt, i)
+            else:
+                assert np.isnan(got[row]).all(), (fmt, i)
+        dec.close()
+
+
 def test_generate_argument_checks():
     pytest.importorskip("torch")
     import jitnn_amd

@@ -140,6 +140,28 @@ def test_quantize_q8_0_invariants():
     assert np.abs(dq.reshape(-1) - x).max() <= scale * (1 / 127.0) + 1e-6
 
 
+def test_quantize_q8_0_ties_round_half_away_from_zero_literals():
+    """Quant.java:113-114 rounds s = x / d half away from zero (Math.round on the magnitude, sign restored) and clamps to +-127.
+    A block whose largest magnitude is 127 has d = (float)(127 / 127.0) = 1, so the quotients are the inputs themselves: the
+    expected bytes below are written out as numbers, not recomputed.  Round-half-even would give 0, 2, 2 for 0.5, 1.5, 2.5
+    and 126 for 126.5."""
+    x = np.zeros(64, dtype=np.float32)
+    x[:9] = [127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, -126.5]
+    x[32:41] = [-127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, -126.5]   # the same with the maximum on the negative side
+    q = oracle.quantize_q8_0(x).reshape(2, 34)
+    for b in range(2):
+        assert q[b, :2].copy().view(np.float16)[0] == np.float16(1.0)
+        qs = q[b, 2:].view(np.int8)
+        assert qs[0] == (127 if b == 0 else -127)
+        assert list(qs[1:9]) == [1, 2, 3, -1, -2, -3, 127, -127]
+        assert not qs[9:].any()
+    # one float below / above a tie falls to the nearer integer
+    y = np.zeros(32, dtype=np.float32)
+    y[:5] = [127.0, np.nextafter(np.float32(2.5), np.float32(0)), np.nextafter(np.float32(2.5), np.float32(3)),
+             np.nextafter(np.float32(-0.5), np.float32(0)), np.nextafter(np.float32(-0.5), np.float32(-1))]
+    assert list(oracle.quantize_q8_0(y).reshape(34)[2:].view(np.int8)[:5]) == [127, 2, 3, 0, -1]
+
+
 def test_cpu_dequant_gemm_baseline_agrees_with_the_oracle():
     """The C restatement of the reference's dequantise + GEMM branch (the CPU baseline of the many-row configurations)
     against the FP64 oracle on the same blocks: equal within FP32 rounding of a K-blocked FMA sum, at ragged sizes (edge

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import random_valid_blocks
+from helpers import GGML_ID, norm_err, random_valid_blocks
 
 pytestmark = pytest.mark.gpu
 
@@ -54,6 +54,46 @@ def test_noalloc_linear_matches_linear_dev(jn):
         assert torch.equal(got, ref), (fmt, n, k, rows)
         again = run(lib, "jitnn_hip_linear_noalloc_dev", w, x, bias, n)
         assert torch.equal(again, ref), (fmt, n, k, rows, "second call")
+
+
+def test_noalloc_linear_against_the_oracle_without_allocating_and_under_graph_replay(jn):
+    """The entry point against the CPU oracle (not only against its sibling), the property it exists for - a first-ever
+    call of a size no earlier call of this process has had leaves the free device memory where it was -, and a many-row
+    call captured into a HIP graph: every replay, with eager work between the replays, equals the eager result."""
+    from jitnn_amd import _lib as lib
+    from oracle import oracle
+    rng = np.random.default_rng(14)
+    g = torch.Generator(device="cuda").manual_seed(14)
+    n, k, rows = 1536, 5120, 600   # (a size no other test of the suite uses)
+    raw = random_valid_blocks(rng, "Q4_K", n, k)
+    w = jn.Tensor.quantized(jn.DType.Q4_K, raw, n, k)
+    x = torch.randn(rows, k, device="cuda", generator=g)
+    y = torch.full((rows, n), float("nan"), device="cuda")
+    st = torch.cuda.current_stream()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    lib.check(lib.lib.jitnn_hip_linear_noalloc_dev(w.handle, vp(x), rows, None, vp(y), C.c_void_p(st.cuda_stream)), "noalloc")
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    sel = np.unique(np.linspace(0, rows - 1, 24).astype(np.int64))
+    ref = oracle.gguf_linear(GGML_ID["Q4_K"], x[torch.as_tensor(sel, device="cuda")].cpu().numpy(), raw, None, n, k)
+    assert norm_err(y.cpu().numpy()[sel], ref) <= 2e-3   # (more than 64 rows: the FP16 matrix-core path's bar)
+    eager = y.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(st)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        y.fill_(0)
+        with torch.cuda.graph(graph, stream=side):
+            lib.check(lib.lib.jitnn_hip_linear_noalloc_dev(w.handle, vp(x), rows, None, vp(y), C.c_void_p(side.cuda_stream)), "noalloc (capture)")
+    torch.cuda.synchronize()
+    for i in range(3):
+        y.fill_(float(i))                      # eager work between the replays
+        small = run(lib, "jitnn_hip_linear_noalloc_dev", w, x[:40].contiguous(), None, n)   # the scratch is used by another call in between
+        assert torch.isfinite(small).all()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), i
 
 
 def test_noalloc_linear_rejects_what_does_not_fit(jn):
