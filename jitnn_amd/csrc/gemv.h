@@ -299,92 +299,6 @@ struct Unit<F_Q6_K> {
             }
         }
     }
-
-    // ---- integer variant (CV == 2), for launches in which a wave sees many rows.
-    // The lane's 64 activations become 22-bit fixed point with a power-of-two step of the lane's own (taken from the
-    // exponent of their largest magnitude), cut into three byte planes: x = (b2 * 65536 + b1 * 256 + b0) * step with
-    // b2 signed, b1 and b0 unsigned.  A row then costs twelve v_dot4 per 16-value run instead of sixteen conversions
-    // and sixteen multiply-adds; the sums are exact integers, so the only error is the rounding of x to 2^-21 of the
-    // largest activation of the lane's unit (the FP32 variant rounds every product to 2^-24).
-    struct XInt {
-        uint32_t p0[16], p1[16];  // quad g of the unit: the four low / middle bytes
-        int p2[16];               // the four high bytes (signed)
-        float si[4];              // sum of the fixed-point values of run k
-        float step;               // value of one step; NaN when an activation is not finite
-    };
-    __device__ static __forceinline__ void to_fixed(const XReg<16, 4> &xs, XInt &xi) {
-        float m = 0.f;
-#pragma unroll
-        for (int g = 0; g < 16; ++g)
-            m = fmaxf(m, fmaxf(fmaxf(fabsf(xs.x[g].x), fabsf(xs.x[g].y)), fmaxf(fabsf(xs.x[g].z), fabsf(xs.x[g].w))));
-        const uint32_t be = __float_as_uint(m) >> 23;  // biased exponent: 2^(be-127) <= m < 2^(be-126)
-        const bool live = be >= 21u && be < 255u;      // smaller: the lane's activations are below 2^-106 and dropped
-        const float inv = live ? __uint_as_float((274u - be) << 23) : 0.f;   // 2^(20 - E): |x * inv| < 2^21
-        const float poison = ((xs.sm[0] + xs.sm[1]) + (xs.sm[2] + xs.sm[3])) * 0.f;  // NaN if any activation is Inf or NaN
-        xi.step = (live ? __uint_as_float((be - 20u) << 23) : 0.f) + poison;
-#pragma unroll
-        for (int g = 0; g < 16; ++g) {
-            // 1.5 * 2^23 + v (round to nearest even): mantissa bits 0..21 are v modulo 2^22, bit 22 is set for v >= 0
-            const uint32_t w0 = __float_as_uint(__builtin_fmaf(xs.x[g].x, inv, 12582912.f));
-            const uint32_t w1 = __float_as_uint(__builtin_fmaf(xs.x[g].y, inv, 12582912.f));
-            const uint32_t w2 = __float_as_uint(__builtin_fmaf(xs.x[g].z, inv, 12582912.f));
-            const uint32_t w3 = __float_as_uint(__builtin_fmaf(xs.x[g].w, inv, 12582912.f));
-            // v_perm_b32: selector bytes 0..3 pick from the second operand, 4..7 from the first
-            const uint32_t t01 = __builtin_amdgcn_perm(w1, w0, 0x05010400u);  // w0.b0 w1.b0 w0.b1 w1.b1
-            const uint32_t t23 = __builtin_amdgcn_perm(w3, w2, 0x05010400u);
-            const uint32_t u01 = __builtin_amdgcn_perm(w1, w0, 0x00000602u);  // w0.b2 w1.b2 - -
-            const uint32_t u23 = __builtin_amdgcn_perm(w3, w2, 0x00000602u);
-            xi.p0[g] = __builtin_amdgcn_perm(t23, t01, 0x05040100u);
-            xi.p1[g] = __builtin_amdgcn_perm(t23, t01, 0x07060302u);
-            // bits 16..23 of the word are 0x40 + (v >> 16): take the 0x40 off and extend the sign from bit 6
-            uint32_t hb = __builtin_amdgcn_perm(u23, u01, 0x05040100u) ^ 0x40404040u;
-            hb |= (hb & 0x40404040u) << 1;
-            xi.p2[g] = (int)hb;
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            uint32_t s0 = 0, s1 = 0;
-            int s2 = 0;
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                s0 = __builtin_amdgcn_udot4(xi.p0[4 * k + p], 0x01010101u, s0, false);
-                s1 = __builtin_amdgcn_udot4(xi.p1[4 * k + p], 0x01010101u, s1, false);
-                s2 = __builtin_amdgcn_sdot4(xi.p2[4 * k + p], 0x01010101, s2, false);
-            }
-            xi.si[k] = __builtin_fmaf((float)s2, 65536.f, __builtin_fmaf((float)s1, 256.f, (float)s0));
-        }
-    }
-    // one row's partial sum of the lane's unit, already in activation units
-    __device__ static __forceinline__ float dot_int(const Raw &w, int u, const XInt &xi) {
-        uint32_t a0[4] = {0, 0, 0, 0}, a1[4] = {0, 0, 0, 0};
-        int a2[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const uint32_t a = w.ql0[p], c = w.ql1[p], h = w.qh[p];
-            uint32_t q[4];
-            q[0] = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
-            q[1] = (c & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
-            q[2] = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
-            q[3] = ((c >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                a0[k] = __builtin_amdgcn_udot4(q[k], xi.p0[4 * k + p], a0[k], false);
-                a1[k] = __builtin_amdgcn_udot4(q[k], xi.p1[4 * k + p], a1[k], false);
-                a2[k] = __builtin_amdgcn_sdot4((int)q[k], xi.p2[4 * k + p], a2[k], false);
-            }
-        }
-        const int sh = (u & 1) * 8;
-        const float d = h2f(w.d);
-        const float cs[4] = {(float)(int)(int8_t)(w.sc.x >> sh), (float)(int)(int8_t)(w.sc.x >> (sh + 16)),
-                             (float)(int)(int8_t)(w.sc.y >> sh), (float)(int)(int8_t)(w.sc.y >> (sh + 16))};
-        float t = 0.f;
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const float f = __builtin_fmaf((float)a2[k], 65536.f, __builtin_fmaf((float)a1[k], 256.f, (float)a0[k]));
-            t = __builtin_fmaf(cs[k], __builtin_fmaf(-32.f, xi.si[k], f), t);
-        }
-        return (d * t) * xi.step;
-    }
 };
 
 // ---------------------------------------------------------------------------------------------- Q4_0
@@ -728,13 +642,6 @@ __device__ __forceinline__ void step_priority(int left) {
 
 constexpr int XREG_THREADS = 256;  // workgroup size of gemv_xreg_kernel (compile-time: the staging is fully unrolled)
 
-// The fixed-point activations of the integer variant (CV == 2), for the units that have one.
-struct NoXInt {};
-template <class U, int CV>
-struct XIntOf { typedef NoXInt type; };
-template <class U>
-struct XIntOf<U, 2> { typedef typename U::XInt type; };
-
 // Arguments of gemv_xreg_kernel.  Up to three matrices of the same format and row length share one launch and
 // one activation vector (the q and k projections of a decode step): their rows are numbered one after the other.
 struct XregArgs {
@@ -857,11 +764,6 @@ __device__ __forceinline__ void gemv_xreg_body(const XregArgs &a, const int bid,
         for (int i = 0; i < NS; ++i) xs[s].sm[i] = sums[(s * 64 + lane) * NS + i];
     }
 
-    typename XIntOf<U, CV>::type xi;
-    if constexpr (CV == 2) {
-        static_assert(STEPS == 1 && !DUAL, "the integer variant takes one 64-value unit per lane");
-        U::to_fixed(xs[0], xi);
-    }
     int left = a.rpw;  // 0: the priority stays where it is
     step_priority(left);
     float gate = 0.f;  // DUAL: the gate row's result, held until the up row of the same index is done
@@ -871,14 +773,10 @@ __device__ __forceinline__ void gemv_xreg_body(const XregArgs &a, const int bid,
             const int row = base + (DUAL ? b / 2 : b) * stride;
             if (row < n) {  // wave-uniform
                 float acc[1][1] = {{0.f}};
-                if constexpr (CV == 2) {
-                    acc[0][0] = U::dot_int(buf[b][0], uc[0], xi);
-                } else {
 #pragma unroll
-                    for (int s = 0; s < STEPS; ++s) {
-                        const typename U::Raw(&w1)[1] = reinterpret_cast<const typename U::Raw(&)[1]>(buf[b][s]);
-                        U::template dot<1, 1, CV>(w1, uc[s], xs[s], acc, a.nib);
-                    }
+                for (int s = 0; s < STEPS; ++s) {
+                    const typename U::Raw(&w1)[1] = reinterpret_cast<const typename U::Raw(&)[1]>(buf[b][s]);
+                    U::template dot<1, 1, CV>(w1, uc[s], xs[s], acc, a.nib);
                 }
                 const float t = wave_sum(acc[0][0]);
                 if (!DUAL || (b & 1)) step_priority(--left);

@@ -11,8 +11,6 @@ size_t gemv_rows_scratch_bytes(int rows, int k) {
     return gemv_rows_ops_bytes(groups, k) + gemv_rows_inv_bytes(groups, k);
 }
 
-static bool group_split = true;
-void gemv_rows_configure(bool split_groups) { group_split = split_groups; }
 
 // Two tiles per wave where that still gives every CU a workgroup - and, for many groups of activation rows, where it gives
 // every other CU one: two tiles share the activation operands, which are what the launch waits for, and the idle half of the
@@ -24,7 +22,7 @@ void gemv_rows_configure(bool split_groups) { group_split = split_groups; }
 static int tiles_per_wave(int fmt, int n, int k, int rows, unsigned max_blocks) {
     const unsigned pairs = (unsigned)(((n + 15) / 16 + 1) / 2);
     bool half = fmt == F_Q6_K && rows > 16 && k >= 8192;
-    if (group_split && rows > 32 && k >= 4096 && (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K || fmt == F_Q4_1)) half = true;
+    if (rows > 32 && k >= 4096 && (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K || fmt == F_Q4_1)) half = true;
     return pairs >= max_blocks || (half && 2 * pairs >= max_blocks) ? 2 : 1;
 }
 
@@ -92,7 +90,7 @@ static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const v
     // each decodes the tile's weights again (the device would idle otherwise) and writes whole outputs of its own rows.
     // 1024 x 4096 at 40 rows: Q6_K 30.0 -> 19.4 us, Q4_K 17.5 -> 13.5; twice as many workgroups as CUs: 23.4, 13.9.
     int gy = 1;
-    if (group_split && (unsigned)nbatch * 2 <= max_blocks) {
+    if ((unsigned)nbatch * 2 <= max_blocks) {
         const int cap = (int)(max_blocks / (unsigned)nbatch), gper = (groups + cap - 1) / cap;
         gy = (groups + gper - 1) / gper;
     }

@@ -73,33 +73,13 @@ struct State {
     float nib = 0.f;  // 1 / (value of E4M3 byte 0x01): 512 for OCP, 1024 for FNUZ
     size_t max_lds = 0;      // LDS one workgroup may ask for
     size_t lds_per_cu = 0;   // LDS of a compute unit
-    int xreg_blocks_per_cu = 0;  // JITNN_HIP_XREG_BLOCKS: override of the workgroups per CU (0 = built-in choice)
-    int xreg_pf = 0;             // JITNN_HIP_XREG_PF: override of the rows in flight per wave, 1 or 2 (0 = built-in choice)
-    bool q6k_int = true;         // JITNN_HIP_Q6K_INT=0: the Q6_K output head through the FP32 variant (A/B measurements)
-    int q6k_int_min_rows = 16;   // JITNN_HIP_Q6K_INT_MIN_ROWS: rows per wave from which Q6_K takes the integer variant (tests: 1)
-    bool xreg_priority = true;   // JITNN_HIP_XREG_PRIORITY=0: no wave priority steps in the register-resident kernels (A/B measurements)
     // JITNN_HIP_GEMV_MAX_ROWS: up to this many rows run the FP32 GEMV kernels (in batches of 8), more rows the FP16
     // MFMA kernel - the counterpart of jitnn.gguf.tiledRows (core/JitnnConfig.java:423-424).  64 keeps every row
     // count the reference's own tests use (1, 5, 40) on the FP32 path, whose error meets their 2e-4 / 1e-3 bars.
     int gemv_max_rows = 64;
-    bool force_lds = false;      // JITNN_HIP_FORCE_LDS=1: route batch 1 through the LDS kernel (A/B measurements)
-    bool batch_mfma = true;      // JITNN_HIP_BATCH_MFMA=0: batches 2..8 through the FP32 LDS kernel instead of the matrix-core one
-    bool batch2_xreg = true;     // JITNN_HIP_BATCH2_XREG=0: batch 2 through the batch 2..8 kernels instead of the two-row register kernel
-    bool prefill_defer_join = true;  // JITNN_HIP_PREFILL_DEFER_JOIN=0: every split-K linear of the prefill step is joined by a kernel of its own
-    bool prefill_group = true;   // JITNN_HIP_PREFILL_GROUP=0: every weight of a group of linears in a launch of its own
-    bool rows_kernel_min_set = false;  // JITNN_HIP_ROWS_MIN was given: no per-shape exceptions
-    int rows_kernel_min = 9;     // JITNN_HIP_ROWS_MIN: fewest rows that take the one-pass kernel of gemv_rows.h (0: never); up to 8 rows gemv_mfma_kernel is faster
-    int prefill_min_slice = 8;      // JITNN_HIP_PREFILL_MIN_SLICE: fewest K steps (of 64 values) a slice of a split many-row launch may have
-    bool rows_prepare_fused = true;   // JITNN_HIP_ROWS_PREPARE_FUSED=0: the SwiGLU in front of a one-pass ffn_down by a kernel of its own
     bool transcode = true;            // JITNN_HIP_TRANSCODE=0: uploaded Q5_0 / Q3_K blocks stay as they are (plain kernels)
-    bool prefill_rope_join = true;    // JITNN_HIP_PREFILL_ROPE_JOIN=0: the K slices of q, k and v of a prefill step joined by a kernel of its own
-    bool prefill_dual = true;         // JITNN_HIP_PREFILL_DUAL=0: gate and up of a prefill step as two products, SwiGLU by the next preparation
-    bool prefill_fuse_swiglu = true;  // JITNN_HIP_PREFILL_FUSE_SWIGLU=0: silu(gate) * up of a prefill step by a kernel of its own
-    bool prefill_attn_mfma = true;  // JITNN_HIP_PREFILL_ATTN_MFMA=0: the FP16 attention of long prompts on v_dot2 instead of the matrix cores
-    bool prefill_attn_fp16 = true;  // JITNN_HIP_PREFILL_ATTN_FP16=0: the prefill step's attention in FP32 whatever the prompt length
     void *scratch_ptr = nullptr;    // device address of `scratch` on g.device (hipGetSymbolAddress at init)
     bool gemv_i8 = true;            // JITNN_HIP_GEMV_I8=0: batch-1 K-quant GEMV on the FP32 register kernels instead of the INT8 matrix-core one
-    int i8_pf = 0, i8_blocks_per_cu = 0;  // JITNN_HIP_I8_PF / JITNN_HIP_I8_BLOCKS: overrides for measurements (0 = built-in choice)
 };
 State g;
 std::mutex g_mu;
@@ -269,6 +249,8 @@ int xreg_args(const XregCall &c, XregArgs &a) {
 
 // The INT8 matrix-core kernel (gemv_i8.h) takes what the register-resident kernels take of the K-quants, and rows of up
 // to 16384 values.
+constexpr int PREFILL_MIN_SLICE = 8;  // fewest K steps (of 64 values) a slice of a split many-row launch may have
+
 // Its row groups are four rows: at least four rows in all, and the segments of a shared launch whole groups; its buffer
 // loads address a matrix with 32 bits.
 bool i8_ok(const XregCall &c) {
@@ -307,10 +289,8 @@ void i8_shape(int groups, int waves, bool dual, int &blocks, int &pf) {
     // (1/1) 14.3 (2/1) 16.2 (1/2).  Tall matrices: one workgroup per CU with two turns in flight behind the one being
     // multiplied; short ones: two workgroups with one; long rows: one with one.
     const int turns1 = (groups + g.cus - 1) / g.cus;
-    int per_cu = waves > 4 ? 1 : turns1 >= 8 ? 1 : 2;
+    const int per_cu = waves > 4 ? 1 : turns1 >= 8 ? 1 : 2;
     pf = waves > 4 ? 1 : turns1 >= 8 ? (dual ? 3 : 2) : 1;  // (gate + up of an 8B layer: 14.4 us with three turns in flight, 15.1 with two)
-    if (g.i8_blocks_per_cu > 0) per_cu = g.i8_blocks_per_cu;
-    if (g.i8_pf > 0) pf = g.i8_pf;
     blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
 }
 
@@ -339,20 +319,13 @@ int launch_xreg(const XregCall &c, hipStream_t stream) {
     // workgroups per CU and one row of prefetch: Q8_0 4096 x 4096 6.9 -> 6.5 us, attn_o of the 8B step 5.34 -> 5.25; from
     // 11008 rows on the two-workgroup shape is level or ahead (Q4_0 11008 x 4096 7.56 against 7.78 us).
     const bool few = n <= 8192 && !c.w2;
-    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : few ? 3 : 2);
+    const int cap = g.cus * (few ? 3 : 2);
     if (blocks > cap) blocks = cap;
     const int rows_per_wave = (n + blocks * waves - 1) / (blocks * waves);
-    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (few || rows_per_wave >= 16 ? 1 : 2);
-    a.rpw = g.xreg_priority ? rows_per_wave : 0;
+    const int pf = few || rows_per_wave >= 16 ? 1 : 2;
+    a.rpw = rows_per_wave;
     const int mode = c.w2 ? 3 : c.norm_w ? 2 : c.bias ? 1 : 0;
     xreg_fn fn = pick_xreg(c.w[0]->fmt, a.k % 64 == 0, mode, pf);
-    // Q6_K with many rows per wave (the output head): the integer variant, whose one-off cost of turning the
-    // activations into byte planes is spread over the rows
-    if (c.w[0]->fmt == F_Q6_K && g.q6k_int && rows_per_wave >= g.q6k_int_min_rows && a.k % 256 == 0) {
-        if (mode == 0) fn = pf == 1 ? gemv_xreg_kernel<Unit<F_Q6_K>, 2, 1, false, false, false> : gemv_xreg_kernel<Unit<F_Q6_K>, 2, 2, false, false, false>;
-        else if (mode == 1) fn = pf == 1 ? gemv_xreg_kernel<Unit<F_Q6_K>, 2, 1, true, false, false> : gemv_xreg_kernel<Unit<F_Q6_K>, 2, 2, true, false, false>;
-        else if (mode == 2) fn = pf == 1 ? gemv_xreg_kernel<Unit<F_Q6_K>, 2, 1, false, true, false> : gemv_xreg_kernel<Unit<F_Q6_K>, 2, 2, false, true, false>;
-    }
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(threads), 0, stream, a);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
@@ -396,7 +369,7 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
     XregArgs a{}, b{};
     const int na = xreg_args(ca, a), nb = xreg_args(cb, b);
     const int waves = XREG_THREADS / 64;
-    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : 2);
+    const int cap = g.cus * 2;
     const double ba = (double)na * ca.w[0]->nbytes / ca.w[0]->n, bb = (double)nb * cb.w[0]->nbytes / cb.w[0]->n;
     int blocks_a = (int)(cap * ba / (ba + bb) + 0.5), blocks_b;
     if (blocks_a < 1) blocks_a = 1;
@@ -406,9 +379,9 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
     if (blocks_b > (nb + waves - 1) / waves) blocks_b = (nb + waves - 1) / waves;
     const int rpw_a = (na + blocks_a * waves - 1) / (blocks_a * waves), rpw_b = (nb + blocks_b * waves - 1) / (blocks_b * waves);
     // (one row of prefetch: the q, k | v launch of an 8B layer - 6144 rows, three per wave - 8.1 -> 7.7 us against two)
-    const int pf = g.xreg_pf > 0 ? g.xreg_pf : 1;
-    a.rpw = g.xreg_priority ? rpw_a : 0;
-    b.rpw = g.xreg_priority ? rpw_b : 0;
+    const int pf = 1;
+    a.rpw = rpw_a;
+    b.rpw = rpw_b;
     xreg2_fn fn = pf == 1 ? pick_xreg2_pf<1>(ca.w[0]->fmt, cb.w[0]->fmt) : pick_xreg2_pf<2>(ca.w[0]->fmt, cb.w[0]->fmt);
     hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(XREG_THREADS), 0, stream, a, b, blocks_a);
     HIP_TRY(hipGetLastError());
@@ -463,9 +436,8 @@ int launch_gemv_ksplit(const jitnn_hip_weight *w, const float *x, const float *b
     // 14.0 -> 13.0, Q4_K 4096 x 8192 8.45 -> 8.2; with many rows per workgroup more of them are better (Q4_K 14336 x 8192
     // 15.4 against 16.8 us with three).
     if (w->n <= 8192 && per_cu > 3) per_cu = 3;
-    if (g.xreg_blocks_per_cu > 0 && per_cu > g.xreg_blocks_per_cu) per_cu = g.xreg_blocks_per_cu;
     int blocks = w->n < g.cus * per_cu ? w->n : g.cus * per_cu;
-    const int pf = g.xreg_pf > 0 ? g.xreg_pf : 1;
+    const int pf = 1;
     gemv1_fn fn = pf == 1 ? pick_ksplit_pf<1>(w->fmt, w->k % 64 == 0) : pick_ksplit_pf<2>(w->fmt, w->k % 64 == 0);
     if (int rc = allow_lds((const void *)fn, lds)) return rc;
     hipLaunchKernelGGL(fn, dim3(blocks), dim3(64 * slices), lds, stream, w->dev, x, bias, y, w->n, w->k, g.nib);
@@ -489,10 +461,10 @@ gemv1_fn pick_xreg_b2_fmt(int fmt, bool pairs) {
 int launch_gemv_xreg_b2(const jitnn_hip_weight *w, const float *x, const float *bias, float *y, hipStream_t stream) {
     const int waves = XREG_THREADS / 64;
     int blocks = (w->n + waves - 1) / waves;
-    const int cap = g.cus * (g.xreg_blocks_per_cu > 0 ? g.xreg_blocks_per_cu : 2);
+    const int cap = g.cus * 2;
     if (blocks > cap) blocks = cap;
     const int rows_per_wave = (w->n + blocks * waves - 1) / (blocks * waves);
-    const int pf = g.xreg_pf > 0 ? g.xreg_pf : (rows_per_wave >= 16 ? 1 : 2);
+    const int pf = rows_per_wave >= 16 ? 1 : 2;
     const bool pairs = w->k % 64 == 0;
     gemv1_fn fn = bias ? (pf == 1 ? pick_xreg_b2_fmt<1, true>(w->fmt, pairs) : pick_xreg_b2_fmt<2, true>(w->fmt, pairs))
                        : (pf == 1 ? pick_xreg_b2_fmt<1, false>(w->fmt, pairs) : pick_xreg_b2_fmt<2, false>(w->fmt, pairs));
@@ -526,14 +498,14 @@ int launch_gemv_plain(const jitnn_hip_weight *w, const float *x, int rows, const
 
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
     if (is_extra_format(w->fmt)) return launch_gemv_plain(w, x, rows, bias, y, stream);
-    if (rows == 2 && w->k <= 4096 && !g.force_lds && g.batch2_xreg) return launch_gemv_xreg_b2(w, x, bias, y, stream);
+    if (rows == 2 && w->k <= 4096) return launch_gemv_xreg_b2(w, x, bias, y, stream);
     // Q6_K pays the most per weight on the matrix-core path (6-bit quants from two arrays, 16-value scale groups): up to
     // four rows its FP32 kernel is still ahead (measured: 33 vs 43 us at 2 rows, 151 vs 167 us at 4 rows on the output head)
-    if (rows >= (w->fmt == F_Q6_K ? 5 : 2) && rows <= 8 && w->k % 256 == 0 && w->n >= 16 && g.batch_mfma) {
+    if (rows >= (w->fmt == F_Q6_K ? 5 : 2) && rows <= 8 && w->k % 256 == 0 && w->n >= 16) {
         const KernelRef v = gemv_mfma_kernel_ref(w->fmt);
         if (v.fn && v.lds <= g.max_lds) return launch_gemv_mfma(v, w, x, rows, bias, y, stream);
     }
-    if (rows == 1 && !g.force_lds) {
+    if (rows == 1) {
         if (w->k <= 4096) return launch_gemv_xreg(w, x, bias, y, stream);
         if (w->k <= 32768 && ksplit_lds(w->fmt, (w->k + 4095) / 4096) <= g.max_lds) return launch_gemv_ksplit(w, x, bias, y, stream);
     }
@@ -730,7 +702,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
         Launch &l = launch[nlaunch++];
         l.first = i;
         int j = i + 1;
-        const bool joinable = !bias && !residual && g.prefill_group;  // (several weights: partial sums of all of them are joined by one kernel)
+        const bool joinable = !bias && !residual;  // (several weights: partial sums of all of them are joined by one kernel)
         while (joinable && j < count && j - i < 3 && ws[j]->fmt == ws[i]->fmt && ws[j]->n % 4 == 0 && ws[i]->n % 4 == 0) ++j;
         l.first_b = j - i;
         if (joinable && j < count && j - i < 3 && ws[j]->fmt != ws[i]->fmt && ws[i]->n % 4 == 0 && ws[j]->n % 4 == 0) {
@@ -752,7 +724,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
         // own partial y, a second kernel adds the slices in order.
         int splits = 1;
         if (nsum % 4 == 0 && ws[i]->n % 4 == 0) {
-            while (splits < 8 && tiles * mtiles * splits * 2 <= g.cus && nsteps / (splits * 2) >= g.prefill_min_slice) splits *= 2;
+            while (splits < 8 && tiles * mtiles * splits * 2 <= g.cus && nsteps / (splits * 2) >= PREFILL_MIN_SLICE) splits *= 2;
         }
         int wgs = tiles * mtiles * splits;
         l.part_bytes = 0;
@@ -761,7 +733,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
             l.splits[q] = splits;
             // the second format of a two-format launch (Q6_K beside Q4_K or Q5_K) takes half as long again per step: its
             // tiles get slices half as long where the device has the room, so that the launch does not wait for them
-            if (q >= l.first_b && splits > 1 && splits < 8 && wgs + tiles_of(wq) * mtiles * splits <= g.cus && nsteps / (splits * 2) >= g.prefill_min_slice) {
+            if (q >= l.first_b && splits > 1 && splits < 8 && wgs + tiles_of(wq) * mtiles * splits <= g.cus && nsteps / (splits * 2) >= PREFILL_MIN_SLICE) {
                 l.splits[q] = splits * 2;
                 wgs += tiles_of(wq) * mtiles * splits;
             }
@@ -844,7 +816,7 @@ int launch_prefill_group(const jitnn_hip_weight *const *ws, float *const *ys, in
 // and the up projection of a Llama FFN as one product whose epilogue forms the SwiGLU - the two [rows, n] products are
 // neither stored nor read back.  pend: as in launch_prefill_group.
 bool prefill_dual_ok(const jitnn_hip_weight *gate, const jitnn_hip_weight *up) {
-    return g.prefill_dual && gate->fmt == up->fmt && gate->n == up->n && gate->k == up->k && !is_extra_format(gate->fmt) &&
+    return gate->fmt == up->fmt && gate->n == up->n && gate->k == up->k && !is_extra_format(gate->fmt) &&
            prefill_prepare_fuses_norm(gate->k);
 }
 
@@ -956,45 +928,12 @@ int jitnn_hip_init(int device_ordinal) {
         if (se != hipSuccess || !sp) return fail(JITNN_HIP_EDEVICE, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(se));
         g.scratch_ptr = sp;
     }
-    if (const char *e = getenv("JITNN_HIP_XREG_BLOCKS")) {
-        int v = atoi(e);
-        if (v >= 1 && v <= 32) g.xreg_blocks_per_cu = v;
-    }
-    if (const char *e = getenv("JITNN_HIP_XREG_PF")) {
-        int v = atoi(e);
-        if (v >= 1 && v <= 2) g.xreg_pf = v;
-    }
-    if (const char *e = getenv("JITNN_HIP_Q6K_INT")) g.q6k_int = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_Q6K_INT_MIN_ROWS")) {
-        int v = atoi(e);
-        if (v >= 1) g.q6k_int_min_rows = v;
-    }
-    if (const char *e = getenv("JITNN_HIP_XREG_PRIORITY")) g.xreg_priority = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_GEMV_MAX_ROWS")) {
         int v = atoi(e);
         if (v >= 1) g.gemv_max_rows = v;
     }
     if (const char *e = getenv("JITNN_HIP_GEMV_I8")) g.gemv_i8 = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_I8_PF")) g.i8_pf = atoi(e);
-    if (const char *e = getenv("JITNN_HIP_I8_BLOCKS")) g.i8_blocks_per_cu = atoi(e);
-    if (const char *e = getenv("JITNN_HIP_FORCE_LDS")) g.force_lds = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_BATCH_MFMA")) g.batch_mfma = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_BATCH2_XREG")) g.batch2_xreg = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_ROWS_MIN")) {
-        g.rows_kernel_min = atoi(e);
-        g.rows_kernel_min_set = true;
-    }
-    if (const char *e = getenv("JITNN_HIP_PREFILL_GROUP")) g.prefill_group = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_PREFILL_DEFER_JOIN")) g.prefill_defer_join = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_FP16")) g.prefill_attn_fp16 = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_PREFILL_ATTN_MFMA")) g.prefill_attn_mfma = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_PREFILL_FUSE_SWIGLU")) g.prefill_fuse_swiglu = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_PREFILL_DUAL")) g.prefill_dual = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_PREFILL_ROPE_JOIN")) g.prefill_rope_join = atoi(e) != 0;
     if (const char *e = getenv("JITNN_HIP_TRANSCODE")) g.transcode = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_ROWS_PREPARE_FUSED")) g.rows_prepare_fused = atoi(e) != 0;
-    if (const char *e = getenv("JITNN_HIP_ROWS_GROUP_SPLIT")) gemv_rows_configure(atoi(e) != 0);
-    if (const char *e = getenv("JITNN_HIP_PREFILL_MIN_SLICE")) g.prefill_min_slice = atoi(e) >= 4 ? atoi(e) : 4;
     g.device = device_ordinal;
     g.ready = true;
     return JITNN_HIP_OK;
@@ -1168,13 +1107,11 @@ namespace {
 // kernels for up to 8 rows are the fastest of all, and 8 + 1..3 rows in two passes still beat the one pass (14336 x 4096
 // Q4_0 at 9 rows 21.9 against 27.0 us, at 12 rows 26.2 against 27.0, at 20 rows 38.9 against 29.9).
 bool rows_path(const jitnn_hip_weight *w, int rows) {
-    int rows_min = g.rows_kernel_min;
-    if (!g.rows_kernel_min_set) {
-        if (w->k >= 12288) rows_min = 3;
-        else if (w->fmt == F_Q4_0 || w->fmt == F_Q4_1) rows_min = 12;
-    }
-    return g.rows_kernel_min > 0 && rows >= rows_min && rows <= 64 && rows <= g.gemv_max_rows && gemv_rows_supported(w->fmt) && w->k % 256 == 0 &&
-           w->n >= 16 && !g.force_lds;
+    int rows_min = 9;  // (up to 8 rows gemv_mfma_kernel is faster)
+    if (w->k >= 12288) rows_min = 3;
+    else if (w->fmt == F_Q4_0 || w->fmt == F_Q4_1) rows_min = 12;
+    return rows >= rows_min && rows <= 64 && rows <= g.gemv_max_rows && gemv_rows_supported(w->fmt) && w->k % 256 == 0 &&
+           w->n >= 16;
 }
 
 // ys[i] = x ws[i]^T (+ bias) (+ residual [rows, n]; bias and residual with one weight only) for weights that all pass
@@ -1505,7 +1442,7 @@ void launch_attention(const jitnn_hip_llama *m, int layer, int pos, hipStream_t 
     else hipLaunchKernelGGL((attn_merge_kernel<D, 2>), dim3(m->heads), dim3(2 * D), 0, st, m->part, m->att, chunks);
 }
 
-bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !g.force_lds && !is_extra_format(w->fmt); }
+bool xreg_ok(const jitnn_hip_weight *w) { return w->k <= 4096 && !is_extra_format(w->fmt); }
 
 // y_i = W_i RMSNorm(x; nw) for `count` (at most 3) weights over the same x.  Weights the register-resident kernel
 // takes get the norm fused into their launch, neighbours of one format share the launch; anything else goes through
@@ -1608,11 +1545,10 @@ int normed_linears_rows(const jitnn_hip_llama *m, const jitnn_hip_weight *const 
 int residual_linear_rows(const jitnn_hip_weight *w, const float *x, int rows, const float *res, float *tmp, float *y, hipStream_t st,
                          const float *up = nullptr, float *h = nullptr, float *part = nullptr, PfPending *defer = nullptr) {
     const bool many = rows > g.gemv_max_rows && has_many_row_kernel(w->fmt) && w->n % 4 == 0;
-    if (many && (!up || (g.prefill_fuse_swiglu && prefill_prepare_fuses_norm(w->k)))) {
-        return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp, up, SCRATCH_THREAD, g.prefill_defer_join ? part : nullptr,
-                                    g.prefill_defer_join ? defer : nullptr);
+    if (many && (!up || prefill_prepare_fuses_norm(w->k))) {
+        return launch_prefill_group(&w, &y, 1, x, rows, nullptr, nullptr, 0.f, st, res, tmp, up, SCRATCH_THREAD, part, defer);
     }
-    if (up && g.rows_prepare_fused && rows_path(w, rows)) {  // silu(x) * up is formed by the preparation of the one-pass kernel
+    if (up && rows_path(w, rows)) {  // silu(x) * up is formed by the preparation of the one-pass kernel
         count_op(ST_GEMV, (long long)w->nbytes + 4ll * rows * ((long long)w->k + w->n));
         return launch_rows_group(&w, &y, 1, x, rows, nullptr, res, st, SCRATCH_THREAD, up);
     }
@@ -1666,9 +1602,9 @@ int launch_attention_rows(const jitnn_hip_llama *m, int layer, int pos0, int tok
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
     const float scale = 1.0f / sqrtf((float)D);
     // prompts beyond the GEMV range have FP16-operand linears on both sides of the attention: FP16 operands here too
-    if (tokens > g.gemv_max_rows && g.prefill_attn_fp16) {
+    if (tokens > g.gemv_max_rows) {
         if constexpr (D == 64 || D == 128) {
-            if (g.prefill_attn_mfma && group <= AM_ROWS) {
+            if (group <= AM_ROWS) {
                 const int qt = AM_ROWS / group;
                 const dim3 grid((tokens + qt - 1) / qt, m->kv);
                 constexpr size_t lds = attn_prefill_mfma_lds_bytes<D>();
@@ -1681,7 +1617,7 @@ int launch_attention_rows(const jitnn_hip_llama *m, int layer, int pos0, int tok
     }
     const int qt = ATT_ROWS / group;
     const dim3 grid((tokens + qt - 1) / qt, m->kv);
-    if (tokens > g.gemv_max_rows && g.prefill_attn_fp16) {
+    if (tokens > g.gemv_max_rows) {
         constexpr size_t lds = attn_prefill_h_lds_bytes<D>();
         if (int rc = allow_lds((const void *)attn_prefill_h_kernel<D>, lds)) return rc;
         hipLaunchKernelGGL(attn_prefill_h_kernel<D>, grid, dim3(256), lds, st, q, m->kc + lo, m->vc + lo, att, m->heads, m->kv, pos0, tokens, scale);
@@ -1899,7 +1835,7 @@ int jitnn_hip_llama_prefill_dev(jitnn_hip_llama *m, const float *x_dev, int pos0
         {
             const jitnn_hip_weight *ws[3] = {w[JITNN_HIP_W_ATTN_Q], w[JITNN_HIP_W_ATTN_K], w[JITNN_HIP_W_ATTN_V]};
             float *ys[3] = {q, k, v};
-            if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st, &pend, g.prefill_rope_join ? &gp : nullptr)) return rc;
+            if (int rc = normed_linears_rows(m, ws, ys, 3, x, T, nw, xn, st, &pend, &gp)) return rc;
         }
         if (gp.part) {  // q, k and v still lie in K slices: the rotation adds them up as it reads them
             hipLaunchKernelGGL(rope_append_rows_join_kernel, dim3(T), dim3(256), 0, st, gp.part, gp.sg.splits[0], gp.sg.splits[1], gp.sg.splits[2], T, q,

@@ -82,7 +82,6 @@ void gemv_mfma_launch(int fmt, unsigned blocks, hipStream_t s, const uint8_t *W,
 // values, the values of a lane consecutive or in the two halves of a 4-bit block) into a scratch of
 // gemv_rows_scratch_bytes and serve every weight of that layout that meets the same activations.
 constexpr int GR_LAYOUT_PLAIN = 0, GR_LAYOUT_SUMS16 = 1, GR_LAYOUT_HALVES = 2, GR_LAYOUTS = 3;
-void gemv_rows_configure(bool split_groups);       // false: a tile's groups of activation rows all stay in one workgroup (A/B runs)
 bool gemv_rows_supported(int fmt);
 int gemv_rows_layout(int fmt);                     // GR_LAYOUT_* of the format, -1: the kernel is not built for it
 size_t gemv_rows_scratch_bytes(int rows, int k);   // operands + scales of `rows` activation rows of k values
