@@ -32,11 +32,15 @@ namespace jitnn {
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int I8_FLUSH = 24;   // turns between two joins of the waves' partial sums (a multiple of every ring length)
 constexpr int I8_MAX_WAVES = 16;
-constexpr size_t I8_LDS_PER_WAVE = 3072;  // 16 chunks x 3 planes x 64 bytes; afterwards the wave's partial sums (2 x 24 turns x 16 floats)
-
-__host__ __device__ constexpr size_t gemv_i8_lds_bytes(int waves) { return (size_t)waves * I8_LDS_PER_WAVE; }
+// turns between two joins of the waves' partial sums (a multiple of every ring length): 24 for one activation row, 12 for more
+__host__ __device__ constexpr int i8_flush(int rows) { return rows == 1 ? 24 : 12; }
+// LDS of a wave: 16 chunks x 3 planes x 64 bytes while the activations are staged; afterwards the wave's partial sums,
+// 2 windows x flush turns x rows x 16 floats
+__host__ __device__ constexpr size_t gemv_i8_lds_per_wave(int rows) {
+    return (size_t)2 * i8_flush(rows) * rows * 64 > 3072 ? (size_t)2 * i8_flush(rows) * rows * 64 : 3072;
+}
+__host__ __device__ constexpr size_t gemv_i8_lds_bytes(int waves, int rows = 1) { return (size_t)waves * gemv_i8_lds_per_wave(rows); }
 
 // The three digit sums of a block as one number.  With quants of at most five bits the whole sum fits 32 bits
 // (31 * 16 * 2^22 < 2^31); six-bit quants (63 * 16 * 2^22) need the last step in floating point.
@@ -88,20 +92,30 @@ struct U8<F_Q4_K> {
         s[0] = s4[0] + s4[1];
         s[1] = s4[2] + s4[3];
     }
-    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
-        i32x4 dl = {0, 0, 0, 0}, dh = {0, 0, 0, 0};
+    // the operands of the turn: dwords 0..7 the low nibbles (values 0..31 of the chunk), 8..15 the high ones (values 32..63)
+    static constexpr int CH = 2;  // chains of products: one per sub-block
+    struct Scale { float d0, d1, m0, m1; };
+    __device__ static __forceinline__ void extract(const Raw &r, int, uint32_t (&v)[16]) {
 #pragma unroll
         for (int m = 0; m < 8; ++m) {
-            const uint32_t v = m < 4 ? r.q0[m & 3] : r.q1[m & 3];
-            dl = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[m], (int)(v & 0x0f0f0f0fu), dl, 0, 0, 0);
-            dh = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + m], (int)((v >> 4) & 0x0f0f0f0fu), dh, 0, 0, 0);
+            const uint32_t w = m < 4 ? r.q0[m & 3] : r.q1[m & 3];
+            v[m] = w & 0x0f0f0f0fu;
+            v[8 + m] = (w >> 4) & 0x0f0f0f0fu;
         }
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int c, Scale &sc) {
         uint32_t sc2, mn2;
         i8_scale_min(r.h, c & 3, sc2, mn2);
-        const float d = h2f(r.h.x) * sinv, dmin = h2f(r.h.x >> 16);
-        const float t = __builtin_fmaf(d * ub0(sc2), (float)i8_combine(dl), (d * ub1(sc2)) * (float)i8_combine(dh));
-        const float m = __builtin_fmaf(dmin * ub0(mn2), s[0], (dmin * ub1(mn2)) * s[1]);
-        return t - m;
+        const float d = h2f(r.h.x), dmin = h2f(r.h.x >> 16);
+        sc.d0 = d * ub0(sc2);
+        sc.d1 = d * ub1(sc2);
+        sc.m0 = dmin * ub0(mn2);
+        sc.m1 = dmin * ub1(mn2);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&s)[NSUM]) {
+        const float t = __builtin_fmaf(sc.d0, (float)i8_combine(d[0]), sc.d1 * (float)i8_combine(d[1]));
+        const float m = __builtin_fmaf(sc.m0, s[0], sc.m1 * s[1]);
+        return __builtin_fmaf(t, sinv, -m);
     }
 };
 
@@ -132,24 +146,29 @@ struct U8<F_Q5_K> {
         s[0] = s4[0] + s4[1];
         s[1] = s4[2] + s4[3];
     }
-    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
-        i32x4 dl = {0, 0, 0, 0}, dh = {0, 0, 0, 0};
+    static constexpr int CH = 2;
+    typedef U8<F_Q4_K>::Scale Scale;
+    __device__ static __forceinline__ void extract(const Raw &r, int c, uint32_t (&v)[16]) {
         const int sh = 2 * (c & 3);
 #pragma unroll
         for (int m = 0; m < 8; ++m) {
-            const uint32_t v = m < 4 ? r.q0[m & 3] : r.q1[m & 3];
+            const uint32_t w = m < 4 ? r.q0[m & 3] : r.q1[m & 3];
             const uint32_t hb = (m < 4 ? r.h0[m & 3] : r.h1[m & 3]) >> sh;  // bit 0 of every byte: sub-block 2j, bit 1: 2j + 1
-            const uint32_t lo = (v & 0x0f0f0f0fu) | ((hb << 4) & 0x10101010u);
-            const uint32_t hi = ((v >> 4) & 0x0f0f0f0fu) | ((hb << 3) & 0x10101010u);
-            dl = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[m], (int)lo, dl, 0, 0, 0);
-            dh = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + m], (int)hi, dh, 0, 0, 0);
+            v[m] = (w & 0x0f0f0f0fu) | ((hb << 4) & 0x10101010u);
+            v[8 + m] = ((w >> 4) & 0x0f0f0f0fu) | ((hb << 3) & 0x10101010u);
         }
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int c, Scale &sc) {
         uint32_t sc2, mn2;
         i8_scale_min(r.h, c & 3, sc2, mn2);
-        const float d = h2f(r.h.x) * sinv, dmin = h2f(r.h.x >> 16);
-        const float t = __builtin_fmaf(d * ub0(sc2), (float)i8_combine(dl), (d * ub1(sc2)) * (float)i8_combine(dh));
-        const float m = __builtin_fmaf(dmin * ub0(mn2), s[0], (dmin * ub1(mn2)) * s[1]);
-        return t - m;
+        const float d = h2f(r.h.x), dmin = h2f(r.h.x >> 16);
+        sc.d0 = d * ub0(sc2);
+        sc.d1 = d * ub1(sc2);
+        sc.m0 = dmin * ub0(mn2);
+        sc.m1 = dmin * ub1(mn2);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&s)[NSUM]) {
+        return U8<F_Q4_K>::finish(sc, d, sinv, s);
     }
 };
 
@@ -177,28 +196,32 @@ struct U8Q6Base {
 #pragma unroll
         for (int i = 0; i < 4; ++i) s[i] = -32.f * s4[i];
     }
-    // la, lb: the lane's 16 bytes of ql at 64 n + 16 r and 32 further on; qh: its 16 bytes of qh; sa, sb: dwords whose bytes 0 and
-    // 2 are the scales of runs 0, 1 | 2, 3; d: the block scale's bits
-    __device__ static __forceinline__ float dot_fields(const u32x4 &la, const u32x4 &lb, const u32x4 &qh, uint32_t sa, uint32_t sb, uint32_t d,
-                                                       const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
-        i32x4 d0 = {0, 0, 0, 0}, d1 = {0, 0, 0, 0}, d2 = {0, 0, 0, 0}, d3 = {0, 0, 0, 0};
+    static constexpr int CH = 4;  // one chain per run of 16 values
+    struct Scale { float c[4]; };  // d * scale of run k
+    // la, lb: the lane's 16 bytes of ql at 64 n + 16 r and 32 further on; qh: its 16 bytes of qh -> operands of run k in dwords 4k..4k+3
+    __device__ static __forceinline__ void extract_fields(const u32x4 &la, const u32x4 &lb, const u32x4 &qh, uint32_t (&v)[16]) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const uint32_t a = la[i], b = lb[i], h = qh[i];
-            const uint32_t v0 = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
-            const uint32_t v1 = (b & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
-            const uint32_t v2 = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
-            const uint32_t v3 = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
-            d0 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[i], (int)v0, d0, 0, 0, 0);
-            d1 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[4 + i], (int)v1, d1, 0, 0, 0);
-            d2 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[8 + i], (int)v2, d2, 0, 0, 0);
-            d3 = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[12 + i], (int)v3, d3, 0, 0, 0);
+            v[i] = (a & 0x0f0f0f0fu) | ((h << 4) & 0x30303030u);
+            v[4 + i] = (b & 0x0f0f0f0fu) | ((h << 2) & 0x30303030u);
+            v[8 + i] = ((a >> 4) & 0x0f0f0f0fu) | (h & 0x30303030u);
+            v[12 + i] = ((b >> 4) & 0x0f0f0f0fu) | ((h >> 2) & 0x30303030u);
         }
-        float acc = (float)(int)(int8_t)sa * __builtin_fmaf(i8_combine_wide(d0), sinv, s[0]);
-        acc = __builtin_fmaf((float)(int)(int8_t)(sa >> 16), __builtin_fmaf(i8_combine_wide(d1), sinv, s[1]), acc);
-        acc = __builtin_fmaf((float)(int)(int8_t)sb, __builtin_fmaf(i8_combine_wide(d2), sinv, s[2]), acc);
-        acc = __builtin_fmaf((float)(int)(int8_t)(sb >> 16), __builtin_fmaf(i8_combine_wide(d3), sinv, s[3]), acc);
-        return acc * h2f(d);
+    }
+    // sa, sb: dwords whose bytes 0 and 2 are the scales of runs 0, 1 | 2, 3; d: the block scale's bits
+    __device__ static __forceinline__ void scale_fields(uint32_t sa, uint32_t sb, uint32_t d, Scale &sc) {
+        const float df = h2f(d);
+        sc.c[0] = df * (float)(int)(int8_t)sa;
+        sc.c[1] = df * (float)(int)(int8_t)(sa >> 16);
+        sc.c[2] = df * (float)(int)(int8_t)sb;
+        sc.c[3] = df * (float)(int)(int8_t)(sb >> 16);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&s)[NSUM]) {
+        float acc = sc.c[0] * __builtin_fmaf(i8_combine_wide(d[0]), sinv, s[0]);
+#pragma unroll
+        for (int k = 1; k < 4; ++k) acc = __builtin_fmaf(sc.c[k], __builtin_fmaf(i8_combine_wide(d[k]), sinv, s[k]), acc);
+        return acc;
     }
 };
 
@@ -222,9 +245,10 @@ struct U8Q6<false> : U8Q6Base {
         r.sc = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)o.sc, (int)soff, 0);
         r.d = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)o.d, (int)soff, 0);
     }
-    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
+    __device__ static __forceinline__ void extract(const Raw &r, int, uint32_t (&v)[16]) { extract_fields(r.la, r.lb, r.qh, v); }
+    __device__ static __forceinline__ void scales(const Raw &r, int c, Scale &sc) {
         const int sh = (c & 1) * 8;
-        return dot_fields(r.la, r.lb, r.qh, r.sc.x >> sh, r.sc.y >> sh, r.d, xa, sinv, s);
+        scale_fields(r.sc.x >> sh, r.sc.y >> sh, r.d, sc);
     }
 };
 
@@ -258,35 +282,182 @@ struct U8Q6<true> : U8Q6Base {
         return u32x4{__builtin_amdgcn_alignbit(w.y, w.x, sh), __builtin_amdgcn_alignbit(w.z, w.y, sh), __builtin_amdgcn_alignbit(w.w, w.z, sh),
                      __builtin_amdgcn_alignbit(after, w.w, sh)};
     }
-    __device__ static __forceinline__ float dot(const Raw &r, int c, const uint32_t (&xa)[16], float sinv, const float (&s)[NSUM]) {
+    __device__ static __forceinline__ void extract(const Raw &r, int c, uint32_t (&v)[16]) {
         const uint32_t sh = (uint32_t)((c >> 2) & 1) * 16u;  // bits the block's fields sit past their windows' starts
         const bool r0 = (c & 1) == 0, n0 = (c & 2) == 0, last = (c & 3) == 3;
         // In memory the windows of a block follow one another as la(b0) la(b1) lb(b0) lb(b1) la(b2) la(b3) lb(b2) lb(b3) qh(b0..b3)
         // scales (b = chunk of the block): the dword after a window is the first dword of the next one.
         const uint32_t nla = next4(r.la.x), nlb = next4(r.lb.x), nqh = next4(r.qh.x), nsc = next4(r.sc.x), plb = prev4(r.lb.x);
-        const u32x4 la = shifted(r.la, r0 ? nla : plb, sh);
-        const u32x4 lb = shifted(r.lb, r0 ? nlb : n0 ? nla : nqh, sh);
-        const u32x4 qh = shifted(r.qh, last ? nsc : nqh, sh);
+        extract_fields(shifted(r.la, r0 ? nla : plb, sh), shifted(r.lb, r0 ? nlb : n0 ? nla : nqh, sh), shifted(r.qh, last ? nsc : nqh, sh), v);
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int c, Scale &sc) {
+        const uint32_t sh = (uint32_t)((c >> 2) & 1) * 16u;
         const uint32_t sx = __builtin_amdgcn_alignbit(r.sc.y, r.sc.x, sh), sy = __builtin_amdgcn_alignbit(r.sc.z, r.sc.y, sh);
         const int s8 = (c & 1) * 8;
-        return dot_fields(la, lb, qh, sx >> s8, sy >> s8, r.d >> sh, xa, sinv, s);
+        scale_fields(sx >> s8, sy >> s8, r.d >> sh, sc);
     }
 };
 
 template <>
 struct U8<F_Q6_K> : U8Q6<false> {};
 
+// ------------------------------------------------------------------------------------- the 32-value formats
+// Q4_0 (18 bytes: f16 d, 16 bytes of nibbles), Q4_1 (20: d, m, nibbles) and Q8_0 (34: d, 32 int8) - core/kernels/GgufKernels.java:85-99,
+// core/ops/Quant.java:137-144.  A chunk is two blocks (rows of a multiple of 64 values): a pair starts on a dword boundary
+// (36, 40 and 68 bytes), the lane fetches it as whole dwords and shifts the first block's quants, which sit two bytes past
+// one, into place with v_alignbit.  Value e of a 4-bit block is the low nibble of qs[e] for e < 16, the high nibble of
+// qs[e - 16] otherwise, so the operands keep the order of the values; one chain of products per block, one scale each.
+// Thirty-two products of up to 128 * 2^22 do not fit 32 bits: the digit sums are joined in floating point.
+__device__ __forceinline__ u32x4 i8_shift2(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3, uint32_t w4) {
+    return u32x4{__builtin_amdgcn_alignbit(w1, w0, 16), __builtin_amdgcn_alignbit(w2, w1, 16), __builtin_amdgcn_alignbit(w3, w2, 16),
+                 __builtin_amdgcn_alignbit(w4, w3, 16)};
+}
+
+struct U8Pair32 {
+    static constexpr int NSUM = 2, CH = 2;
+    __device__ static __forceinline__ int x_first(int c, int j) { return c * 64 + j * 16; }
+    __device__ static __forceinline__ int x_pos(int c, int e) { return c * 64 + e; }
+    __device__ static __forceinline__ void nibbles(const u32x4 &q0, const u32x4 &q1, uint32_t (&v)[16]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = q0[i] & 0x0f0f0f0fu;
+            v[4 + i] = (q0[i] >> 4) & 0x0f0f0f0fu;
+            v[8 + i] = q1[i] & 0x0f0f0f0fu;
+            v[12 + i] = (q1[i] >> 4) & 0x0f0f0f0fu;
+        }
+    }
+};
+
+template <>
+struct U8<F_Q4_0> : U8Pair32 {
+    static constexpr int FMT = F_Q4_0;
+    struct Raw { u32x4 a, b; uint32_t c; };  // bytes 0-1 d0, 2-17 qs0, 18-19 d1, 20-35 qs1
+    struct Off { uint32_t o; };
+    struct Scale { float d0, d1; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) { return Off{row_off + (uint32_t)c * 36u}; }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.a = i8_ld128(rs, o.o, soff);
+        r.b = i8_ld128(rs, o.o + 16u, soff);
+        r.c = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, (int)(o.o + 32u), (int)soff, 0);
+    }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {  // the -8 of the format meets the sums of x
+        s[0] = -8.f * (s4[0] + s4[1]);
+        s[1] = -8.f * (s4[2] + s4[3]);
+    }
+    __device__ static __forceinline__ void extract(const Raw &r, int, uint32_t (&v)[16]) {
+        nibbles(i8_shift2(r.a.x, r.a.y, r.a.z, r.a.w, r.b.x), u32x4{r.b.y, r.b.z, r.b.w, r.c}, v);
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int, Scale &sc) {
+        sc.d0 = h2f(r.a.x);
+        sc.d1 = h2f(r.b.x >> 16);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&s)[NSUM]) {
+        return __builtin_fmaf(sc.d0, __builtin_fmaf(i8_combine_wide(d[0]), sinv, s[0]), sc.d1 * __builtin_fmaf(i8_combine_wide(d[1]), sinv, s[1]));
+    }
+};
+
+template <>
+struct U8<F_Q4_1> : U8Pair32 {
+    static constexpr int FMT = F_Q4_1;
+    struct Raw { u32x4 a, b; u32x2 c; };  // bytes 0-3 d0 m0, 4-19 qs0, 20-23 d1 m1, 24-39 qs1
+    struct Off { uint32_t o; };
+    struct Scale { float d0, m0, d1, m1; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) { return Off{row_off + (uint32_t)c * 40u}; }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.a = i8_ld128(rs, o.o, soff);
+        r.b = i8_ld128(rs, o.o + 16u, soff);
+        r.c = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)(o.o + 32u), (int)soff, 0);
+    }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
+        s[0] = s4[0] + s4[1];
+        s[1] = s4[2] + s4[3];
+    }
+    __device__ static __forceinline__ void extract(const Raw &r, int, uint32_t (&v)[16]) {
+        nibbles(u32x4{r.a.y, r.a.z, r.a.w, r.b.x}, u32x4{r.b.z, r.b.w, r.c.x, r.c.y}, v);
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int, Scale &sc) {
+        sc.d0 = h2f(r.a.x);
+        sc.m0 = h2f(r.a.x >> 16);
+        sc.d1 = h2f(r.b.y);
+        sc.m1 = h2f(r.b.y >> 16);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&s)[NSUM]) {
+        const float t = __builtin_fmaf(sc.d0, i8_combine_wide(d[0]), sc.d1 * i8_combine_wide(d[1]));
+        return __builtin_fmaf(t, sinv, __builtin_fmaf(sc.m0, s[0], sc.m1 * s[1]));
+    }
+};
+
+template <>
+struct U8<F_Q8_0> : U8Pair32 {
+    static constexpr int FMT = F_Q8_0;
+    struct Raw { u32x4 a, b, c, d; uint32_t e; };  // bytes 0-1 d0, 2-33 qs0, 34-35 d1, 36-67 qs1
+    struct Off { uint32_t o; };
+    struct Scale { float d0, d1; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) { return Off{row_off + (uint32_t)c * 68u}; }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.a = i8_ld128(rs, o.o, soff);
+        r.b = i8_ld128(rs, o.o + 16u, soff);
+        r.c = i8_ld128(rs, o.o + 32u, soff);
+        r.d = i8_ld128(rs, o.o + 48u, soff);
+        r.e = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, (int)(o.o + 64u), (int)soff, 0);
+    }
+    __device__ static __forceinline__ void sums(const float (&)[4], float (&s)[NSUM]) { s[0] = s[1] = 0.f; }
+    __device__ static __forceinline__ void extract(const Raw &r, int, uint32_t (&v)[16]) {  // the quants are INT8 operands as they stand
+        const u32x4 lo = i8_shift2(r.a.x, r.a.y, r.a.z, r.a.w, r.b.x), hi = i8_shift2(r.b.x, r.b.y, r.b.z, r.b.w, r.c.x);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[i] = lo[i];
+            v[4 + i] = hi[i];
+        }
+        v[8] = r.c.y; v[9] = r.c.z; v[10] = r.c.w; v[11] = r.d.x; v[12] = r.d.y; v[13] = r.d.z; v[14] = r.d.w; v[15] = r.e;
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int, Scale &sc) {
+        sc.d0 = h2f(r.a.x);
+        sc.d1 = h2f(r.c.x >> 16);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&)[NSUM]) {
+        return __builtin_fmaf(sc.d0, i8_combine_wide(d[0]), sc.d1 * i8_combine_wide(d[1])) * sinv;
+    }
+};
+
+// The partial sums of a turn for B activation rows: the operands and scales of the weights are made once, every row runs its
+// chains of products (the chains of a row interleaved, so that a product never waits for the one before it).
+template <class U, int B>
+__device__ __forceinline__ void i8_dot(const typename U::Raw &r, int c, const uint32_t (&xa)[B][16], const float (&sinv)[B], const float (&s)[B][U::NSUM],
+                                       float (&out)[B]) {
+    constexpr int CH = U::CH, L = 16 / CH;
+    uint32_t v[16];
+    U::extract(r, c, v);
+    typename U::Scale sc;
+    U::scales(r, c, sc);
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+        i32x4 d[CH];
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) d[ch] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < L; ++i)
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch) d[ch] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[b][ch * L + i], (int)v[ch * L + i], d[ch], 0, 0, 0);
+        out[b] = U::finish(sc, d, sinv[b], s[b]);
+    }
+}
+
 // -------------------------------------------------------------------------------------------------- the kernel body
-template <class U, int PF, bool BIAS, bool NORM, bool DUAL>
-__device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, const int nblocks) {
-    constexpr int FMT = U::FMT, NB = PF + 1, FL = I8_FLUSH;
+// rb: the first activation row of this workgroup (launches of more than B rows put the row groups of B along blockIdx.y:
+// their workgroups stream the same weight bytes at the same time, so one of them finds them in the cache)
+template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL>
+__device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, const int nblocks, const int rb = 0) {
+    constexpr int FMT = U::FMT, NB = PF + 1, FL = i8_flush(B);
     static_assert(FL % NB == 0 && FL % 2 == 0, "whole rings (and gate/up pairs) per flush window");
+    static_assert(B == 1 || (!NORM && !DUAL), "the fused norm and the SwiGLU pair are batch-1 launches");
     extern __shared__ __align__(16) uint8_t i8_smem[];
     __shared__ float red[I8_MAX_WAVES];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
-    u32x4 *const planes = reinterpret_cast<u32x4 *>(i8_smem + (size_t)wave * I8_LDS_PER_WAVE);
-    float *const mypart = reinterpret_cast<float *>(planes);  // after the staging: [2][FL][4 dpp rows][4 rows] partial sums of this wave
+    constexpr size_t WAVE_LDS = gemv_i8_lds_per_wave(B);
+    u32x4 *const planes = reinterpret_cast<u32x4 *>(i8_smem + (size_t)wave * WAVE_LDS);
+    float *const mypart = reinterpret_cast<float *>(planes);  // after the staging: [2][FL][B][4 dpp rows][4 rows] partial sums of this wave
     const int b = lane >> 2, j = lane & 3;
     const int k = a.k, chunks = k >> 6;
     const int n = a.n[0] + a.n[1] + a.n[2];
@@ -298,13 +469,18 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
     const int turns = (groups + nblocks - 1) / nblocks;  // row groups this workgroup takes (the last may be missing)
     const int vturns = DUAL ? 2 * turns : turns;         // DUAL: a group's gate rows, then its up rows
 
-    // ---- the activations this lane stages: 16 values of chunk c
+    // ---- the activations this lane stages: 16 values of chunk c of every activation row
     const int xf = U::x_first(c, j);
-    float4 xv[4], nv[4];
+    float4 xv[B][4], nv[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        xv[i] = inrow ? reinterpret_cast<const float4 *>(a.x + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        if (NORM) nv[i] = inrow ? reinterpret_cast<const float4 *>(a.nw + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int r = 0; r < B; ++r) {
+        const bool have = inrow && (B == 1 || rb + r < a.rows);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xv[r][i] = have ? reinterpret_cast<const float4 *>(a.x + (size_t)(rb + r) * k + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (NORM) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) nv[i] = inrow ? reinterpret_cast<const float4 *>(a.nw + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
     // ---- the ring of weight bytes
@@ -343,39 +519,44 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
         // barrier that precedes the first outputs anyway.
         float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ss += (xv[i].x * xv[i].x + xv[i].y * xv[i].y) + (xv[i].z * xv[i].z + xv[i].w * xv[i].w);
+        for (int i = 0; i < 4; ++i) ss += (xv[0][i].x * xv[0][i].x + xv[0][i].y * xv[0][i].y) + (xv[0][i].z * xv[0][i].z + xv[0][i].w * xv[0][i].w);
         ss = wave_sum(ss);
         if (lane == 0) red[wave] = ss;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) xv[i] = make_float4(xv[i].x * nv[i].x, xv[i].y * nv[i].y, xv[i].z * nv[i].z, xv[i].w * nv[i].w);
+        for (int i = 0; i < 4; ++i)
+            xv[0][i] = make_float4(xv[0][i].x * nv[i].x, xv[0][i].y * nv[i].y, xv[0][i].z * nv[i].z, xv[0][i].w * nv[i].w);
     }
 
-    // ---- fixed point: v = rint(x * s), |v| < 2^22, s a power of two from the chunk's largest magnitude
-    uint32_t am = 0u;
-    float sm = 0.f;
+    // ---- fixed point, row by row: v = rint(x * s), |v| < 2^22, s a power of two from the chunk's largest magnitude
+    uint32_t xa[B][16];
+    float sinv[B], sums[B][U::NSUM];
+    bool slow = false;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        am = max(max(am, max(__float_as_uint(xv[i].x) & 0x7fffffffu, __float_as_uint(xv[i].y) & 0x7fffffffu)),
-                 max(__float_as_uint(xv[i].z) & 0x7fffffffu, __float_as_uint(xv[i].w) & 0x7fffffffu));
-        sm += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
-    }
-    am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
-    am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
-    const bool slow = __builtin_amdgcn_ballot_w64(am >= 0x7f800000u) != 0;                  // an Inf or NaN in this wave's slice
-    const uint32_t eb = max(am >> 23, 22u);
-    const float s = __uint_as_float((275u - min(eb, 254u)) << 23), sinv = __uint_as_float((min(eb, 254u) - 21u) << 23);
-    float s4[4], sums[U::NSUM];
-    s4[0] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x00, 0xF, 0xF, true));  // quad_perm [0,0,0,0]
-    s4[1] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x55, 0xF, 0xF, true));
-    s4[2] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xAA, 0xF, 0xF, true));
-    s4[3] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xFF, 0xF, 0xF, true));
-    U::sums(s4, sums);
-    uint32_t xa[16];
-    if (!slow) {
+    for (int r = 0; r < B; ++r) {
+        uint32_t am = 0u;
+        float sm = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            am = max(max(am, max(__float_as_uint(xv[r][i].x) & 0x7fffffffu, __float_as_uint(xv[r][i].y) & 0x7fffffffu)),
+                     max(__float_as_uint(xv[r][i].z) & 0x7fffffffu, __float_as_uint(xv[r][i].w) & 0x7fffffffu));
+            sm += (xv[r][i].x + xv[r][i].y) + (xv[r][i].z + xv[r][i].w);
+        }
+        am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+        am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+        slow = slow || __builtin_amdgcn_ballot_w64(am >= 0x7f800000u) != 0;                    // an Inf or NaN in this wave's slice
+        const uint32_t eb = min(max(am >> 23, 22u), 254u);
+        const float s = __uint_as_float((275u - eb) << 23);
+        sinv[r] = __uint_as_float((eb - 21u) << 23);
+        float s4[4];
+        s4[0] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x00, 0xF, 0xF, true));  // quad_perm [0,0,0,0]
+        s4[1] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x55, 0xF, 0xF, true));
+        s4[2] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xAA, 0xF, 0xF, true));
+        s4[3] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xFF, 0xF, 0xF, true));
+        U::sums(s4, sums[r]);
         uint32_t pl[3][4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float f[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+            const float f[4] = {xv[r][i].x, xv[r][i].y, xv[r][i].z, xv[r][i].w};
             uint32_t u[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) u[e] = __float_as_uint(__builtin_fmaf(f[e], s, 12582912.f)) + (0x00808080u - 0x4B400000u);
@@ -386,6 +567,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
             const uint32_t w01 = __builtin_amdgcn_perm(u[1], u[0], 0x00000602u), w23 = __builtin_amdgcn_perm(u[3], u[2], 0x00000602u);
             pl[2][i] = __builtin_amdgcn_perm(w23, w01, 0x05040100u) ^ 0x80808080u;
         }
+        // (a row that is not finite leaves garbage here; the slow path below does not read it)
 #pragma unroll
         for (int p = 0; p < 3; ++p) planes[(b * 3 + p) * 4 + j] = u32x4{pl[p][0], pl[p][1], pl[p][2], pl[p][3]};
         // (the LDS accesses of a wave complete in order: its reads below see its writes above without a barrier)
@@ -394,28 +576,28 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
             const u32x4 v = planes[(b * 3 + p) * 4 + qd];
-            xa[qd * 4 + 0] = v.x; xa[qd * 4 + 1] = v.y; xa[qd * 4 + 2] = v.z; xa[qd * 4 + 3] = v.w;
+            xa[r][qd * 4 + 0] = v.x; xa[r][qd * 4 + 1] = v.y; xa[r][qd * 4 + 2] = v.z; xa[r][qd * 4 + 3] = v.w;
         }
         __builtin_amdgcn_wave_barrier();
     }
 
     auto group_of = [&](int t) { return bid + (DUAL ? t >> 1 : t) * nblocks; };
-    // one output of the window that started at turn t0: the partial sums of all waves in wave order
-    auto joined = [&](int half, int tt, int jj) {
+    // one output of a window: the partial sums of all waves in wave order
+    auto joined = [&](int half, int tt, int r, int jj) {
         float sum = 0.f;
         for (int w = 0; w < waves; ++w) {
-            const float *p = reinterpret_cast<const float *>(i8_smem + (size_t)w * I8_LDS_PER_WAVE) + (half * FL + tt) * 16 + jj;
+            const float *p = reinterpret_cast<const float *>(i8_smem + (size_t)w * WAVE_LDS) + ((half * FL + tt) * B + r) * 16 + jj;
             sum += (p[0] + p[4]) + (p[8] + p[12]);
         }
         return sum;
     };
 
     // a turn's partial sums of this wave: fold the sixteen chunks of every row (lanes 4b + j, b = 0..15) to four per row
-    auto emit = [&](float acc, int half, int tt) {
+    auto emit = [&](float acc, int half, int tt, int r) {
         if (!inrow) acc = 0.f;
         acc += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc), 0x114, 0xF, 0xF, true));  // row_shr:4
         acc += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(acc), 0x118, 0xF, 0xF, true));  // row_shr:8
-        if ((lane & 15) >= 12) mypart[(half * FL + tt) * 16 + (lane >> 4) * 4 + j] = acc;
+        if ((lane & 15) >= 12) mypart[((half * FL + tt) * B + r) * 16 + (lane >> 4) * 4 + j] = acc;
     };
 
     for (int t0 = 0, half = 0; t0 < vturns; t0 += FL, half ^= 1) {
@@ -426,7 +608,12 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
                     const int t = tb + i;
-                    if (t < tend && group_of(t) < groups) emit(U::dot(buf[i], c, xa, sinv, sums), half, t - t0);  // wave-uniform
+                    if (t < tend && group_of(t) < groups) {  // wave-uniform
+                        float acc[B];
+                        i8_dot<U, B>(buf[i], c, xa, sinv, sums, acc);
+#pragma unroll
+                        for (int r = 0; r < B; ++r) emit(acc[r], half, t - t0, r);
+                    }
                     fill(buf[i], t + NB);
                 }
             }
@@ -441,22 +628,27 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
                 const bool in1 = row >= n0, in2 = row >= n01;
                 const uint8_t *rp = (DUAL ? ((t & 1) ? wd : w0) : w0 + (in1 ? d01 : 0) + (in2 ? d12 : 0)) +
                                     (size_t)(row - (in1 ? n0 : 0) - (in2 ? n01 - n0 : 0)) * rowbytes;
-                float acc = 0.f;
 #pragma unroll 1
-                for (int e = 0; e < 64; e += 4) {
-                    const int p = U::x_pos(c, e);
-                    const float4 w4 = dequant4<FMT>(rp, (size_t)p);
-                    float4 x4 = *reinterpret_cast<const float4 *>(a.x + p);
-                    if (NORM) {
-                        const float4 n4 = *reinterpret_cast<const float4 *>(a.nw + p);
-                        x4 = make_float4(x4.x * n4.x, x4.y * n4.y, x4.z * n4.z, x4.w * n4.w);
+                for (int r = 0; r < B; ++r) {
+                    float acc = 0.f;
+                    if (B == 1 || rb + r < a.rows) {
+#pragma unroll 1
+                        for (int e = 0; e < 64; e += 4) {
+                            const int p = U::x_pos(c, e);
+                            const float4 w4 = dequant4<FMT>(rp, (size_t)p);
+                            float4 x4 = *reinterpret_cast<const float4 *>(a.x + (size_t)(rb + r) * k + p);
+                            if (NORM) {
+                                const float4 n4 = *reinterpret_cast<const float4 *>(a.nw + p);
+                                x4 = make_float4(x4.x * n4.x, x4.y * n4.y, x4.z * n4.z, x4.w * n4.w);
+                            }
+                            acc = __builtin_fmaf(w4.x, x4.x, acc);
+                            acc = __builtin_fmaf(w4.y, x4.y, acc);
+                            acc = __builtin_fmaf(w4.z, x4.z, acc);
+                            acc = __builtin_fmaf(w4.w, x4.w, acc);
+                        }
                     }
-                    acc = __builtin_fmaf(w4.x, x4.x, acc);
-                    acc = __builtin_fmaf(w4.y, x4.y, acc);
-                    acc = __builtin_fmaf(w4.z, x4.z, acc);
-                    acc = __builtin_fmaf(w4.w, x4.w, acc);
+                    emit(acc, half, t - t0, r);
                 }
-                emit(acc, half, t - t0);
             }
         }
         __syncthreads();  // (one barrier per window: the next window writes the other half of the partial-sum area)
@@ -466,44 +658,44 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
             for (int w = 0; w < waves; ++w) tot += red[w];
             nscale = 1.f / sqrtf(tot / (float)k + a.eps);
         }
-        const int outs = DUAL ? 2 * (tend - t0) : 4 * (tend - t0);
+        const int outs = DUAL ? 2 * (tend - t0) : 4 * B * (tend - t0);
         for (int o = tid; o < outs; o += (int)blockDim.x) {  // (a one-wave workgroup has fewer threads than a window has outputs)
             if (DUAL) {
                 const int pr = o >> 2, jj = o & 3;
                 const int g = group_of(t0 + 2 * pr), row = min(4 * g, n - 4) + jj;
                 if (g < groups && row >= 4 * g) {
-                    const float gate = joined(half, 2 * pr, jj) * nscale, up = joined(half, 2 * pr + 1, jj) * nscale;
+                    const float gate = joined(half, 2 * pr, 0, jj) * nscale, up = joined(half, 2 * pr + 1, 0, jj) * nscale;
                     a.y[0][row] = (gate / (1.f + __expf(-gate))) * up;
                 }
             } else {
-                const int tt = o >> 2, jj = o & 3;
+                const int jj = o & 3, r = (o >> 2) % B, tt = (o >> 2) / B;
                 const int g = group_of(t0 + tt), row = min(4 * g, n - 4) + jj;
-                if (g < groups && row >= 4 * g) {
+                if (g < groups && row >= 4 * g && (B == 1 || rb + r < a.rows)) {
                     // (segment pointers by differences, as in fill: no dependent load from the argument block on the way out)
                     const bool in1 = row >= a.n[0], in2 = row >= a.n[0] + a.n[1];
                     const int local = row - (in1 ? a.n[0] : 0) - (in2 ? a.n[1] : 0);
                     float *const yp = a.y[0] + (in1 ? a.y[1] - a.y[0] : 0) + (in2 ? a.y[2] - a.y[1] : 0);
                     float bias = 0.f;
                     if (BIAS) bias = (a.bias[0] + (in1 ? a.bias[1] - a.bias[0] : 0) + (in2 ? a.bias[2] - a.bias[1] : 0))[local];
-                    const float sum = NORM ? joined(half, tt, jj) * nscale : joined(half, tt, jj);
-                    yp[local] = BIAS ? sum + bias : sum;
+                    const float sum = NORM ? joined(half, tt, r, jj) * nscale : joined(half, tt, r, jj);
+                    yp[(size_t)(rb + r) * n + local] = BIAS ? sum + bias : sum;
                 }
             }
         }
     }
 }
 
-template <class U, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
-__global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_kernel(const I8Args a) {
-    gemv_i8_body<U, PF, BIAS, NORM, DUAL>(a, blockIdx.x, gridDim.x);
+template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
+__global__ void __launch_bounds__(64 * MAXW, (B > 1 ? 2 : 4)) gemv_i8_kernel(const I8Args a) {
+    gemv_i8_body<U, B, PF, BIAS, NORM, DUAL>(a, blockIdx.x, gridDim.x, B * (int)blockIdx.y);
 }
 
 // Two sets of matrices in two formats over the same (normalised) activations in one launch - the q / k and the v
 // projections of a Q4_K_M layer: workgroups below `split` run the first set, the others the second.
 template <class UA, class UB, int PF, int MAXW>
 __global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_pair_kernel(const I8Args a, const I8Args b, const int split) {
-    if ((int)blockIdx.x < split) gemv_i8_body<UA, PF, false, true, false>(a, blockIdx.x, split);
-    else gemv_i8_body<UB, PF, false, true, false>(b, blockIdx.x - split, gridDim.x - split);
+    if ((int)blockIdx.x < split) gemv_i8_body<UA, 1, PF, false, true, false>(a, blockIdx.x, split);
+    else gemv_i8_body<UB, 1, PF, false, true, false>(b, blockIdx.x - split, gridDim.x - split);
 }
 
 }  // namespace jitnn

@@ -4,7 +4,9 @@
 
 namespace jitnn {
 
+// K-quants; the 32-value formats with rows of whole pairs of blocks (their matrices on dword boundaries: the caller checks)
 bool gemv_i8_supported(int fmt, int k) {
+    if (fmt == F_Q4_0 || fmt == F_Q4_1 || fmt == F_Q8_0) return k % 64 == 0 && k >= 64 && k <= 1024 * I8_MAX_WAVES;
     return (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K) && k % 256 == 0 && k >= 256 && k <= 1024 * I8_MAX_WAVES;
 }
 
@@ -13,28 +15,35 @@ typedef void (*i8_fn)(const I8Args);
 template <class U, int PF, int MAXW>
 static i8_fn pick_mode(int mode) {
     switch (mode) {
-    case I8_BIAS: return gemv_i8_kernel<U, PF, true, false, false, MAXW>;
-    case I8_NORM: return gemv_i8_kernel<U, PF, false, true, false, MAXW>;
-    case I8_DUAL: return gemv_i8_kernel<U, PF, false, true, true, MAXW>;
-    default: return gemv_i8_kernel<U, PF, false, false, false, MAXW>;
+    case I8_BIAS: return gemv_i8_kernel<U, 1, PF, true, false, false, MAXW>;
+    case I8_NORM: return gemv_i8_kernel<U, 1, PF, false, true, false, MAXW>;
+    case I8_DUAL: return gemv_i8_kernel<U, 1, PF, false, true, true, MAXW>;
+    default: return gemv_i8_kernel<U, 1, PF, false, false, false, MAXW>;
     }
 }
 
 template <class U, int MAXW>
 static i8_fn pick_pf(int mode, int pf) {
-    if constexpr (U::FMT == F_Q5_K) return pf <= 1 ? pick_mode<U, 1, MAXW>(mode) : pick_mode<U, 2, MAXW>(mode);
+    if constexpr (U::FMT == F_Q5_K || U::FMT == F_Q8_0) return pf <= 1 ? pick_mode<U, 1, MAXW>(mode) : pick_mode<U, 2, MAXW>(mode);  // (five loads a turn: a fourth buffer does not fit 128 registers)
     else return pf <= 1 ? pick_mode<U, 1, MAXW>(mode) : pf == 2 ? pick_mode<U, 2, MAXW>(mode) : pick_mode<U, 3, MAXW>(mode);
 }
 
-template <int MAXW>
-static i8_fn pick_fmt(int fmt, int mode, int pf, bool q6_aligned) {
-    switch (fmt) {
-    case F_Q4_K: return pick_pf<U8<F_Q4_K>, MAXW>(mode, pf);
-    case F_Q5_K: return pick_pf<U8<F_Q5_K>, MAXW>(mode, pf < 2 ? pf : 2);  // (five loads a turn: a fourth buffer does not fit 128 registers)
-    case F_Q6_K: return q6_aligned ? pick_pf<U8Q6<true>, MAXW>(mode, pf) : pick_pf<U8Q6<false>, MAXW>(mode, pf);
-    default: return nullptr;
-    }
+// two activation rows, rows of at most 4096 values (the body takes any number; more than two are not instantiated: from three
+// rows on the 16-row tiles of gemv_mfma_kernel are faster)
+template <class U, int B>
+static i8_fn pick_batch(int mode, int pf) {
+    if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, B, 1, true, false, false, 4> : gemv_i8_kernel<U, B, 2, true, false, false, 4>;
+    return pf <= 1 ? gemv_i8_kernel<U, B, 1, false, false, false, 4> : gemv_i8_kernel<U, B, 2, false, false, false, 4>;
 }
+
+template <class U>
+static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
+    if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_pf<U, I8_MAX_WAVES>(mode, pf);
+    if (waves > 4 || rows > 2 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
+    return pick_batch<U, 2>(mode, pf);
+}
+
+static int batch_of(int rows) { return rows == 1 ? 1 : 2; }
 
 // Q6_K rows a multiple of four bytes long in matrices on dword boundaries take the variant with dword-aligned loads
 static bool q6_aligned(const I8Args &a) {
@@ -44,11 +53,20 @@ static bool q6_aligned(const I8Args &a) {
 }
 
 void gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a) {
-    const int waves = (a.k + 1023) / 1024;
-    const bool al = fmt == F_Q6_K && q6_aligned(a);
-    const i8_fn fn = waves <= 4 ? pick_fmt<4>(fmt, mode, pf, al) : pick_fmt<I8_MAX_WAVES>(fmt, mode, pf, al);
+    const int waves = (a.k + 1023) / 1024, rows = a.rows < 1 ? 1 : a.rows;
+    i8_fn fn = nullptr;
+    switch (fmt) {
+    case F_Q4_K: fn = pick_rows<U8<F_Q4_K>>(rows, waves, mode, pf); break;
+    case F_Q5_K: fn = pick_rows<U8<F_Q5_K>>(rows, waves, mode, pf); break;
+    case F_Q4_0: fn = pick_rows<U8<F_Q4_0>>(rows, waves, mode, pf); break;
+    case F_Q4_1: fn = pick_rows<U8<F_Q4_1>>(rows, waves, mode, pf); break;
+    case F_Q8_0: fn = pick_rows<U8<F_Q8_0>>(rows, waves, mode, pf); break;
+    case F_Q6_K: fn = q6_aligned(a) ? pick_rows<U8Q6<true>>(rows, waves, mode, pf) : pick_rows<U8Q6<false>>(rows, waves, mode, pf); break;
+    default: break;
+    }
     if (!fn) return;
-    hipLaunchKernelGGL(fn, dim3(blocks), dim3(64 * waves), gemv_i8_lds_bytes(waves), s, a);
+    const int bt = batch_of(rows);
+    hipLaunchKernelGGL(fn, dim3(blocks, (rows + bt - 1) / bt), dim3(64 * waves), gemv_i8_lds_bytes(waves, bt), s, a);
 }
 
 typedef void (*i8_pair_fn)(const I8Args, const I8Args, int);

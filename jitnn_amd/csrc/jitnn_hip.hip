@@ -260,6 +260,7 @@ bool i8_ok(const XregCall &c) {
         if (!c.w[i]) continue;
         n += c.w[i]->n;
         if (c.w[i]->nbytes >= (1ll << 32) || (c.w[1] && c.w[i]->n % 4 != 0)) return false;
+        if (block_values(c.w[i]->fmt) == 32 && ((uintptr_t)c.w[i]->dev & 3) != 0) return false;  // (pairs of 32-value blocks are fetched as dwords)
     }
     if (c.w2 && c.w2->nbytes >= (1ll << 32)) return false;
     return n >= 4;
@@ -279,6 +280,7 @@ int i8_args(const XregCall &c, I8Args &a) {
     a.nw = c.norm_w;
     a.eps = c.eps;
     a.k = c.w[0]->k;
+    a.rows = 1;
     return n;
 }
 
@@ -302,6 +304,34 @@ int launch_i8(const XregCall &c, hipStream_t stream) {
     i8_shape((n + 3) / 4, (a.k + 1023) / 1024, c.w2 != nullptr, blocks, pf);
     if (c.w[0]->fmt == F_Q5_K && pf > 2) pf = 2;  // (five loads per turn: a fourth buffer does not fit 128 registers)
     gemv_i8_launch(c.w[0]->fmt, mode, pf, (unsigned)blocks, stream, a);
+    HIP_TRY(hipGetLastError());
+    return JITNN_HIP_OK;
+}
+
+// Two activation rows of a K-quant weight with rows of at most 4096 values: the same kernel with the activations of both rows
+// in registers (Q4_K 14336 x 4096: 10.2 us against 11.3 for the two-row FP32 register kernel).  The kernel is written for any
+// number of rows, but its 4x4x4 products cost about 16 cycles each whatever they multiply: with four rows (64 products a
+// turn) it measured 13.5 us, with eight (two groups of four) 20.4 - gemv_mfma_kernel's 16-row tiles stay ahead from three rows on.
+bool i8_batch_ok(const jitnn_hip_weight *w, int rows) {
+    return g.gemv_i8 && rows == 2 && gemv_i8_supported(w->fmt, w->k) && w->k <= 4096 && w->n >= 4 && w->nbytes < (1ll << 32) &&
+           (block_values(w->fmt) != 32 || ((uintptr_t)w->dev & 3) == 0);
+}
+
+int launch_i8_batch(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
+    I8Args a{};
+    for (int i = 0; i < 3; ++i) {
+        a.w[i] = w->dev;
+        a.y[i] = y;
+        a.bias[i] = bias;
+    }
+    a.n[0] = w->n;
+    a.x = x;
+    a.k = w->k;
+    a.rows = rows;
+    const int groups = (w->n + 3) / 4;
+    const int per_cu = 2, pf = 1;
+    const int blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
+    gemv_i8_launch(w->fmt, bias ? I8_BIAS : I8_PLAIN, pf, (unsigned)blocks, stream, a);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
@@ -498,6 +528,7 @@ int launch_gemv_plain(const jitnn_hip_weight *w, const float *x, int rows, const
 
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
     if (is_extra_format(w->fmt)) return launch_gemv_plain(w, x, rows, bias, y, stream);
+    if (i8_batch_ok(w, rows)) return launch_i8_batch(w, x, rows, bias, y, stream);
     if (rows == 2 && w->k <= 4096) return launch_gemv_xreg_b2(w, x, bias, y, stream);
     // Q6_K pays the most per weight on the matrix-core path (6-bit quants from two arrays, 16-value scale groups): up to
     // four rows its FP32 kernel is still ahead (measured: 33 vs 43 us at 2 rows, 151 vs 167 us at 4 rows on the output head)

@@ -102,15 +102,17 @@ struct I8Args {
     const float *bias[3];  // BIAS: added to the segment's rows (a residual rides here)
     int n[3];
     const uint8_t *w2;
-    const float *x;   // [k]
+    const float *x;   // [rows, k]
     const float *nw;  // NORM: RMSNorm weight [k]
     float eps;
     int k;
+    int rows;  // activation rows (x [rows, k], y [rows, n]); more than one: a single matrix, no norm, no pair
 };
 
 constexpr int I8_PLAIN = 0, I8_BIAS = 1, I8_NORM = 2, I8_DUAL = 3;  // DUAL: norm + the SwiGLU pair
 bool gemv_i8_supported(int fmt, int k);
-// blockDim = 64 * ceil(k / 1024); pf = turns of weight bytes in flight per wave beyond the one being multiplied (1..3)
+// blockDim = 64 * ceil(k / 1024); pf = turns of weight bytes in flight per wave beyond the one being multiplied (1..3; 1..2 for
+// two activation rows - a.rows == 2, rows of at most 4096 values, modes I8_PLAIN and I8_BIAS only)
 void gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a);
 bool gemv_i8_pair_supported(int fmt_a, int fmt_b);
 void gemv_i8_pair_launch(int fmt_a, int fmt_b, int pf, unsigned blocks_a, unsigned blocks_b, hipStream_t s, const I8Args &a, const I8Args &b);
