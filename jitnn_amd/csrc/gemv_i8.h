@@ -490,9 +490,12 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
     // arithmetic, and no branch - with conditional loads the compiler cannot count the loads in flight.
     // (the segment's matrix by differences: a choice among three pointers by two conditions gets compiled into a table in
     // private memory)
+    // Row segments (several matrices in one launch) exist only where the decode step uses them: with the fused norm.  Every other
+    // launch has one matrix, and its per-turn scalar arithmetic - which a wave alone on its SIMD pays in full - stays short.
+    constexpr bool SEGMENTS = NORM && !DUAL;
     const uint8_t *const w0 = a.w[0], *const wd = a.w2;
-    const ptrdiff_t d01 = a.w[1] - a.w[0], d12 = a.w[2] - a.w[1];
-    const int n0 = a.n[0], n01 = a.n[0] + a.n[1];
+    const ptrdiff_t d01 = SEGMENTS ? a.w[1] - a.w[0] : 0, d12 = SEGMENTS ? a.w[2] - a.w[1] : 0;
+    const int n0 = SEGMENTS ? a.n[0] : n, n01 = SEGMENTS ? a.n[0] + a.n[1] : n;
     auto fill = [&](typename U::Raw &dst, int t) {
         const int g = bid + (DUAL ? t >> 1 : t) * nblocks;
         // extent of the descriptor: everything for a group that exists, nothing past the last group (turns at or past
@@ -501,7 +504,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
         // load then runs in a loop over the descriptor values the lanes hold)
         const int extent = __builtin_amdgcn_readfirstlane((g - groups) >> 31);
         const int r0 = min(4 * g, n - 4);
-        const bool in1 = r0 >= n0, in2 = r0 >= n01;
+        const bool in1 = SEGMENTS && r0 >= n0, in2 = SEGMENTS && r0 >= n01;
         const uint8_t *base = w0 + (in1 ? d01 : 0) + (in2 ? d12 : 0);
         if (DUAL) base = (t & 1) ? wd : w0;
         const int local = r0 - (in1 ? n0 : 0) - (in2 ? n01 - n0 : 0);
@@ -625,7 +628,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
                 const int g = group_of(t);
                 if (g >= groups) continue;
                 const int row = min(4 * g, n - 4) + j;
-                const bool in1 = row >= n0, in2 = row >= n01;
+                const bool in1 = SEGMENTS && row >= n0, in2 = SEGMENTS && row >= n01;
                 const uint8_t *rp = (DUAL ? ((t & 1) ? wd : w0) : w0 + (in1 ? d01 : 0) + (in2 ? d12 : 0)) +
                                     (size_t)(row - (in1 ? n0 : 0) - (in2 ? n01 - n0 : 0)) * rowbytes;
 #pragma unroll 1
@@ -672,7 +675,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
                 const int g = group_of(t0 + tt), row = min(4 * g, n - 4) + jj;
                 if (g < groups && row >= 4 * g && (B == 1 || rb + r < a.rows)) {
                     // (segment pointers by differences, as in fill: no dependent load from the argument block on the way out)
-                    const bool in1 = row >= a.n[0], in2 = row >= a.n[0] + a.n[1];
+                    const bool in1 = SEGMENTS && row >= a.n[0], in2 = SEGMENTS && row >= a.n[0] + a.n[1];
                     const int local = row - (in1 ? a.n[0] : 0) - (in2 ? a.n[1] : 0);
                     float *const yp = a.y[0] + (in1 ? a.y[1] - a.y[0] : 0) + (in2 ? a.y[2] - a.y[1] : 0);
                     float bias = 0.f;

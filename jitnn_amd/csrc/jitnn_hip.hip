@@ -263,6 +263,7 @@ bool i8_ok(const XregCall &c) {
         if (block_values(c.w[i]->fmt) == 32 && ((uintptr_t)c.w[i]->dev & 3) != 0) return false;  // (pairs of 32-value blocks are fetched as dwords)
     }
     if (c.w2 && c.w2->nbytes >= (1ll << 32)) return false;
+    if (c.w[1] && (!c.norm_w || c.w2)) return false;  // (several matrices in one launch: the kernel has that for the fused norm only)
     return n >= 4;
 }
 
