@@ -85,6 +85,8 @@ class Workload:
         self.y = torch.zeros(b, n, device="cuda")
         self.bytes = alg_bytes(fmt, n, k, b)
         self._xp, self._yp = C.c_void_p(self.x.data_ptr()), C.c_void_p(self.y.data_ptr())
+        torch.cuda.synchronize()
+        self.stream = torch.cuda.Stream()  # the timed launches and their events go on a stream of their own, not the legacy default stream
 
     def step(self, i: int, stream) -> None:
         rc = self.lib.lib.jitnn_hip_linear_dev(self.handles[i % len(self.handles)], self._xp, self.b, None, self._yp, stream)
@@ -95,6 +97,11 @@ class Workload:
         """(wall seconds, event seconds) for `steps` back-to-back launches after `warmup` untimed ones;
         rotate=False keeps to one weight copy (cache-resident figure)."""
         torch = self.torch
+        with torch.cuda.stream(self.stream):
+            return self._time(steps, warmup, rotate)
+
+    def _time(self, steps: int, warmup: int, rotate: bool):
+        torch = self.torch
         stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         m = 1 if rotate else 0
         # every weight copy gets one untimed launch first: the first kernel touch of an allocation pays for its address
@@ -103,15 +110,21 @@ class Workload:
             self.step(i, stream)
         for i in range(warmup):
             self.step(i * m, stream)
+        # the timed loop calls the C ABI with everything bound beforehand, so that the host stays ahead of a 6-8 us kernel
+        f, xp, yp, b = self.lib.lib.jitnn_hip_linear_dev, self._xp, self._yp, self.b
+        order = [self.handles[(i * m) % len(self.handles)] for i in range(steps)]
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
+        rc = 0
         t0 = time.perf_counter()
         e0.record()
-        for i in range(steps):
-            self.step(i * m, stream)
+        for h in order:
+            rc |= f(h, xp, b, None, yp, stream)
         e1.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
+        if rc != 0:
+            self.lib.check(rc, "jitnn_hip_linear_dev")
         return t1 - t0, e0.elapsed_time(e1) * 1e-3
 
     def time_streams(self, steps: int, nstreams: int = 4):
@@ -142,21 +155,42 @@ class Workload:
         return {"streams": nstreams, "steps": steps, "us_per_launch": dt / steps * 1e6, "GBps": self.bytes * steps / dt / 1e9,
                 "pct_of_peak": self.bytes * steps / dt / 1e9 / PEAK_HBM_GBPS * 100, "results_equal_across_streams": same}
 
-    def read_probe(self, steps: int):
-        """Microseconds per launch of a pure 128-bit streaming read over the same weight bytes, rotating like time()."""
+    def read_probe(self, steps: int, shape=None):
+        """Microseconds per launch of a pure 128-bit streaming read over the same weight bytes, rotating like time();
+        shape = (workgroups per CU, loads in flight per lane, non-temporal) or None for the library's default shape."""
         torch = self.torch
         stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         ptrs = [(C.c_void_p(t.data_ptr()), t.numel()) for t in self.weights]
-        for i in range(10):
-            self.lib.lib.jitnn_hip_probe_read_dev(ptrs[i % len(ptrs)][0], ptrs[i % len(ptrs)][1], stream)
+
+        def launch(i):
+            p, nb = ptrs[i % len(ptrs)]
+            rc = (self.lib.lib.jitnn_hip_probe_read_dev(p, nb, stream) if shape is None
+                  else self.lib.lib.jitnn_hip_probe_read_shape_dev(p, nb, shape[0], shape[1], shape[2], stream))
+            if rc != 0:
+                self.lib.check(rc, "jitnn_hip_probe_read")
+        for i in range(len(ptrs) + 10):
+            launch(i)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         e0.record()
         for i in range(steps):
-            self.lib.lib.jitnn_hip_probe_read_dev(ptrs[i % len(ptrs)][0], ptrs[i % len(ptrs)][1], stream)
+            launch(i)
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / steps
+
+    def read_probe_sweep(self, steps: int = 400):
+        """The pure read over launch shapes: workgroups per CU x 16-byte loads in flight per lane x (non-)temporal loads.
+        Returns the list of (shape, us) and the fastest - the ceiling a launch that only reads these bytes reaches here."""
+        rows = []
+        for wg in (1, 2, 4, 8, 16):
+            for u in (1, 2, 4, 8, 16):
+                if wg * u > 32:   # (more than 128 KiB in flight per CU: measured slower every time, not swept)
+                    continue
+                for nt in (0, 1):
+                    rows.append({"workgroups_per_cu": wg, "loads_in_flight": u, "nontemporal": nt, "us": self.read_probe(steps, (wg, u, nt))})
+        best = min(rows, key=lambda r: r["us"])
+        return rows, best
 
     def parity(self, rows: int = 192):
         """Normalised max error of the device result against the CPU oracle on a spread of output rows."""
@@ -184,11 +218,12 @@ class Workload:
 def measure(torch, lib, fmt, n, k, b, copies, steps, warmup, seed, parity=True):
     wl = Workload(torch, lib, fmt, n, k, b, copies, seed)
     err = wl.parity() if parity else None
+    # the kernel's average launch duration for the roofline: a fixed, well-sampled event region whatever --steps is, behind
+    # enough untimed launches for the device to have left its idle clocks (a region that starts cold reads 5 % slower)
+    roof_launches = max(steps, 2000 if n < 100000 else 300)
+    _, roof_ev = wl.time(roof_launches, max(warmup, roof_launches // 4))
     wall, ev = wl.time(steps, warmup)
-    # the kernel's average launch duration for the roofline: a fixed, well-sampled event region, whatever --steps is
-    roof_launches = max(steps, 1000 if n < 100000 else 200)
-    _, roof_ev = (wall, ev) if roof_launches == steps else wl.time(roof_launches, 0)
-    probe_us = wl.read_probe(min(steps, 400))
+    probe_us = wl.read_probe(400 if n < 100000 else 100)
     out = {"workload": f"{fmt} GEMV {n}x{k} batch {b}", "copies": copies, "steps": steps, "bytes_per_step": wl.bytes,
            "pure_read_us_per_launch": probe_us, "pure_read_GBps": wl.weights[0].numel() / probe_us / 1e3,
            "us_per_step_wall": wall / steps * 1e6, "us_per_step_events": ev / steps * 1e6, "GBps": wl.bytes * steps / wall / 1e9,
@@ -618,8 +653,9 @@ def main() -> int:
 
     # ---- headline: Q4_K 14336x4096 batch 1, rotating over 16 copies
     wl, head = measure(torch, lib, "Q4_K", 14336, 4096, 1, 16, a.steps, a.warmup, seed=1030)
-    hot_wall, hot_ev = wl.time(min(a.steps, 2000), 50, rotate=False)
-    sustained = wl.time_streams(min(a.steps, 2000), 4)
+    sweep, best = ([], None) if a.quick else wl.read_probe_sweep()
+    hot_wall, hot_ev = wl.time(2000, 50, rotate=False)
+    sustained = wl.time_streams(2000, 4)
     cpu = None if a.no_cpu else cpu_baseline(wl, 3.0 if a.quick else 8.0)
     host = host_path(torch, lib, wl)
     head_bytes = wl.bytes
@@ -679,8 +715,10 @@ def main() -> int:
         "config": {"workload": "Q4_K GEMV 14336x4096 batch 1 (BASELINE configs[2]), weights N(0,0.02) quantised to Q4_K, x N(0,1); "
                                "16 weight copies rotated per step (528 MB > 256 MB Infinity Cache)",
                    "bytes_per_step": head_bytes, "device": info["name"], "compute_units": info["compute_units"],
-                   "cache_resident_GBps": head_bytes * min(a.steps, 2000) / hot_ev / 1e9, "parity_norm_err": head["parity_norm_err"],
+                   "cache_resident_GBps": head_bytes * 2000 / hot_ev / 1e9, "parity_norm_err": head["parity_norm_err"],
                    "pure_read_GBps": head["pure_read_GBps"], "pure_read_us_per_launch": head["pure_read_us_per_launch"],
+                   "pure_read_best_of_sweep": best, "pure_read_sweep": sweep,
+                   "gemv_over_pure_read": head["us_per_launch_events"] / (best["us"] if best else head["pure_read_us_per_launch"]),
                    "sustained_4_streams": sustained},
         "roofline": {"bound": "hbm", "achieved": head["GBps_events"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
                      "frac": head["GBps_events"] / PEAK_HBM_GBPS, "traffic": headline_traffic_bytes(),

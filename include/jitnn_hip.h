@@ -167,6 +167,11 @@ JITNN_HIP_API int jitnn_hip_stats_reset(void);
  * device gives a pure read of the same bytes, launch included.  The benchmark prints it beside the GEMV figures;
  * it has no counterpart in the reference. */
 JITNN_HIP_API int jitnn_hip_probe_read_dev(const void *dev, long long nbytes, void *stream);
+/* The same with the launch shape given: workgroups of 256 threads per CU (1..16), 16-byte loads in flight per lane (1, 2, 4,
+ * 8, 16), non-temporal loads or not - the benchmark sweeps these to find what a read of a buffer of that size can reach.
+ * jitnn_hip_probe_read_dev uses 8 workgroups per CU with one load in flight each. */
+JITNN_HIP_API int jitnn_hip_probe_read_shape_dev(const void *dev, long long nbytes, int workgroups_per_cu, int loads_in_flight, int nontemporal,
+                                                 void *stream);
 
 /* ---- device memory for callers that have no HIP binding of their own (the Java side) ------------- */
 

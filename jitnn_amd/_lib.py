@@ -51,6 +51,7 @@ def _bind() -> C.CDLL:
         "jitnn_hip_quantize_q8_0": (i, [vp, ll, vp]),
         "jitnn_hip_quantize_q8_0_dev": (i, [vp, ll, vp, vp]),
         "jitnn_hip_probe_read_dev": (i, [vp, ll, vp]),
+        "jitnn_hip_probe_read_shape_dev": (i, [vp, ll, i, i, i, vp]),
         "jitnn_hip_malloc": (i, [ll, C.POINTER(vp)]),
         "jitnn_hip_free": (i, [vp]),
         "jitnn_hip_memcpy_h2d": (i, [vp, vp, ll]),

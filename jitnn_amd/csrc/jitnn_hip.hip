@@ -92,14 +92,18 @@ __global__ void fp8_probe_kernel(float *out) {
 }
 
 // Pure streaming read: every thread xors the 16-byte words it loads; the store can never happen for real data
-// but keeps the loads alive.
+// but keeps the loads alive.  U loads in flight per lane (the workgroups stride the buffer together), NT: non-temporal loads.
+template <int U, bool NT>
 __global__ void __launch_bounds__(256) probe_read_kernel(const u32x4 *__restrict__ p, size_t n16, uint32_t *sink) {
     const size_t stride = (size_t)gridDim.x * 256;
     u32x4 acc = {0, 0, 0, 0};
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        const u32x4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], d = p[i + 3 * stride];
-        acc ^= a ^ b ^ c ^ d;
+    for (; i + (U - 1) * stride < n16; i += U * stride) {
+        u32x4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = NT ? __builtin_nontemporal_load(p + i + u * stride) : p[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= v[u];
     }
     for (; i < n16; i += stride) acc ^= p[i];
     if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) *sink = acc.x;
@@ -1295,12 +1299,27 @@ int jitnn_hip_thread_release(void) {
     return JITNN_HIP_OK;
 }
 
-int jitnn_hip_probe_read_dev(const void *dev, long long nbytes, void *stream) {
+int jitnn_hip_probe_read_shape_dev(const void *dev, long long nbytes, int workgroups_per_cu, int loads_in_flight, int nontemporal, void *stream) {
     if (!dev || nbytes < 16 || ((uintptr_t)dev & 15) != 0) return fail(JITNN_HIP_EINVAL, "need a 16-byte aligned buffer of at least 16 bytes");
+    if (workgroups_per_cu < 1 || workgroups_per_cu > 16) return fail(JITNN_HIP_EINVAL, "%d workgroups per CU", workgroups_per_cu);
     if (int rc = check_ready()) return rc;
-    hipLaunchKernelGGL(probe_read_kernel, dim3(g.cus * 2), dim3(256), 0, (hipStream_t)stream, (const u32x4 *)dev, (size_t)nbytes / 16, (uint32_t *)nullptr);
+    typedef void (*fn_t)(const u32x4 *, size_t, uint32_t *);
+    fn_t fn = nullptr;
+    switch (loads_in_flight) {
+    case 1: fn = nontemporal ? probe_read_kernel<1, true> : probe_read_kernel<1, false>; break;
+    case 2: fn = nontemporal ? probe_read_kernel<2, true> : probe_read_kernel<2, false>; break;
+    case 4: fn = nontemporal ? probe_read_kernel<4, true> : probe_read_kernel<4, false>; break;
+    case 8: fn = nontemporal ? probe_read_kernel<8, true> : probe_read_kernel<8, false>; break;
+    case 16: fn = nontemporal ? probe_read_kernel<16, true> : probe_read_kernel<16, false>; break;
+    default: return fail(JITNN_HIP_EINVAL, "%d loads in flight (1, 2, 4, 8 or 16)", loads_in_flight);
+    }
+    hipLaunchKernelGGL(fn, dim3(g.cus * workgroups_per_cu), dim3(256), 0, (hipStream_t)stream, (const u32x4 *)dev, (size_t)nbytes / 16, (uint32_t *)nullptr);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
+}
+
+int jitnn_hip_probe_read_dev(const void *dev, long long nbytes, void *stream) {
+    return jitnn_hip_probe_read_shape_dev(dev, nbytes, 8, 1, 0, stream);  // the shape a sweep found fastest on 33 MB (6.4 us against 7.5 for 2 x 4)
 }
 
 int jitnn_hip_malloc(long long nbytes, void **dev) {
