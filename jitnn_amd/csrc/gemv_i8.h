@@ -17,8 +17,8 @@
 // partial sums of a turn leave the wave through a two-step DPP fold (16 floats to LDS); every I8_FLUSH turns the
 // workgroup meets at a barrier and one thread per output adds the partial sums in a fixed order - no atomics, the
 // result does not depend on the launch shape.  Weight bytes are prefetched PF turns ahead through a register ring with
-// unconditional loads (turns past the end read one 16-byte piece) so the hardware's in-order load counter is waited on
-// exactly.
+// unconditional loads (turns past the end get a descriptor of extent zero: zeros, no traffic) so the hardware's
+// in-order load counter is waited on exactly.
 //
 // A slice that holds an activation that is not finite takes a slow path (every weight decoded by the bit-exact
 // expression of the dequantiser and multiplied in FP32) so that +-Inf and NaN come out as the reference's FP64 sum

@@ -122,8 +122,9 @@ def test_gemv_vs_oracle(jn, fmt, n, k):
 
 @pytest.mark.parametrize("k", [256, 1024, 4096])
 def test_q6k_many_rows_integer_variant(jn, k):
-    """A Q6_K matrix tall enough that every wave sees 16 rows or more takes the integer variant of the batch-1 kernel
-    (activations as 22-bit fixed point in byte planes, v_dot4): same bar, and in fact FP32-grade error, on ordinary,
+    """A tall Q6_K matrix (many turns per workgroup, a row count that is no multiple of four) through the INT8
+    matrix-core kernel - activations as 22-bit fixed point in three byte planes - with rows of 256 (one wave, more
+    outputs per flush than threads), 1024 and longer: same bar, and in fact FP32-grade error, on ordinary,
     outlier-ridden, tiny, partly zero and unit-vector activations, with and without bias."""
     from oracle import oracle
     rng = np.random.default_rng(4242 + k)
