@@ -420,6 +420,113 @@ struct U8<F_Q8_0> : U8Pair32 {
     }
 };
 
+// ------------------------------------------------------------------------------------- Q5_1
+// block_q5_1, 24 bytes: f16 d, f16 m, 32 fifth bits qh, 16 bytes of nibbles; value e = (nibble e % 16 (low for e < 16) + 16 * bit e
+// of qh) * d + m (core/kernels/GgufKernels.java:155-163).  A chunk is two blocks = 48 bytes = three 16-byte loads (matrices on
+// dword boundaries: the caller checks).
+template <>
+struct U8<F_Q5_1> : U8Pair32 {
+    static constexpr int FMT = F_Q5_1;
+    struct Raw { u32x4 a, b, c; };  // a: d0 | m0, qh0, qs0[0..7]; b: qs0[8..15], d1 | m1, qh1; c: qs1
+    struct Off { uint32_t o; };
+    struct Scale { float d0, d1, m0, m1; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) { return Off{row_off + (uint32_t)c * 48u}; }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.a = i8_ld128(rs, o.o, soff);
+        r.b = i8_ld128(rs, o.o + 16u, soff);
+        r.c = i8_ld128(rs, o.o + 32u, soff);
+    }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
+        s[0] = s4[0] + s4[1];
+        s[1] = s4[2] + s4[3];
+    }
+    // the fifth bits of values 4i .. 4i + 3 (bits 4i .. of qh) as bit 4 of the four bytes of a dword: the four copies of the
+    // nibble that the product makes (shifted by 0, 7, 14, 21) do not overlap, bit t of the nibble lands on bit 8t
+    __device__ static __forceinline__ uint32_t fifth(uint32_t qh, int i) { return ((((qh >> (4 * i)) & 15u) * 0x00204081u) & 0x01010101u) << 4; }
+    __device__ static __forceinline__ void extract(const Raw &r, int, uint32_t (&v)[16]) {
+        nibbles(u32x4{r.a.z, r.a.w, r.b.x, r.b.y}, r.c, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            v[i] |= fifth(r.a.y, i);
+            v[8 + i] |= fifth(r.b.w, i);
+        }
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int, Scale &sc) {
+        sc.d0 = h2f(r.a.x);
+        sc.m0 = h2f(r.a.x >> 16);
+        sc.d1 = h2f(r.b.z);
+        sc.m1 = h2f(r.b.z >> 16);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&s)[NSUM]) {
+        const float t = __builtin_fmaf(sc.d0, i8_combine_wide(d[0]), sc.d1 * i8_combine_wide(d[1]));
+        return __builtin_fmaf(t, sinv, __builtin_fmaf(sc.m0, s[0], sc.m1 * s[1]));
+    }
+};
+
+// ------------------------------------------------------------------------------------- Q2_K
+// block_q2_K, 84 bytes: 16 scale bytes (low nibble scale, high nibble min), 64 bytes of 2-bit quants, f16 d, f16 dmin; value
+// 128 n + 32 j + l is bits 2j.. of qs[32 n + l], scaled by byte 8 n + 2 j + l / 16 (core/kernels/GgufKernels.java:166-175).
+// Chunk c = 4 sb + 2 n + r takes the 16 bytes l in [16 r, 16 r + 16) of half n of super-block sb: four runs of 16 values
+// (j = 0..3), each with its own scale byte - the element order of the Q6_K chunk.
+template <>
+struct U8<F_Q2_K> {
+    static constexpr int FMT = F_Q2_K, NSUM = 4, CH = 4;
+    struct Raw { u32x4 q; u32x2 sc; uint32_t dd; };
+    struct Off { uint32_t q, sc, dd; };
+    struct Scale { float c[4], m[4]; };
+    __device__ static __forceinline__ Off offsets(int c, uint32_t row_off) {
+        Off o;
+        const uint32_t blk = row_off + (uint32_t)(c >> 2) * 84u, n = (uint32_t)(c >> 1) & 1u, r = (uint32_t)c & 1u;
+        o.q = blk + 16u + 32u * n + 16u * r;
+        o.sc = blk + 8u * n;
+        o.dd = blk + 80u;
+        return o;
+    }
+    __device__ static __forceinline__ int x_first(int c, int j) { return U8Q6Base::x_first(c, j); }
+    __device__ static __forceinline__ int x_pos(int c, int e) { return U8Q6Base::x_pos(c, e); }
+    __device__ static __forceinline__ void load(Raw &r, __amdgpu_buffer_rsrc_t rs, const Off &o, uint32_t soff) {
+        r.q = i8_ld128(rs, o.q, soff);
+        r.sc = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)o.sc, (int)soff, 0);
+        r.dd = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, (int)o.dd, (int)soff, 0);
+    }
+    __device__ static __forceinline__ void sums(const float (&s4)[4], float (&s)[NSUM]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s[i] = s4[i];
+    }
+    __device__ static __forceinline__ void extract(const Raw &r, int, uint32_t (&v)[16]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t w = r.q[i];
+            v[i] = w & 0x03030303u;
+            v[4 + i] = (w >> 2) & 0x03030303u;
+            v[8 + i] = (w >> 4) & 0x03030303u;
+            v[12 + i] = (w >> 6) & 0x03030303u;
+        }
+    }
+    __device__ static __forceinline__ void scales(const Raw &r, int c, Scale &sc) {
+        const int sh = (c & 1) * 8;
+        const uint32_t sa = r.sc.x >> sh, sb = r.sc.y >> sh;  // bytes 0 and 2: the scale bytes of runs 0, 1 | 2, 3
+        const float d = h2f(r.dd), dmin = h2f(r.dd >> 16);
+        sc.c[0] = d * (float)(sa & 15u);
+        sc.m[0] = dmin * (float)((sa >> 4) & 15u);
+        sc.c[1] = d * (float)((sa >> 16) & 15u);
+        sc.m[1] = dmin * (float)((sa >> 20) & 15u);
+        sc.c[2] = d * (float)(sb & 15u);
+        sc.m[2] = dmin * (float)((sb >> 4) & 15u);
+        sc.c[3] = d * (float)((sb >> 16) & 15u);
+        sc.m[3] = dmin * (float)((sb >> 20) & 15u);
+    }
+    __device__ static __forceinline__ float finish(const Scale &sc, const i32x4 (&d)[CH], float sinv, const float (&s)[NSUM]) {
+        float acc = sc.c[0] * (float)i8_combine(d[0]), m = sc.m[0] * s[0];
+#pragma unroll
+        for (int k = 1; k < 4; ++k) {
+            acc = __builtin_fmaf(sc.c[k], (float)i8_combine(d[k]), acc);
+            m = __builtin_fmaf(sc.m[k], s[k], m);
+        }
+        return __builtin_fmaf(acc, sinv, -m);
+    }
+};
+
 // The partial sums of a turn for B activation rows: the operands and scales of the weights are made once, every row runs its
 // chains of products (the chains of a row interleaved, so that a product never waits for the one before it).
 template <class U, int B>

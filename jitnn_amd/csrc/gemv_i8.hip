@@ -1,13 +1,14 @@
-// gemv_i8_kernel: batch-1 GEMV of Q4_K, Q5_K and Q6_K weights with INT8 matrix-core products.
+// gemv_i8_kernel: batch-1 (and two-row) GEMV on raw quantised blocks with INT8 matrix-core products.
 #include "gemv_i8.h"
 #include "tu.h"
 
 namespace jitnn {
 
-// K-quants; the 32-value formats with rows of whole pairs of blocks (their matrices on dword boundaries: the caller checks)
+// K-quants with rows of whole super-blocks; the 32-value formats with rows of whole pairs of blocks (matrices of the formats
+// fetched as dwords - the 32-value ones and Q2_K - on dword boundaries: the caller checks)
 bool gemv_i8_supported(int fmt, int k) {
-    if (fmt == F_Q4_0 || fmt == F_Q4_1 || fmt == F_Q8_0) return k % 64 == 0 && k >= 64 && k <= 1024 * I8_MAX_WAVES;
-    return (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K) && k % 256 == 0 && k >= 256 && k <= 1024 * I8_MAX_WAVES;
+    if (fmt == F_Q4_0 || fmt == F_Q4_1 || fmt == F_Q8_0 || fmt == F_Q5_1) return k % 64 == 0 && k >= 64 && k <= 1024 * I8_MAX_WAVES;
+    return (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K || fmt == F_Q2_K) && k % 256 == 0 && k >= 256 && k <= 1024 * I8_MAX_WAVES;
 }
 
 typedef void (*i8_fn)(const I8Args);
@@ -36,6 +37,14 @@ static i8_fn pick_batch(int mode, int pf) {
     return pf <= 1 ? gemv_i8_kernel<U, B, 1, false, false, false, 4> : gemv_i8_kernel<U, B, 2, false, false, false, 4>;
 }
 
+// Q5_1 and Q2_K: formats no fused launch of the decode step is built for - one activation row, with or without a bias
+template <class U, int MAXW>
+static i8_fn pick_plain(int mode, int pf) {
+    if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, true, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, true, false, false, MAXW>;
+    if (mode == I8_PLAIN) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, false, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, false, false, false, MAXW>;
+    return nullptr;
+}
+
 template <class U>
 static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
     if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_pf<U, I8_MAX_WAVES>(mode, pf);
@@ -61,6 +70,8 @@ void gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, c
     case F_Q4_0: fn = pick_rows<U8<F_Q4_0>>(rows, waves, mode, pf); break;
     case F_Q4_1: fn = pick_rows<U8<F_Q4_1>>(rows, waves, mode, pf); break;
     case F_Q8_0: fn = pick_rows<U8<F_Q8_0>>(rows, waves, mode, pf); break;
+    case F_Q5_1: fn = rows != 1 ? nullptr : waves <= 4 ? pick_plain<U8<F_Q5_1>, 4>(mode, pf) : pick_plain<U8<F_Q5_1>, I8_MAX_WAVES>(mode, pf); break;
+    case F_Q2_K: fn = rows != 1 ? nullptr : waves <= 4 ? pick_plain<U8<F_Q2_K>, 4>(mode, pf) : pick_plain<U8<F_Q2_K>, I8_MAX_WAVES>(mode, pf); break;
     case F_Q6_K: fn = q6_aligned(a) ? pick_rows<U8Q6<true>>(rows, waves, mode, pf) : pick_rows<U8Q6<false>>(rows, waves, mode, pf); break;
     default: break;
     }

@@ -264,7 +264,8 @@ bool i8_ok(const XregCall &c) {
         if (!c.w[i]) continue;
         n += c.w[i]->n;
         if (c.w[i]->nbytes >= (1ll << 32) || (c.w[1] && c.w[i]->n % 4 != 0)) return false;
-        if (block_values(c.w[i]->fmt) == 32 && ((uintptr_t)c.w[i]->dev & 3) != 0) return false;  // (pairs of 32-value blocks are fetched as dwords)
+        if ((block_values(c.w[i]->fmt) == 32 || c.w[i]->fmt == F_Q2_K) && ((uintptr_t)c.w[i]->dev & 3) != 0) return false;  // (fetched as dwords)
+        if (is_extra_format(c.w[i]->fmt) && (c.w[1] || c.w2 || c.norm_w)) return false;  // (Q5_1, Q2_K: no fused launches)
     }
     if (c.w2 && c.w2->nbytes >= (1ll << 32)) return false;
     if (c.w[1] && (!c.norm_w || c.w2)) return false;  // (several matrices in one launch: the kernel has that for the fused norm only)
@@ -519,7 +520,8 @@ int launch_gemv_mfma(const KernelRef &v, const jitnn_hip_weight *w, const float 
     return JITNN_HIP_OK;
 }
 
-// Formats without a tuned kernel (Q5_0, Q5_1, Q2_K, Q3_K): one wave per row on the bit-exact decoder.
+// Formats without a tuned kernel for this row count (Q5_0 and Q3_K left as they are, Q5_1 and Q2_K at more than one row or in
+// shapes the INT8 kernel does not take): one wave per row on the bit-exact decoder.
 int launch_gemv_plain(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
     int blocks = (w->n + 3) / 4;
     if (blocks > g.cus * 8) blocks = g.cus * 8;
@@ -532,7 +534,17 @@ int launch_gemv_plain(const jitnn_hip_weight *w, const float *x, int rows, const
 }
 
 int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
-    if (is_extra_format(w->fmt)) return launch_gemv_plain(w, x, rows, bias, y, stream);
+    if (is_extra_format(w->fmt)) {
+        if (rows == 1) {  // Q5_1 and Q2_K have units of the INT8 matrix-core kernel
+            XregCall c;
+            c.w[0] = w;
+            c.y[0] = y;
+            c.bias = bias;
+            c.x = x;
+            if (i8_ok(c)) return launch_i8(c, stream);
+        }
+        return launch_gemv_plain(w, x, rows, bias, y, stream);
+    }
     if (i8_batch_ok(w, rows)) return launch_i8_batch(w, x, rows, bias, y, stream);
     if (rows == 2 && w->k <= 4096) return launch_gemv_xreg_b2(w, x, bias, y, stream);
     // Q6_K pays the most per weight on the matrix-core path (6-bit quants from two arrays, 16-value scale groups): up to

@@ -411,6 +411,42 @@ def test_extra_format_dequant_and_linear_vs_oracle(jn, fmt):
         assert norm_err(y, ref) <= bar, (fmt, rows, norm_err(y, ref))
 
 
+@pytest.mark.parametrize("fmt", ["Q5_1", "Q2_K"])
+@pytest.mark.parametrize("n,k", [(4, 256), (37, 1024), (259, 4096), (64, 14336), (6, 16384), (3, 512), (16, 320)])
+def test_q5_1_q2_k_batch_1_matrix_core_units(jn, fmt, n, k):
+    """Q5_1 and Q2_K at one activation row: the INT8 matrix-core kernel's units for them (rows of one to sixteen waves, a row
+    count that is no multiple of four, with and without bias) and, for the shapes it does not take (fewer than four rows,
+    rows of 320 values for Q5_1 only), the plain kernel - ordinary, outlier-ridden, tiny and unit-vector activations
+    against the oracle, non-finite ones class by class."""
+    from oracle import oracle
+    if fmt == "Q2_K" and k % 256:
+        pytest.skip("Q2_K rows are whole super-blocks")
+    rng = np.random.default_rng(77 * GGML_ID[fmt] + n + k)
+    raw = random_valid_blocks(rng, fmt, n, k)
+    w = weight(jn, fmt, raw, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    xs = [rng.standard_normal(k).astype(np.float32)]
+    x = rng.standard_normal(k).astype(np.float32)
+    x[rng.integers(0, k, 5)] *= 1e4
+    xs.append(x)
+    xs.append((rng.standard_normal(k) * 1e-30).astype(np.float32))
+    x = np.zeros(k, dtype=np.float32)
+    x[k - 1] = 1.0
+    xs.append(x)
+    for i, x in enumerate(xs):
+        b = bias if i % 2 == 0 else None
+        ref = oracle.gguf_linear(GGML_ID[fmt], x[None, :], raw, b, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x[None, :]), w, jn.Tensor.of(b) if b is not None else None).numpy()
+        assert norm_err(y, ref) <= GEMV_BAR, (fmt, n, k, i, norm_err(y, ref))
+    x = rng.standard_normal(k).astype(np.float32)
+    x[k // 3] = np.inf
+    x[k // 2] = np.nan if n % 2 else -np.inf
+    ref = oracle.gguf_linear(GGML_ID[fmt], x[None, :], raw, None, n, k)
+    y = jn.Gguf.linear(jn.Tensor.of(x[None, :]), w, None).numpy()
+    assert np.array_equal(np.isnan(y), np.isnan(ref)) and np.array_equal(np.isposinf(y), np.isposinf(ref)) and \
+        np.array_equal(np.isneginf(y), np.isneginf(ref)), (fmt, n, k)
+
+
 @pytest.mark.parametrize("fmt", sorted(REWRITTEN))
 def test_rewritten_formats_keep_their_face_and_every_value(jn, fmt):
     """An uploaded Q5_0 / Q3_K weight reports the caller's format and byte count, dequantises to the oracle's bits for
