@@ -93,14 +93,16 @@ class Workload:
         if rc != 0:
             self.lib.check(rc, "jitnn_hip_linear_dev")
 
-    def time(self, steps: int, warmup: int, rotate: bool = True):
+    def time(self, steps: int, warmup: int, rotate: bool = True, events: bool = True):
         """(wall seconds, event seconds) for `steps` back-to-back launches after `warmup` untimed ones;
-        rotate=False keeps to one weight copy (cache-resident figure)."""
+        rotate=False keeps to one weight copy (cache-resident figure).  events=False: no event records inside the timed
+        region (a pair costs about 10 us of wall clock, half a microsecond per step of a 20-step region); the event
+        seconds are then None."""
         torch = self.torch
         with torch.cuda.stream(self.stream):
-            return self._time(steps, warmup, rotate)
+            return self._time(steps, warmup, rotate, events)
 
-    def _time(self, steps: int, warmup: int, rotate: bool):
+    def _time(self, steps: int, warmup: int, rotate: bool, events: bool = True):
         torch = self.torch
         stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         m = 1 if rotate else 0
@@ -117,15 +119,17 @@ class Workload:
         torch.cuda.synchronize()
         rc = 0
         t0 = time.perf_counter()
-        e0.record()
+        if events:
+            e0.record()
         for h in order:
             rc |= f(h, xp, b, None, yp, stream)
-        e1.record()
+        if events:
+            e1.record()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         if rc != 0:
             self.lib.check(rc, "jitnn_hip_linear_dev")
-        return t1 - t0, e0.elapsed_time(e1) * 1e-3
+        return t1 - t0, (e0.elapsed_time(e1) * 1e-3 if events else None)
 
     def time_streams(self, steps: int, nstreams: int = 4):
         """GB/s of `steps` launches spread round-robin over `nstreams` streams (all of default priority), weight copies
@@ -222,7 +226,8 @@ def measure(torch, lib, fmt, n, k, b, copies, steps, warmup, seed, parity=True):
     # enough untimed launches for the device to have left its idle clocks (a region that starts cold reads 5 % slower)
     roof_launches = max(steps, 2000 if n < 100000 else 300)
     _, roof_ev = wl.time(roof_launches, max(warmup, roof_launches // 4))
-    wall, ev = wl.time(steps, warmup)
+    wall, _ = wl.time(steps, warmup, events=False)  # `value`: exactly `steps` launches between two synchronisations, nothing else
+    _, ev = wl.time(steps, warmup)
     probe_us = wl.read_probe(400 if n < 100000 else 100)
     out = {"workload": f"{fmt} GEMV {n}x{k} batch {b}", "copies": copies, "steps": steps, "bytes_per_step": wl.bytes,
            "pure_read_us_per_launch": probe_us, "pure_read_GBps": wl.weights[0].numel() / probe_us / 1e3,
