@@ -411,6 +411,29 @@ def test_extra_format_dequant_and_linear_vs_oracle(jn, fmt):
         assert norm_err(y, ref) <= bar, (fmt, rows, norm_err(y, ref))
 
 
+def test_batch_1_and_2_random_shapes_all_formats(jn):
+    """Forty seeded shapes - any row count from 1 to 300, row lengths of 1 to 16 waves of the INT8 matrix-core kernel and lengths
+    it does not take (odd multiples of 32 for the 32-value formats), one or two activation rows, with and without bias, all
+    eight formats that kernel has units for - against the oracle."""
+    from oracle import oracle
+    rng = np.random.default_rng(20261)
+    fmts = ["Q4_K", "Q5_K", "Q6_K", "Q4_0", "Q4_1", "Q8_0", "Q5_1", "Q2_K"]
+    for case in range(40):
+        fmt = fmts[case % len(fmts)]
+        kq = 32 if fmt in ("Q4_0", "Q4_1", "Q8_0", "Q5_1") else 256
+        k = kq * int(rng.integers(1, 16384 // kq + 1)) if case % 5 else kq * int(rng.integers(1, 9))
+        n = int(rng.integers(1, 301))
+        rows = 1 + case % 2
+        raw = random_valid_blocks(rng, fmt, n, k)
+        w = weight(jn, fmt, raw, n, k)
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32) if case % 3 else None
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, bias, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias) if bias is not None else None).numpy()
+        assert y.shape == (rows, n)
+        assert norm_err(y, ref) <= GEMV_BAR, (case, fmt, n, k, rows, norm_err(y, ref))
+
+
 @pytest.mark.parametrize("fmt", ["Q5_1", "Q2_K"])
 @pytest.mark.parametrize("n,k", [(4, 256), (37, 1024), (259, 4096), (64, 14336), (6, 16384), (3, 512), (16, 320)])
 def test_q5_1_q2_k_batch_1_matrix_core_units(jn, fmt, n, k):
