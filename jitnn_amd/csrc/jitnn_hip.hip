@@ -391,6 +391,12 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
         const double ba = (double)ga * ca.w[0]->nbytes / ca.w[0]->n, bb = (double)gb * cb.w[0]->nbytes / cb.w[0]->n;
         int total, pf;
         i8_shape(ga + gb, (a.k + 1023) / 1024, false, total, pf);
+        // (q, k | v of an 8B layer - 1536 row groups, six per CU -, us per launch by workgroups per CU / turns in flight: 6.7 (1 / 2)
+        // 7.1 (1 / 1) 8.0 (2 / 1) 8.4 (2 / 2) 9.1 (3 / 1): the two formats' workgroups pace differently, one per CU keeps them apart)
+        if (ga + gb >= 4 * g.cus) {
+            total = g.cus;
+            pf = 2;
+        }
         if (total < 2) total = 2;
         int blocks_a = (int)(total * ba / (ba + bb) + 0.5);
         if (blocks_a < 1) blocks_a = 1;
