@@ -335,7 +335,9 @@ int launch_i8_batch(const jitnn_hip_weight *w, const float *x, int rows, const f
     a.k = w->k;
     a.rows = rows;
     const int groups = (w->n + 3) / 4;
-    const int per_cu = 2, pf = 1;
+    // (us per launch by workgroups per CU / turns in flight - Q4_K 14336 x 4096: 10.4 (1 / 2) 10.3 (2 / 2) 10.6 (2 / 1) 11.6 (1 / 1) 11.9 (3 / 1);
+    // Q4_0 11008 x 4096: 7.9 (1 / 2) 8.4 (2 / 1, 2 / 2) 8.6 (1 / 1); Q8_0 4096 x 4096: 6.4 (1 / 1) 6.7 (1 / 2) 6.9 (2 / 1) 7.7 (2 / 2))
+    const int per_cu = 1, pf = (groups + g.cus - 1) / g.cus >= 8 ? 2 : 1;
     const int blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
     gemv_i8_launch(w->fmt, bias ? I8_BIAS : I8_PLAIN, pf, (unsigned)blocks, stream, a);
     HIP_TRY(hipGetLastError());
