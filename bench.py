@@ -226,12 +226,18 @@ def measure(torch, lib, fmt, n, k, b, copies, steps, warmup, seed, parity=True):
     # enough untimed launches for the device to have left its idle clocks (a region that starts cold reads 5 % slower)
     roof_launches = max(steps, 2000 if n < 100000 else 300)
     _, roof_ev = wl.time(roof_launches, max(warmup, roof_launches // 4))
-    wall, _ = wl.time(steps, warmup, events=False)  # `value`: exactly `steps` launches between two synchronisations, nothing else
+    # The first synchronised region after the 2000-launch one pays the runtime's housekeeping for those 2000 commands (about
+    # 40 us, once: 10-11 us per step over 20 steps where every later region reads 8.3): one untimed region takes it.
+    wl.time(steps, warmup, events=False)
+    # `value`: exactly `steps` launches between two synchronisations, nothing else in the region.  Three such regions, the median
+    # reported: a region of 20 launches is 170 us of wall clock, and one host hiccup of 40 us in it reads as 25 %.
+    walls = sorted(wl.time(steps, warmup, events=False)[0] for _ in range(3))
+    wall = walls[1]
     _, ev = wl.time(steps, warmup)
     probe_us = wl.read_probe(400 if n < 100000 else 100)
     out = {"workload": f"{fmt} GEMV {n}x{k} batch {b}", "copies": copies, "steps": steps, "bytes_per_step": wl.bytes,
            "pure_read_us_per_launch": probe_us, "pure_read_GBps": wl.weights[0].numel() / probe_us / 1e3,
-           "us_per_step_wall": wall / steps * 1e6, "us_per_step_events": ev / steps * 1e6, "GBps": wl.bytes * steps / wall / 1e9,
+           "us_per_step_wall": wall / steps * 1e6, "us_per_step_wall_regions": [w / steps * 1e6 for w in walls], "us_per_step_events": ev / steps * 1e6, "GBps": wl.bytes * steps / wall / 1e9,
            "roofline_launches_timed": roof_launches, "us_per_launch_events": roof_ev / roof_launches * 1e6,
            "GBps_events": wl.bytes * roof_launches / roof_ev / 1e9, "pct_of_peak": wl.bytes * roof_launches / roof_ev / 1e9 / PEAK_HBM_GBPS * 100,
            "parity_norm_err": err}
