@@ -29,8 +29,8 @@ static i8_fn pick_pf(int mode, int pf) {
     else return pf <= 1 ? pick_mode<U, 1, MAXW>(mode) : pf == 2 ? pick_mode<U, 2, MAXW>(mode) : pick_mode<U, 3, MAXW>(mode);
 }
 
-// two activation rows, rows of at most 4096 values (the body takes any number; more than two are not instantiated: from three
-// rows on the 16-row tiles of gemv_mfma_kernel are faster)
+// two or four activation rows (three run as four with one absent), rows of at most 4096 values; the body takes any number, but
+// its products multiply one activation row each: from five rows on the 16-row tiles of gemv_mfma_kernel are faster
 template <class U, int B>
 static i8_fn pick_batch(int mode, int pf) {
     if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, B, 1, true, false, false, 4> : gemv_i8_kernel<U, B, 2, true, false, false, 4>;
@@ -48,11 +48,11 @@ static i8_fn pick_plain(int mode, int pf) {
 template <class U>
 static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
     if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_pf<U, I8_MAX_WAVES>(mode, pf);
-    if (waves > 4 || rows > 2 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
-    return pick_batch<U, 2>(mode, pf);
+    if (waves > 4 || rows > 4 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
+    return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }
 
-static int batch_of(int rows) { return rows == 1 ? 1 : 2; }
+static int batch_of(int rows) { return rows == 1 ? 1 : rows == 2 ? 2 : 4; }
 
 // Q6_K rows a multiple of four bytes long in matrices on dword boundaries take the variant with dword-aligned loads
 static bool q6_aligned(const I8Args &a) {

@@ -314,13 +314,15 @@ int launch_i8(const XregCall &c, hipStream_t stream) {
     return JITNN_HIP_OK;
 }
 
-// Two activation rows of a K-quant weight with rows of at most 4096 values: the same kernel with the activations of both rows
-// in registers (Q4_K 14336 x 4096: 10.2 us against 11.3 for the two-row FP32 register kernel).  The kernel is written for any
-// number of rows, but its 4x4x4 products cost about 16 cycles each whatever they multiply: with four rows (64 products a
-// turn) it measured 13.5 us, with eight (two groups of four) 20.4 - gemv_mfma_kernel's 16-row tiles stay ahead from three rows on.
+// Two to four activation rows, rows of at most 4096 values: the same kernel with the activations of all rows in registers - the
+// operands and scales of the weights are made once, every row runs its own chains of products.  us per launch against the FP32
+// two-row kernel / gemv_mfma_kernel - Q4_K 14336 x 4096: 10.3 (11.3) at two rows, 12.8 (13.9) at three, 13.1 (13.8) at four; Q4_0
+// 11008 x 4096 at four: 10.6 (11.8); Q8_0 4096 x 4096: 7.1 (10.1); Q6_K 14336 x 4096: 16.2 (23.0).  Its 4x4x4 products multiply one
+// activation row each, so their number grows with the rows: eight rows (two groups of four along blockIdx.y) measured 20.4 us
+// where gemv_mfma_kernel's 16-row tiles take 14.5 - from five rows on those stay ahead.
 bool i8_batch_ok(const jitnn_hip_weight *w, int rows) {
-    return g.gemv_i8 && rows == 2 && gemv_i8_supported(w->fmt, w->k) && w->k <= 4096 && w->n >= 4 && w->nbytes < (1ll << 32) &&
-           (block_values(w->fmt) != 32 || ((uintptr_t)w->dev & 3) == 0);
+    return g.gemv_i8 && rows >= 2 && rows <= 4 && gemv_i8_supported(w->fmt, w->k) && !is_extra_format(w->fmt) && w->k <= 4096 && w->n >= 4 &&
+           w->nbytes < (1ll << 32) && (block_values(w->fmt) != 32 || ((uintptr_t)w->dev & 3) == 0);
 }
 
 int launch_i8_batch(const jitnn_hip_weight *w, const float *x, int rows, const float *bias, float *y, hipStream_t stream) {
@@ -335,8 +337,9 @@ int launch_i8_batch(const jitnn_hip_weight *w, const float *x, int rows, const f
     a.k = w->k;
     a.rows = rows;
     const int groups = (w->n + 3) / 4;
-    // (us per launch by workgroups per CU / turns in flight - Q4_K 14336 x 4096: 10.4 (1 / 2) 10.3 (2 / 2) 10.6 (2 / 1) 11.6 (1 / 1) 11.9 (3 / 1);
-    // Q4_0 11008 x 4096: 7.9 (1 / 2) 8.4 (2 / 1, 2 / 2) 8.6 (1 / 1); Q8_0 4096 x 4096: 6.4 (1 / 1) 6.7 (1 / 2) 6.9 (2 / 1) 7.7 (2 / 2))
+    // (us per launch by workgroups per CU / turns in flight, two rows - Q4_K 14336 x 4096: 10.4 (1 / 2) 10.3 (2 / 2) 10.6 (2 / 1) 11.6 (1 / 1)
+    // 11.9 (3 / 1); Q4_0 11008 x 4096: 7.9 (1 / 2) 8.4 (2 / 1, 2 / 2) 8.6 (1 / 1); Q8_0 4096 x 4096: 6.4 (1 / 1) 6.7 (1 / 2) 6.9 (2 / 1) 7.7 (2 / 2);
+    // four rows - Q4_K: 13.1 (1 / 2, 2 / 1) 14.0 (1 / 1); Q4_0: 10.6 (1 / 2) 10.9 (1 / 1) 11.0 (2 / 1); Q8_0: 7.1 (1 / 1) 7.7 (1 / 2) 9.1 (2 / 1))
     const int per_cu = 1, pf = (groups + g.cus - 1) / g.cus >= 8 ? 2 : 1;
     const int blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
     gemv_i8_launch(w->fmt, bias ? I8_BIAS : I8_PLAIN, pf, (unsigned)blocks, stream, a);
