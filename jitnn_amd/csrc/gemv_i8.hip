@@ -61,7 +61,7 @@ static bool q6_aligned(const I8Args &a) {
     return ok;
 }
 
-void gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a) {
+bool gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a) {
     const int waves = (a.k + 1023) / 1024, rows = a.rows < 1 ? 1 : a.rows;
     i8_fn fn = nullptr;
     switch (fmt) {
@@ -75,9 +75,10 @@ void gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, c
     case F_Q6_K: fn = q6_aligned(a) ? pick_rows<U8Q6<true>>(rows, waves, mode, pf) : pick_rows<U8Q6<false>>(rows, waves, mode, pf); break;
     default: break;
     }
-    if (!fn) return;
+    if (!fn) return false;
     const int bt = batch_of(rows);
     hipLaunchKernelGGL(fn, dim3(blocks, (rows + bt - 1) / bt), dim3(64 * waves), gemv_i8_lds_bytes(waves, bt), s, a);
+    return true;
 }
 
 typedef void (*i8_pair_fn)(const I8Args, const I8Args, int);
@@ -92,12 +93,13 @@ static i8_pair_fn pick_pair(int fa, int fb, bool al) {
 
 bool gemv_i8_pair_supported(int fmt_a, int fmt_b) { return pick_pair<1>(fmt_a, fmt_b, false) != nullptr; }
 
-void gemv_i8_pair_launch(int fmt_a, int fmt_b, int pf, unsigned blocks_a, unsigned blocks_b, hipStream_t s, const I8Args &a, const I8Args &b) {
+bool gemv_i8_pair_launch(int fmt_a, int fmt_b, int pf, unsigned blocks_a, unsigned blocks_b, hipStream_t s, const I8Args &a, const I8Args &b) {
     const int waves = (a.k + 1023) / 1024;
     const bool al = fmt_b == F_Q6_K && q6_aligned(b);
     const i8_pair_fn fn = pf <= 1 ? pick_pair<1>(fmt_a, fmt_b, al) : pick_pair<2>(fmt_a, fmt_b, al);
-    if (!fn || waves > 4) return;
+    if (!fn || waves > 4) return false;
     hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(64 * waves), gemv_i8_lds_bytes(waves), s, a, b, (int)blocks_a);
+    return true;
 }
 
 }  // namespace jitnn

@@ -309,7 +309,8 @@ int launch_i8(const XregCall &c, hipStream_t stream) {
     int blocks, pf;
     i8_shape((n + 3) / 4, (a.k + 1023) / 1024, c.w2 != nullptr, blocks, pf);
     if (c.w[0]->fmt == F_Q5_K && pf > 2) pf = 2;  // (five loads per turn: a fourth buffer does not fit 128 registers)
-    gemv_i8_launch(c.w[0]->fmt, mode, pf, (unsigned)blocks, stream, a);
+    if (!gemv_i8_launch(c.w[0]->fmt, mode, pf, (unsigned)blocks, stream, a))
+        return fail(JITNN_HIP_EDEVICE, "no INT8 GEMV kernel for format %d in mode %d, rows of %d values", c.w[0]->fmt, mode, a.k);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
@@ -342,7 +343,8 @@ int launch_i8_batch(const jitnn_hip_weight *w, const float *x, int rows, const f
     // four rows - Q4_K: 13.1 (1 / 2, 2 / 1) 14.0 (1 / 1); Q4_0: 10.6 (1 / 2) 10.9 (1 / 1) 11.0 (2 / 1); Q8_0: 7.1 (1 / 1) 7.7 (1 / 2) 9.1 (2 / 1))
     const int per_cu = 1, pf = (groups + g.cus - 1) / g.cus >= 8 ? 2 : 1;
     const int blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
-    gemv_i8_launch(w->fmt, bias ? I8_BIAS : I8_PLAIN, pf, (unsigned)blocks, stream, a);
+    if (!gemv_i8_launch(w->fmt, bias ? I8_BIAS : I8_PLAIN, pf, (unsigned)blocks, stream, a))
+        return fail(JITNN_HIP_EDEVICE, "no INT8 GEMV kernel for format %d at %d rows of %d values", w->fmt, rows, a.k);
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
@@ -409,7 +411,8 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
         if (blocks_a > ga) blocks_a = ga;
         int blocks_b = total - blocks_a;
         if (blocks_b > gb) blocks_b = gb;
-        gemv_i8_pair_launch(ca.w[0]->fmt, cb.w[0]->fmt, pf > 2 ? 2 : pf, (unsigned)blocks_a, (unsigned)blocks_b, stream, a, b);
+        if (!gemv_i8_pair_launch(ca.w[0]->fmt, cb.w[0]->fmt, pf > 2 ? 2 : pf, (unsigned)blocks_a, (unsigned)blocks_b, stream, a, b))
+            return fail(JITNN_HIP_EDEVICE, "no INT8 GEMV kernel for the formats %d and %d in one launch", ca.w[0]->fmt, cb.w[0]->fmt);
         HIP_TRY(hipGetLastError());
         return JITNN_HIP_OK;
     }

@@ -93,7 +93,7 @@ void gemv_rows_prepare_launch(hipStream_t s, const float *x, const float *swiglu
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,
                            int n, int k, int rows);
 
-// ---- gemv_i8.hip: gemv_i8_kernel<fmt>: batch-1 GEMV of the K-quants with INT8 matrix-core products
+// ---- gemv_i8.hip: gemv_i8_kernel<unit>: GEMV of one to four activation rows with INT8 matrix-core products on the raw quants
 // Arguments of gemv_i8_kernel: up to three matrices of one format and row length share a launch and an activation vector (row segments
 // numbered one after the other).  DUAL: w2 is a second matrix of the shape of w[0]; y[0] = silu(w[0] x) * (w2 x).
 struct I8Args {
@@ -112,9 +112,9 @@ struct I8Args {
 constexpr int I8_PLAIN = 0, I8_BIAS = 1, I8_NORM = 2, I8_DUAL = 3;  // DUAL: norm + the SwiGLU pair
 bool gemv_i8_supported(int fmt, int k);
 // blockDim = 64 * ceil(k / 1024); pf = turns of weight bytes in flight per wave beyond the one being multiplied (1..3; 1..2 for
-// two activation rows - a.rows == 2, rows of at most 4096 values, modes I8_PLAIN and I8_BIAS only)
-void gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a);
+// two to four activation rows - a.rows in 2..4, rows of at most 4096 values, modes I8_PLAIN and I8_BIAS only)
+bool gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a);  // false: no kernel for this call, nothing launched
 bool gemv_i8_pair_supported(int fmt_a, int fmt_b);
-void gemv_i8_pair_launch(int fmt_a, int fmt_b, int pf, unsigned blocks_a, unsigned blocks_b, hipStream_t s, const I8Args &a, const I8Args &b);
+bool gemv_i8_pair_launch(int fmt_a, int fmt_b, int pf, unsigned blocks_a, unsigned blocks_b, hipStream_t s, const I8Args &a, const I8Args &b);
 
 }  // namespace jitnn
