@@ -37,7 +37,7 @@ static i8_fn pick_batch(int mode, int pf) {
     return pf <= 1 ? gemv_i8_kernel<U, B, 1, false, false, false, 4> : gemv_i8_kernel<U, B, 2, false, false, false, 4>;
 }
 
-// Q5_1 and Q2_K: formats no fused launch of the decode step is built for - one activation row, with or without a bias
+// Q5_1 and Q2_K: formats no fused launch of the decode step is built for - with or without a bias, nothing else
 template <class U, int MAXW>
 static i8_fn pick_plain(int mode, int pf) {
     if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, true, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, true, false, false, MAXW>;
@@ -48,6 +48,13 @@ static i8_fn pick_plain(int mode, int pf) {
 template <class U>
 static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
     if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_pf<U, I8_MAX_WAVES>(mode, pf);
+    if (waves > 4 || rows > 4 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
+    return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
+}
+
+template <class U>
+static i8_fn pick_rows_plain(int rows, int waves, int mode, int pf) {
+    if (rows == 1) return waves <= 4 ? pick_plain<U, 4>(mode, pf) : pick_plain<U, I8_MAX_WAVES>(mode, pf);
     if (waves > 4 || rows > 4 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
     return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }
@@ -70,8 +77,8 @@ bool gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, c
     case F_Q4_0: fn = pick_rows<U8<F_Q4_0>>(rows, waves, mode, pf); break;
     case F_Q4_1: fn = pick_rows<U8<F_Q4_1>>(rows, waves, mode, pf); break;
     case F_Q8_0: fn = pick_rows<U8<F_Q8_0>>(rows, waves, mode, pf); break;
-    case F_Q5_1: fn = rows != 1 ? nullptr : waves <= 4 ? pick_plain<U8<F_Q5_1>, 4>(mode, pf) : pick_plain<U8<F_Q5_1>, I8_MAX_WAVES>(mode, pf); break;
-    case F_Q2_K: fn = rows != 1 ? nullptr : waves <= 4 ? pick_plain<U8<F_Q2_K>, 4>(mode, pf) : pick_plain<U8<F_Q2_K>, I8_MAX_WAVES>(mode, pf); break;
+    case F_Q5_1: fn = pick_rows_plain<U8<F_Q5_1>>(rows, waves, mode, pf); break;
+    case F_Q2_K: fn = pick_rows_plain<U8<F_Q2_K>>(rows, waves, mode, pf); break;
     case F_Q6_K: fn = q6_aligned(a) ? pick_rows<U8Q6<true>>(rows, waves, mode, pf) : pick_rows<U8Q6<false>>(rows, waves, mode, pf); break;
     default: break;
     }

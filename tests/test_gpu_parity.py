@@ -436,8 +436,8 @@ def test_batch_1_and_2_random_shapes_all_formats(jn):
 
 @pytest.mark.parametrize("fmt", ["Q5_1", "Q2_K"])
 @pytest.mark.parametrize("n,k", [(4, 256), (37, 1024), (259, 4096), (64, 14336), (6, 16384), (3, 512), (16, 320)])
-def test_q5_1_q2_k_batch_1_matrix_core_units(jn, fmt, n, k):
-    """Q5_1 and Q2_K at one activation row: the INT8 matrix-core kernel's units for them (rows of one to sixteen waves, a row
+def test_q5_1_q2_k_matrix_core_units(jn, fmt, n, k):
+    """Q5_1 and Q2_K at one to four activation rows: the INT8 matrix-core kernel's units for them (rows of one to sixteen waves, a row
     count that is no multiple of four, with and without bias) and, for the shapes it does not take (fewer than four rows,
     rows of 320 values for Q5_1 only), the plain kernel - ordinary, outlier-ridden, tiny and unit-vector activations
     against the oracle, non-finite ones class by class."""
@@ -468,6 +468,14 @@ def test_q5_1_q2_k_batch_1_matrix_core_units(jn, fmt, n, k):
     y = jn.Gguf.linear(jn.Tensor.of(x[None, :]), w, None).numpy()
     assert np.array_equal(np.isnan(y), np.isnan(ref)) and np.array_equal(np.isposinf(y), np.isposinf(ref)) and \
         np.array_equal(np.isneginf(y), np.isneginf(ref)), (fmt, n, k)
+    for rows in (2, 3, 4):  # the same kernel with the activations of several rows in registers (rows of at most 4096 values)
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        x[rows - 1] *= 1e-3
+        b = bias if rows % 2 else None
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, b, n, k)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(b) if b is not None else None).numpy()
+        for r in range(rows):
+            assert norm_err(y[r], ref[r]) <= GEMV_BAR, (fmt, n, k, rows, r, norm_err(y[r], ref[r]))
 
 
 @pytest.mark.parametrize("fmt", sorted(REWRITTEN))
