@@ -48,7 +48,7 @@ static i8_fn pick_plain(int mode, int pf) {
 template <class U>
 static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
     if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_pf<U, I8_MAX_WAVES>(mode, pf);
-    if (waves > 4 || rows > 4 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
+    if (waves > 4 || rows > 8 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;  // (five to eight rows: two groups of four)
     return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }
 
