@@ -553,7 +553,7 @@ __device__ __forceinline__ void i8_dot(const typename U::Raw &r, int c, const ui
 // -------------------------------------------------------------------------------------------------- the kernel body
 // rb: the first activation row of this workgroup (launches of more than B rows put the row groups of B along blockIdx.y:
 // their workgroups stream the same weight bytes at the same time, so one of them finds them in the cache)
-template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL>
+template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
 __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, const int nblocks, const int rb = 0) {
     constexpr int FMT = U::FMT, NB = PF + 1, FL = i8_flush(B);
     static_assert(FL % NB == 0 && FL % 2 == 0, "whole rings (and gate/up pairs) per flush window");
@@ -693,12 +693,19 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
 
     auto group_of = [&](int t) { return bid + (DUAL ? t >> 1 : t) * nblocks; };
     // one output of a window: the partial sums of all waves in wave order
+    // (all reads issued before the first addition - a loop over the workgroup's actual number of waves waits for every wave's four
+    // values in turn, 0.6 us at the end of a 14-wave workgroup; waves the workgroup does not have add zeros)
     auto joined = [&](int half, int tt, int r, int jj) {
-        float sum = 0.f;
-        for (int w = 0; w < waves; ++w) {
-            const float *p = reinterpret_cast<const float *>(i8_smem + (size_t)w * WAVE_LDS) + ((half * FL + tt) * B + r) * 16 + jj;
-            sum += (p[0] + p[4]) + (p[8] + p[12]);
+        float part[MAXW];
+#pragma unroll
+        for (int w = 0; w < MAXW; ++w) {
+            const float *p = reinterpret_cast<const float *>(i8_smem + (size_t)min(w, waves - 1) * WAVE_LDS) + ((half * FL + tt) * B + r) * 16 + jj;
+            const float v = (p[0] + p[4]) + (p[8] + p[12]);
+            part[w] = w < waves ? v : 0.f;
         }
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < MAXW; ++w) sum += part[w];
         return sum;
     };
 
@@ -797,15 +804,15 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
 
 template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
 __global__ void __launch_bounds__(64 * MAXW, (B > 1 ? 2 : 4)) gemv_i8_kernel(const I8Args a) {
-    gemv_i8_body<U, B, PF, BIAS, NORM, DUAL>(a, blockIdx.x, gridDim.x, B * (int)blockIdx.y);
+    gemv_i8_body<U, B, PF, BIAS, NORM, DUAL, MAXW>(a, blockIdx.x, gridDim.x, B * (int)blockIdx.y);
 }
 
 // Two sets of matrices in two formats over the same (normalised) activations in one launch - the q / k and the v
 // projections of a Q4_K_M layer: workgroups below `split` run the first set, the others the second.
 template <class UA, class UB, int PF, int MAXW>
 __global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_pair_kernel(const I8Args a, const I8Args b, const int split) {
-    if ((int)blockIdx.x < split) gemv_i8_body<UA, 1, PF, false, true, false>(a, blockIdx.x, split);
-    else gemv_i8_body<UB, 1, PF, false, true, false>(b, blockIdx.x - split, gridDim.x - split);
+    if ((int)blockIdx.x < split) gemv_i8_body<UA, 1, PF, false, true, false, MAXW>(a, blockIdx.x, split);
+    else gemv_i8_body<UB, 1, PF, false, true, false, MAXW>(b, blockIdx.x - split, gridDim.x - split);
 }
 
 }  // namespace jitnn

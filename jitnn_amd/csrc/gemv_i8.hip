@@ -40,21 +40,25 @@ static i8_fn pick_batch(int mode, int pf) {
 // Q5_1 and Q2_K: formats no fused launch of the decode step is built for - with or without a bias, nothing else
 template <class U, int MAXW>
 static i8_fn pick_plain(int mode, int pf) {
-    if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, true, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, true, false, false, MAXW>;
-    if (mode == I8_PLAIN) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, false, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, false, false, false, MAXW>;
-    return nullptr;
+    if constexpr (MAXW > 4) {  // (long rows: one turn in flight)
+        return mode == I8_BIAS ? gemv_i8_kernel<U, 1, 1, true, false, false, MAXW> : mode == I8_PLAIN ? gemv_i8_kernel<U, 1, 1, false, false, false, MAXW> : nullptr;
+    } else {
+        if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, true, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, true, false, false, MAXW>;
+        if (mode == I8_PLAIN) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, false, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, false, false, false, MAXW>;
+        return nullptr;
+    }
 }
 
 template <class U>
 static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
-    if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_pf<U, I8_MAX_WAVES>(mode, pf);
+    if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_mode<U, 1, I8_MAX_WAVES>(mode);  // (long rows: one turn in flight)
     if (waves > 4 || rows > 8 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;  // (five to eight rows: two groups of four)
     return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }
 
 template <class U>
 static i8_fn pick_rows_plain(int rows, int waves, int mode, int pf) {
-    if (rows == 1) return waves <= 4 ? pick_plain<U, 4>(mode, pf) : pick_plain<U, I8_MAX_WAVES>(mode, pf);
+    if (rows == 1) return waves <= 4 ? pick_plain<U, 4>(mode, pf) : pick_plain<U, I8_MAX_WAVES>(mode, 1);
     if (waves > 4 || rows > 4 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
     return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }
