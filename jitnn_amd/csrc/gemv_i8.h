@@ -33,8 +33,9 @@ namespace jitnn {
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int I8_MAX_WAVES = 16;
-// turns between two joins of the waves' partial sums (a multiple of every ring length): 24 for one activation row, 12 for more
-__host__ __device__ constexpr int i8_flush(int rows) { return rows == 1 ? 24 : 12; }
+// turns between two joins of the waves' partial sums (a multiple of every ring length): 36 for one activation row - the 28 turns
+// of a gate / up launch of an 8B layer fit one window: 14.1 against 14.5 us with 24 -, 12 for more
+__host__ __device__ constexpr int i8_flush(int rows) { return rows == 1 ? 36 : 12; }
 // LDS of a wave: 16 chunks x 3 planes x 64 bytes while the activations are staged; afterwards the wave's partial sums,
 // 2 windows x flush turns x rows x 16 floats
 __host__ __device__ constexpr size_t gemv_i8_lds_per_wave(int rows) {
