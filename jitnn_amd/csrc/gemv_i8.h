@@ -551,6 +551,61 @@ __device__ __forceinline__ void i8_dot(const typename U::Raw &r, int c, const ui
     }
 }
 
+// The 16 activations xv of lane (chunk b, quarter j) of a wave's 1024-value slice -> fixed point, v = rint(x * s), |v| < 2^22, s a
+// power of two from the chunk's largest magnitude, cut into three signed byte digits; the planes cross the wave's own LDS
+// (`planes`, 3 KB) from staging order into operand order: xa = the sixteen operand dwords of this lane's plane, sinv = 1 / s,
+// sums = the sums of x the unit's offset terms need.  Returns whether the slice holds an Inf or a NaN (xa is garbage then).
+template <class U>
+__device__ __forceinline__ bool i8_stage(const float4 (&xv)[4], u32x4 *planes, int b, int j, uint32_t (&xa)[16], float &sinv, float (&sums)[U::NSUM]) {
+    uint32_t am = 0u;
+    float sm = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        am = max(max(am, max(__float_as_uint(xv[i].x) & 0x7fffffffu, __float_as_uint(xv[i].y) & 0x7fffffffu)),
+                 max(__float_as_uint(xv[i].z) & 0x7fffffffu, __float_as_uint(xv[i].w) & 0x7fffffffu));
+        sm += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+    }
+    am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+    am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+    const bool nonfinite = __builtin_amdgcn_ballot_w64(am >= 0x7f800000u) != 0;
+    const uint32_t eb = min(max(am >> 23, 22u), 254u);
+    const float s = __uint_as_float((275u - eb) << 23);
+    sinv = __uint_as_float((eb - 21u) << 23);
+    float s4[4];
+    s4[0] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x00, 0xF, 0xF, true));  // quad_perm [0,0,0,0]
+    s4[1] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x55, 0xF, 0xF, true));
+    s4[2] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xAA, 0xF, 0xF, true));
+    s4[3] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xFF, 0xF, 0xF, true));
+    U::sums(s4, sums);
+    uint32_t pl[3][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float f[4] = {xv[i].x, xv[i].y, xv[i].z, xv[i].w};
+        uint32_t u[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u[e] = __float_as_uint(__builtin_fmaf(f[e], s, 12582912.f)) + (0x00808080u - 0x4B400000u);
+        // bytes 0..2 of u are the digits + 128; gather byte p of the four values into one dword, then flip the top bits
+        const uint32_t t01 = __builtin_amdgcn_perm(u[1], u[0], 0x05010400u), t23 = __builtin_amdgcn_perm(u[3], u[2], 0x05010400u);
+        pl[0][i] = __builtin_amdgcn_perm(t23, t01, 0x05040100u) ^ 0x80808080u;
+        pl[1][i] = __builtin_amdgcn_perm(t23, t01, 0x07060302u) ^ 0x80808080u;
+        const uint32_t w01 = __builtin_amdgcn_perm(u[1], u[0], 0x00000602u), w23 = __builtin_amdgcn_perm(u[3], u[2], 0x00000602u);
+        pl[2][i] = __builtin_amdgcn_perm(w23, w01, 0x05040100u) ^ 0x80808080u;
+    }
+    // (a slice that is not finite leaves garbage here; the slow path does not read it)
+#pragma unroll
+    for (int p = 0; p < 3; ++p) planes[(b * 3 + p) * 4 + j] = u32x4{pl[p][0], pl[p][1], pl[p][2], pl[p][3]};
+    // (the LDS accesses of a wave complete in order: its reads below see its writes above without a barrier)
+    __builtin_amdgcn_wave_barrier();
+    const int p = min(j, 2);  // operand row 3 of the product is not used: lane 4b + 3 feeds plane 2 again
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+        const u32x4 v = planes[(b * 3 + p) * 4 + qd];
+        xa[qd * 4 + 0] = v.x; xa[qd * 4 + 1] = v.y; xa[qd * 4 + 2] = v.z; xa[qd * 4 + 3] = v.w;
+    }
+    __builtin_amdgcn_wave_barrier();
+    return nonfinite;
+}
+
 // -------------------------------------------------------------------------------------------------- the kernel body
 // rb: the first activation row of this workgroup (launches of more than B rows put the row groups of B along blockIdx.y:
 // their workgroups stream the same weight bytes at the same time, so one of them finds them in the cache)
@@ -638,59 +693,12 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
             xv[0][i] = make_float4(xv[0][i].x * nv[i].x, xv[0][i].y * nv[i].y, xv[0][i].z * nv[i].z, xv[0][i].w * nv[i].w);
     }
 
-    // ---- fixed point, row by row: v = rint(x * s), |v| < 2^22, s a power of two from the chunk's largest magnitude
+    // ---- fixed point, row by row
     uint32_t xa[B][16];
     float sinv[B], sums[B][U::NSUM];
     bool slow = false;
 #pragma unroll
-    for (int r = 0; r < B; ++r) {
-        uint32_t am = 0u;
-        float sm = 0.f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            am = max(max(am, max(__float_as_uint(xv[r][i].x) & 0x7fffffffu, __float_as_uint(xv[r][i].y) & 0x7fffffffu)),
-                     max(__float_as_uint(xv[r][i].z) & 0x7fffffffu, __float_as_uint(xv[r][i].w) & 0x7fffffffu));
-            sm += (xv[r][i].x + xv[r][i].y) + (xv[r][i].z + xv[r][i].w);
-        }
-        am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
-        am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
-        slow = slow || __builtin_amdgcn_ballot_w64(am >= 0x7f800000u) != 0;                    // an Inf or NaN in this wave's slice
-        const uint32_t eb = min(max(am >> 23, 22u), 254u);
-        const float s = __uint_as_float((275u - eb) << 23);
-        sinv[r] = __uint_as_float((eb - 21u) << 23);
-        float s4[4];
-        s4[0] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x00, 0xF, 0xF, true));  // quad_perm [0,0,0,0]
-        s4[1] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0x55, 0xF, 0xF, true));
-        s4[2] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xAA, 0xF, 0xF, true));
-        s4[3] = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sm), 0xFF, 0xF, 0xF, true));
-        U::sums(s4, sums[r]);
-        uint32_t pl[3][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float f[4] = {xv[r][i].x, xv[r][i].y, xv[r][i].z, xv[r][i].w};
-            uint32_t u[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) u[e] = __float_as_uint(__builtin_fmaf(f[e], s, 12582912.f)) + (0x00808080u - 0x4B400000u);
-            // bytes 0..2 of u are the digits + 128; gather byte p of the four values into one dword, then flip the top bits
-            const uint32_t t01 = __builtin_amdgcn_perm(u[1], u[0], 0x05010400u), t23 = __builtin_amdgcn_perm(u[3], u[2], 0x05010400u);
-            pl[0][i] = __builtin_amdgcn_perm(t23, t01, 0x05040100u) ^ 0x80808080u;
-            pl[1][i] = __builtin_amdgcn_perm(t23, t01, 0x07060302u) ^ 0x80808080u;
-            const uint32_t w01 = __builtin_amdgcn_perm(u[1], u[0], 0x00000602u), w23 = __builtin_amdgcn_perm(u[3], u[2], 0x00000602u);
-            pl[2][i] = __builtin_amdgcn_perm(w23, w01, 0x05040100u) ^ 0x80808080u;
-        }
-        // (a row that is not finite leaves garbage here; the slow path below does not read it)
-#pragma unroll
-        for (int p = 0; p < 3; ++p) planes[(b * 3 + p) * 4 + j] = u32x4{pl[p][0], pl[p][1], pl[p][2], pl[p][3]};
-        // (the LDS accesses of a wave complete in order: its reads below see its writes above without a barrier)
-        __builtin_amdgcn_wave_barrier();
-        const int p = min(j, 2);  // operand row 3 of the product is not used: lane 4b + 3 feeds plane 2 again
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-            const u32x4 v = planes[(b * 3 + p) * 4 + qd];
-            xa[r][qd * 4 + 0] = v.x; xa[r][qd * 4 + 1] = v.y; xa[r][qd * 4 + 2] = v.z; xa[r][qd * 4 + 3] = v.w;
-        }
-        __builtin_amdgcn_wave_barrier();
-    }
+    for (int r = 0; r < B; ++r) slow = i8_stage<U>(xv[r], planes, b, j, xa[r], sinv[r], sums[r]) || slow;  // an Inf or NaN in this wave's slice
 
     auto group_of = [&](int t) { return bid + (DUAL ? t >> 1 : t) * nblocks; };
     // one output of a window: the partial sums of all waves in wave order
