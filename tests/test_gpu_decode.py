@@ -47,12 +47,17 @@ def jn():
     return jitnn_amd
 
 
-@pytest.mark.parametrize("mix_name", ["q4_k_m", "q8_0", "q4_0_q5_k"])
+@pytest.mark.parametrize("mix_name", ["q4_k_m", "q8_0", "q4_0_q5_k", "q4_k_q5_k", "q5_k_m", "q6_k", "q4_1"])
 def test_decode_small_model(jn, mix_name):
-    """Two layers, grouped heads 8/2 of size 64, three tokens decoded in a row on a pre-filled cache."""
+    """Two layers, grouped heads 8/2 of size 64, three tokens decoded in a row on a pre-filled cache.  The mixes cover the
+    two-format q, k | v launches the library has (Q4_K | Q6_K, Q4_K | Q5_K, Q5_K | Q6_K), a single format for all three and a
+    pair it launches separately (Q4_0 | Q5_K); every format of the path as the gate / up pair of the fused SwiGLU launch."""
     cfg = dict(layers=2, d_model=512, heads=8, kv_heads=2, head_dim=64, ffn=1024, vocab=1000, max_ctx=48, rms_eps=1e-5, rope_theta=5e5)
     mix = {"q4_k_m": MIX, "q8_0": {s: "Q8_0" for s in SLOTS},
-           "q4_0_q5_k": {**{s: "Q4_0" for s in SLOTS}, "attn_v": "Q5_K", "ffn_down": "Q5_K", "attn_o": "Q4_1"}}[mix_name]
+           "q4_0_q5_k": {**{s: "Q4_0" for s in SLOTS}, "attn_v": "Q5_K", "ffn_down": "Q5_K", "attn_o": "Q4_1"},
+           "q4_k_q5_k": {**{s: "Q4_K" for s in SLOTS}, "attn_v": "Q5_K", "ffn_down": "Q5_K"},
+           "q5_k_m": {**{s: "Q5_K" for s in SLOTS}, "attn_v": "Q6_K", "ffn_down": "Q6_K"},
+           "q6_k": {s: "Q6_K" for s in SLOTS}, "q4_1": {s: "Q4_1" for s in SLOTS}}[mix_name]
     dec, layers, out_norm, out_w = build(jn, cfg, 5, mix, "Q8_0" if mix_name == "q8_0" else "Q6_K")
     rng = np.random.default_rng(1)
     ctx0 = 37
