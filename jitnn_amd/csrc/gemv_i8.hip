@@ -51,7 +51,7 @@ static i8_fn pick_plain(int mode, int pf) {
 
 template <class U>
 static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
-    if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_mode<U, 1, I8_MAX_WAVES>(mode);  // (long rows: one turn in flight)
+    if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_plain<U, I8_MAX_WAVES>(mode, 1);  // (long rows: plain or biased, one turn in flight - the fused launches of the decode step have rows of at most 4096 values)
     if (waves > 4 || rows > 8 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;  // (five to eight rows: two groups of four)
     return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }

@@ -47,6 +47,30 @@ def jn():
     return jitnn_amd
 
 
+@pytest.mark.parametrize("mix_name", ["q4_k_m", "q8_0"])
+def test_decode_wide_model(jn, mix_name):
+    """A residual stream of 5120 values - rows longer than 4096 for q, k, v, gate and up, which the norm-fused launches do not
+    take: a norm kernel of its own, then every linear with one wave per 1024 values (five here) - two tokens on a pre-filled
+    cache."""
+    cfg = dict(layers=1, d_model=5120, heads=8, kv_heads=2, head_dim=64, ffn=768, vocab=512, max_ctx=40, rms_eps=1e-5, rope_theta=1e4)
+    mix = {"q4_k_m": MIX, "q8_0": {s: "Q8_0" for s in SLOTS}}[mix_name]
+    dec, layers, out_norm, out_w = build(jn, cfg, 9, mix, "Q6_K")
+    rng = np.random.default_rng(2)
+    ctx0 = 33
+    kc = np.zeros((cfg["layers"], cfg["max_ctx"], cfg["kv_heads"], cfg["head_dim"]), dtype=np.float32)
+    vc = np.zeros_like(kc)
+    kc[:, :ctx0] = rng.standard_normal(kc[:, :ctx0].shape)
+    vc[:, :ctx0] = rng.standard_normal(vc[:, :ctx0].shape)
+    dec.kv_write(0, 0, kc[0, :ctx0], vc[0, :ctx0])
+    for step in range(2):
+        pos = ctx0 + step
+        x = rng.standard_normal(cfg["d_model"]).astype(np.float32)
+        ref = decode_ref(cfg, layers, out_norm, out_w, kc, vc, x, pos)
+        y = dec.decode(x, pos)
+        assert norm_err(y, ref) <= 1e-4, (mix_name, step, norm_err(y, ref))
+    dec.close()
+
+
 @pytest.mark.parametrize("mix_name", ["q4_k_m", "q8_0", "q4_0_q5_k", "q4_k_q5_k", "q5_k_m", "q6_k", "q4_1"])
 def test_decode_small_model(jn, mix_name):
     """Two layers, grouped heads 8/2 of size 64, three tokens decoded in a row on a pre-filled cache.  The mixes cover the
