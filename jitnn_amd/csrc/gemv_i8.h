@@ -39,7 +39,8 @@ __host__ __device__ constexpr int i8_flush(int rows) { return rows == 1 ? 36 : 1
 // LDS of a wave: 16 chunks x 3 planes x 64 bytes while the activations are staged; afterwards the wave's partial sums,
 // 2 windows x flush turns x rows x 16 floats
 __host__ __device__ constexpr size_t gemv_i8_lds_per_wave(int rows) {
-    return (size_t)2 * i8_flush(rows) * rows * 64 > 3072 ? (size_t)2 * i8_flush(rows) * rows * 64 : 3072;
+    const size_t stage = rows == 4 ? 4 * 3072 : 3072, sums = (size_t)2 * i8_flush(rows) * rows * 64;  // (four rows: all their planes at once)
+    return sums > stage ? sums : stage;
 }
 __host__ __device__ constexpr size_t gemv_i8_lds_bytes(int waves, int rows = 1) { return (size_t)waves * gemv_i8_lds_per_wave(rows); }
 
@@ -538,16 +539,42 @@ __device__ __forceinline__ void i8_dot(const typename U::Raw &r, int c, const ui
     U::extract(r, c, v);
     typename U::Scale sc;
     U::scales(r, c, sc);
+    if constexpr (B == 4) {
+        // Four rows have twelve digit planes, and a product has four operand rows: packed - operand set m = the plane vectors
+        // 4 m .. 4 m + 3, vector 3 r + p being plane p of row r - they fill three products where a product per row leaves a quarter
+        // of four empty.  The sums of (weight row j, chunk b) still all come back to lane 4 b + j: row r's three are picked out of
+        // the three results by constant indices.
+        i32x4 d[3][CH];
 #pragma unroll
-    for (int b = 0; b < B; ++b) {
-        i32x4 d[CH];
+        for (int m = 0; m < 3; ++m)
 #pragma unroll
-        for (int ch = 0; ch < CH; ++ch) d[ch] = i32x4{0, 0, 0, 0};
+            for (int ch = 0; ch < CH; ++ch) d[m][ch] = i32x4{0, 0, 0, 0};
 #pragma unroll
         for (int i = 0; i < L; ++i)
 #pragma unroll
-            for (int ch = 0; ch < CH; ++ch) d[ch] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[b][ch * L + i], (int)v[ch * L + i], d[ch], 0, 0, 0);
-        out[b] = U::finish(sc, d, sinv[b], s[b]);
+            for (int ch = 0; ch < CH; ++ch)
+#pragma unroll
+                for (int m = 0; m < 3; ++m) d[m][ch] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[m][ch * L + i], (int)v[ch * L + i], d[m][ch], 0, 0, 0);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            i32x4 dd[CH];
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch)
+                dd[ch] = i32x4{d[(3 * b) / 4][ch][(3 * b) % 4], d[(3 * b + 1) / 4][ch][(3 * b + 1) % 4], d[(3 * b + 2) / 4][ch][(3 * b + 2) % 4], 0};
+            out[b] = U::finish(sc, dd, sinv[b], s[b]);
+        }
+    } else {
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            i32x4 d[CH];
+#pragma unroll
+            for (int ch = 0; ch < CH; ++ch) d[ch] = i32x4{0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < L; ++i)
+#pragma unroll
+                for (int ch = 0; ch < CH; ++ch) d[ch] = __builtin_amdgcn_mfma_i32_4x4x4i8((int)xa[b][ch * L + i], (int)v[ch * L + i], d[ch], 0, 0, 0);
+            out[b] = U::finish(sc, d, sinv[b], s[b]);
+        }
     }
 }
 
@@ -697,8 +724,25 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
     uint32_t xa[B][16];
     float sinv[B], sums[B][U::NSUM];
     bool slow = false;
+    if constexpr (B == 4) {
+        // (four rows: every row's planes into a region of its own, then the lane's three packed operand sets - see i8_dot)
+        uint32_t unused[16];
 #pragma unroll
-    for (int r = 0; r < B; ++r) slow = i8_stage<U>(xv[r], planes, b, j, xa[r], sinv[r], sums[r]) || slow;  // an Inf or NaN in this wave's slice
+        for (int r = 0; r < 4; ++r) slow = i8_stage<U>(xv[r], planes + r * 192, b, j, unused, sinv[r], sums[r]) || slow;
+#pragma unroll
+        for (int m = 0; m < 3; ++m) {
+            const int vec = 4 * m + j, rr = vec / 3, p = vec - 3 * rr;
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const u32x4 v = planes[rr * 192 + (b * 3 + p) * 4 + qd];
+                xa[m][qd * 4 + 0] = v.x; xa[m][qd * 4 + 1] = v.y; xa[m][qd * 4 + 2] = v.z; xa[m][qd * 4 + 3] = v.w;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    } else {
+#pragma unroll
+        for (int r = 0; r < B; ++r) slow = i8_stage<U>(xv[r], planes, b, j, xa[r], sinv[r], sums[r]) || slow;  // an Inf or NaN in this wave's slice
+    }
 
     auto group_of = [&](int t) { return bid + (DUAL ? t >> 1 : t) * nblocks; };
     // one output of a window: the partial sums of all waves in wave order
