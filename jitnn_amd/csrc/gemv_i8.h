@@ -34,8 +34,9 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int I8_MAX_WAVES = 16;
 // turns between two joins of the waves' partial sums (a multiple of every ring length): 36 for one activation row - the 28 turns
-// of a gate / up launch of an 8B layer fit one window: 14.1 against 14.5 us with 24 -, 12 for more
-__host__ __device__ constexpr int i8_flush(int rows) { return rows == 1 ? 36 : 12; }
+// of a gate / up launch of an 8B layer fit one window: 14.1 against 14.5 us with 24 -, 24 for more (the 14 turns of a 14336-row
+// matrix in one window: Q4_K 14336 x 4096 at two rows 9.2 against 10.2 us with 12)
+__host__ __device__ constexpr int i8_flush(int rows) { return rows == 1 ? 36 : 24; }
 // LDS of a wave: 16 chunks x 3 planes x 64 bytes while the activations are staged; afterwards the wave's partial sums,
 // 2 windows x flush turns x rows x 16 floats
 __host__ __device__ constexpr size_t gemv_i8_lds_per_wave(int rows) {

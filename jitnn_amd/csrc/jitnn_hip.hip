@@ -317,8 +317,8 @@ int launch_i8(const XregCall &c, hipStream_t stream) {
 
 // Two to four activation rows, rows of at most 4096 values: the same kernel with the activations of all rows in registers - the
 // operands and scales of the weights are made once, every row runs its own chains of products.  us per launch against the FP32
-// two-row kernel / gemv_mfma_kernel - Q4_K 14336 x 4096: 10.2 (11.3) at two rows, 12.0 (13.9) at three, 12.2 (13.8) at four; Q4_0
-// 11008 x 4096 at four: 9.9 (11.8); Q8_0 4096 x 4096: 7.0 (10.1); Q6_K 14336 x 4096: 15.1 (23.0).  The number of its 4x4x4 products
+// two-row kernel / gemv_mfma_kernel - Q4_K 14336 x 4096: 9.2 (11.3) at two rows, 11.1 (13.9) at three, 11.5 (13.8) at four; Q4_0
+// 11008 x 4096 at four: 9.9 (11.8); Q8_0 4096 x 4096: 7.0 (10.1); Q6_K 14336 x 4096: 14.7 (23.0).  The number of its 4x4x4 products
 // grows with the rows (four rows: twelve digit planes in three products a step): eight rows (two groups of four along
 // blockIdx.y) stay behind gemv_mfma_kernel, whose 16-row tiles take 14.5 us whatever the rows - from five rows on those stay
 // ahead, except for Q6_K, whose tiles cost the most there (14336 x 4096 at eight rows: 23.1 against 28.4 us).
