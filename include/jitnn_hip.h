@@ -15,7 +15,7 @@
  *    Q5_0=6 Q5_1=7 Q2_K=10 Q3_K=11 (the other block formats the reference dequantises,
  *    core/kernels/GgufKernels.java:147-198: bit-exact dequantiser; Q5_0 and Q3_K are served by the Q8_0 / Q6_K
  *    kernels after an exact rewrite at upload, Q5_1 and Q2_K by units of their own in the batch-1 kernel - up to four
- *    rows a launch, more as a chain of launches - and by the many-row kernel beyond 64 rows).
+ *    rows a launch -, by tiles of their own in the one-pass kernel from five rows to 64, and by the many-row kernel beyond).
  *  - A weight is [n, k] row-major rows of k/block_values blocks, byte-for-byte as in the GGUF file
  *    (core/Tensor.java:249-278); it stays in that layout in HBM.
  *  - Activations and outputs are FP32 row-major: x [rows, k], y [rows, n], bias [n].

@@ -154,9 +154,10 @@ struct RStaged {
     static constexpr int STRIDE = ROW_STRIDE;
     static constexpr int STAGE_BYTES = 16 * STRIDE;
     static constexpr bool STAGED = true;
-    static_assert(REST > 0 && STRIDE >= 16 * CHUNKS && STRIDE % 16 == 0, "chunks of sixteen bytes");
+    static constexpr int RD = REST > 0 ? REST : 1;  // (a row of whole four-chunk loads has no load of odd chunks)
+    static_assert(STRIDE >= 16 * CHUNKS && STRIDE % 16 == 0, "chunks of sixteen bytes");
     struct Raw {
-        u32x4 c[FULL + 1];
+        u32x4 c[FULL + (REST > 0 ? 1 : 0)];
         uint32_t tail;  // (formats with bytes past the chunks)
     };
     struct Ptr {
@@ -166,20 +167,22 @@ struct RStaged {
     // r0: first row of the tile
     __device__ static __forceinline__ Ptr ptr(const uint8_t *W, int r0, size_t rowbytes, int lane) {
         const int rb = (int)rowbytes, lr = lane >> 2;
-        return {W + (size_t)(r0 + lr) * rowbytes + 16 * (lane & 3), (((lane / REST) & 15) - lr) * rb + 16 * (4 * FULL + lane % REST - (lane & 3)),
+        return {W + (size_t)(r0 + lr) * rowbytes + 16 * (lane & 3), (((lane / RD) & 15) - lr) * rb + 16 * (4 * FULL + lane % RD - (lane & 3)),
                 ((lane & 15) - lr) * rb - 16 * (lane & 3)};
     }
     __device__ static __forceinline__ void load(Raw &r, const Ptr &p, int c) {
         const uint8_t *q = p.full + (size_t)c * BYTES;
 #pragma unroll
         for (int i = 0; i < FULL; ++i) r.c[i] = ld128<ALIGN>(q + 64 * i);
-        r.c[FULL] = ld128<ALIGN>(q + p.rest);  // (lanes past 16 REST repeat rows: the same lines)
+        if constexpr (REST > 0) r.c[FULL] = ld128<ALIGN>(q + p.rest);  // (lanes past 16 REST repeat rows: the same lines)
     }
     // -> this lane's row (lane & 15 of the tile) in the wave's stage
     __device__ static __forceinline__ const uint8_t *park(const Raw &r, uint8_t *stage, int lane) {
 #pragma unroll
         for (int i = 0; i < FULL; ++i) *reinterpret_cast<u32x4 *>(stage + (lane >> 2) * STRIDE + 16 * (lane & 3) + 64 * i) = r.c[i];
-        if (lane < 16 * REST) *reinterpret_cast<u32x4 *>(stage + (lane / REST) * STRIDE + 16 * (4 * FULL + lane % REST)) = r.c[FULL];
+        if constexpr (REST > 0) {
+            if (lane < 16 * REST) *reinterpret_cast<u32x4 *>(stage + (lane / RD) * STRIDE + 16 * (4 * FULL + lane % RD)) = r.c[FULL];
+        }
         // the lanes of a wave run in step and LDS serves them in order: a fence for the compiler is all this needs
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -413,6 +416,92 @@ struct RTile<F_Q8_0> : RStaged<8 * 34, 272, 2> {
             dblk[s] = h2f(ld16(row + 34 * s));
         }
         Bm = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+};
+
+// Q5_1: blocks of 24 bytes - d, m, 32 fifth bits (bit i: value i), 16 bytes of nibbles (core/kernels/GgufKernels.java:155-163) -
+// are Q4_1 blocks with a bit on top of every nibble: the four bits of a lane's low-nibble values and the four of its
+// high-nibble values are spread to a byte each by one multiplication and OR-ed under the exponent with the nibbles.
+// Eight blocks of a row are 192 bytes: three whole four-chunk loads.
+template <>
+struct RTile<F_Q5_1> : RStaged<8 * 24, 208, 16> {
+    static constexpr int NOPS = 8, SUMS = 32;
+    static constexpr bool BLOCK_SCALES = true, HALVES = true, MINS = true;
+    __device__ static __forceinline__ void decode(const Raw &r, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float (&dblk)[8]) {
+        const uint8_t *row = park(r, stage, lane);
+        const int kq = lane >> 4;
+        const uint32_t mg = magic1024();
+        const f16x2 off = splat2(-1024.f);
+        uint32_t dm[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            const u32x2 hd = *reinterpret_cast<const u32x2 *>(row + 24 * s);  // d | m, the fifth bits
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(row + 24 * s + 8 + 4 * kq);
+            dm[s] = hd.x;
+            const uint32_t h = hd.y >> (4 * kq);
+            // byte e = the fifth bit of value 4 kq + e (of value 16 + 4 kq + e): four disjoint shifted copies, no carries
+            const uint32_t f0 = ((h & 15u) * 0x00204081u) & 0x01010101u, f1 = (((h >> 16) & 15u) * 0x00204081u) & 0x01010101u;
+            B[s] = cat8(as_h2((w & 0x000f000fu) | ((f0 & 0x00010001u) << 4) | mg) + off, as_h2(((w >> 8) & 0x000f000fu) | (((f0 >> 8) & 0x00010001u) << 4) | mg) + off,
+                        as_h2(((w >> 4) & 0x000f000fu) | ((f1 & 0x00010001u) << 4) | mg) + off,
+                        as_h2(((w >> 12) & 0x000f000fu) | (((f1 >> 8) & 0x00010001u) << 4) | mg) + off);
+            dblk[s] = h2f(dm[s]);
+        }
+        u32x4 mb;  // (the offsets m against the block sums of x, as for Q4_1)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) mb[j] = kq == 0 ? (dm[2 * j] >> 16) | (dm[2 * j + 1] & 0xffff0000u) : 0u;
+        Bm = __builtin_bit_cast(f16x8, mb);
+    }
+};
+
+// Q2_K: 84 bytes = 16 scale bytes (low nibble: scale, high nibble: min, of 16 values each), qs[64] (2-bit quants), d, dmin.
+// Value 128 n + 32 j + l is bits 2 j, 2 j + 1 of qs[32 n + l], its scale byte number 8 n + 2 j + l / 16
+// (core/kernels/GgufKernels.java:166-175): Q6_K's element order and scale index, with a 4-bit scale (scale times quant at most
+// 45: one exact operand per step) and, like Q4_K, minima - against the sums of x per 16 values - under a dmin of their own.
+template <>
+struct RTile<F_Q2_K> : RStaged<84, 80, 4> {
+    static constexpr int NOPS = 8, SUMS = 16;
+    static constexpr bool BLOCK_SCALES = false, HALVES = false, MINS = true;
+    __device__ static constexpr int aidx(int q) { return q; }
+    // five chunks and d | dmin, the last four bytes of the block, straight to the lanes of its row
+    __device__ static __forceinline__ void load(Raw &r, const Ptr &p, int c) {
+        RStaged<84, 80, 4>::load(r, p, c);
+        r.tail = ld32<4>(p.full + (size_t)c * BYTES + p.row + 80);
+    }
+    __device__ static __forceinline__ void decode(const Raw &raw, uint8_t *stage, int lane, f16x8 (&B)[8], f16x8 &Bm, float &d, float &dmin) {
+        const uint8_t *p = park(raw, stage, lane);
+        const int kq = lane >> 4;
+        const u32x4 sc = *reinterpret_cast<const u32x4 *>(p);
+        u32x2 q[2];
+#pragma unroll
+        for (int n = 0; n < 2; ++n) q[n] = *reinterpret_cast<const u32x2 *>(p + 16 + 32 * n + 8 * kq);
+        d = h2f(raw.tail);
+        dmin = h2f(raw.tail >> 16);
+        const uint32_t mg = magic1024();
+#pragma unroll
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int ty = 0; ty < 4; ++ty) {
+                const int is0 = 8 * n + 2 * ty;  // (even: the scale bytes is0 and is0 + 1 share a dword)
+                const float scf = (float)((sc[is0 >> 2] >> (8 * ((is0 & 3) + (kq >> 1)))) & 15u);
+                const f16x2 ml = splat2(scf), al = splat2(-1024.f * scf);  // (1024 + q) sc - 1024 sc
+                f16x2 v[4];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const uint32_t w = (t ? q[n].y : q[n].x) >> (2 * ty);
+                    v[2 * t] = h2fma((w & 0x00030003u) | mg, ml, al);             // bytes 0, 2
+                    v[2 * t + 1] = h2fma(((w >> 8) & 0x00030003u) | mg, ml, al);  // bytes 1, 3
+                }
+                B[4 * n + ty] = cat8(v[0], v[1], v[2], v[3]);
+            }
+        // operand of the minima: slot j of the lanes kq = 0 (1) = the min of scale byte j (j + 8); the other lanes zero
+        const uint32_t s0 = kq == 0 ? sc.x : sc.z, s1 = kq == 0 ? sc.y : sc.w;
+        f16x2 m[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t sw = (j < 2 ? s0 : s1) >> (16 * (j & 1));
+            m[j] = kq < 2 ? f16x2{(_Float16)(float)((sw >> 4) & 15u), (_Float16)(float)((sw >> 12) & 15u)} : f16x2{(_Float16)0.f, (_Float16)0.f};
+        }
+        Bm = cat8(m[0], m[1], m[2], m[3]);
     }
 };
 

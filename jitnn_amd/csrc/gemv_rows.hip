@@ -41,6 +41,8 @@ KernelRef gemv_rows_kernel_ref(int fmt, int n, int k, int rows, unsigned max_blo
     case F_Q4_0: return kernel_ref<F_Q4_0>(two);
     case F_Q4_1: return kernel_ref<F_Q4_1>(two);
     case F_Q8_0: return kernel_ref<F_Q8_0>(two);
+    case F_Q5_1: return kernel_ref<F_Q5_1>(two);
+    case F_Q2_K: return kernel_ref<F_Q2_K>(two);
     default: return {nullptr, 0};
     }
 }
@@ -59,6 +61,8 @@ int gemv_rows_layout(int fmt) {
     case F_Q4_0: return layout_of<F_Q4_0>();
     case F_Q4_1: return layout_of<F_Q4_1>();
     case F_Q8_0: return layout_of<F_Q8_0>();
+    case F_Q5_1: return layout_of<F_Q5_1>();
+    case F_Q2_K: return layout_of<F_Q2_K>();
     default: return -1;
     }
 }
@@ -107,6 +111,8 @@ void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const ui
     case F_Q4_0: launch<F_Q4_0>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
     case F_Q4_1: launch<F_Q4_1>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
     case F_Q8_0: launch<F_Q8_0>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
+    case F_Q5_1: launch<F_Q5_1>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
+    case F_Q2_K: launch<F_Q2_K>(max_blocks, s, W, scratch, bias, res, y, n, k, rows); break;
     default: break;
     }
 }

@@ -558,8 +558,9 @@ int launch_gemv(const jitnn_hip_weight *w, const float *x, int rows, const float
             c.x = x;
             if (i8_ok(c)) return launch_i8(c, stream);
         } else if (i8_batch_ok(w, rows < 4 ? rows : 4)) {
-            // up to four rows per launch; more rows (the one-pass kernel of 9..64 rows has no decoder for these formats) as a chain
-            // of such launches, each streaming the weights again - Q5_1 14336 x 4096 at 40 rows 150 us where the plain kernel takes 443
+            // up to four rows per launch; more rows - where the one-pass kernel of gemv_rows.h does not take the shape (it has tiles
+            // for both formats: 14336 x 4096 at 5..8 rows Q5_1 23 us, Q2_K 19 us against 28, 29 as two launches here) - as a chain of
+            // such launches, each streaming the weights again
             for (int r0 = 0; r0 < rows; r0 += 4)
                 if (int rc = launch_i8_batch(w, x + (size_t)r0 * w->k, rows - r0 < 4 ? rows - r0 : 4, bias, y + (size_t)r0 * w->n, stream)) return rc;
             return JITNN_HIP_OK;
@@ -1179,6 +1180,7 @@ bool rows_path(const jitnn_hip_weight *w, int rows) {
     int rows_min = 9;  // (up to 8 rows gemv_mfma_kernel is faster)
     if (w->k >= 12288) rows_min = 3;
     else if (w->fmt == F_Q4_0 || w->fmt == F_Q4_1) rows_min = 12;
+    else if (is_extra_format(w->fmt)) rows_min = 5;  // (Q5_1, Q2_K: up to four rows are one launch of the INT8 kernel)
     return rows >= rows_min && rows <= 64 && rows <= g.gemv_max_rows && gemv_rows_supported(w->fmt) && w->k % 256 == 0 &&
            w->n >= 16;
 }

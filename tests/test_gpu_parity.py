@@ -203,19 +203,20 @@ def test_small_k_32_blocks_and_many_rows(jn, fmt):
         assert norm_err(y, ref) <= bar(rows), (fmt, rows, norm_err(y, ref))
 
 
-@pytest.mark.parametrize("fmt", ["Q4_K", "Q5_K", "Q6_K", "Q4_0", "Q4_1", "Q8_0"])
+@pytest.mark.parametrize("fmt", ["Q4_K", "Q5_K", "Q6_K", "Q4_0", "Q4_1", "Q8_0", "Q5_1", "Q2_K"])
 @pytest.mark.parametrize("n,k", [(16, 256), (100, 2048), (1000, 4096 + 256), (259, 14336)])
 def test_one_pass_rows_kernel(jn, fmt, n, k):
     """9..64 rows take one pass over the weights (K-quants: block scales folded into FP16 weight operands; 32-value
     formats: the quants as operands, every block's sum scaled on its own; the activations split hi + lo): whole and
     ragged tiles of 16 weight rows, one to many 256-value columns, every number of groups of eight rows, bias, and
-    activation rows of very different magnitudes - bar 1e-4 of the largest output per row."""
+    activation rows of very different magnitudes - bar 1e-4 of the largest output per row.  (Q5_1 - a Q4_1 tile with a
+    fifth bit - and Q2_K - Q6_K's element order, 4-bit scales and minima - take this kernel from five rows.)"""
     from oracle import oracle
     rng = np.random.default_rng(n + k + GGML_ID[fmt])
     raw = random_valid_blocks(rng, fmt, n, k)
     w = weight(jn, fmt, raw, n, k)
     bias = rng.standard_normal(n).astype(np.float32)
-    for rows in (9, 16, 24, 33, 40, 57, 64):
+    for rows in ((5, 8) if fmt in ("Q5_1", "Q2_K") else ()) + (9, 16, 24, 33, 40, 57, 64):
         x = rng.standard_normal((rows, k)).astype(np.float32)
         x[1] *= np.float32(1e6)
         x[2] *= np.float32(1e-6)
