@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import ggml_numpy
-from helpers import (GGML_ID, GGML_NAMES, GOLDEN_CODE_TO_GGML, HOT_FORMATS, JavaRandom, checks_close, java_string_hash, norm_err,
+from helpers import (BLOCK, GGML_ID, GGML_NAMES, GOLDEN_CODE_TO_GGML, HOT_FORMATS, JavaRandom, checks_close, java_string_hash, norm_err,
                      random_valid_blocks)
 
 pytestmark = pytest.mark.gpu
@@ -433,6 +433,42 @@ def test_batch_1_and_2_random_shapes_all_formats(jn):
         y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias) if bias is not None else None).numpy()
         assert y.shape == (rows, n)
         assert norm_err(y, ref) <= GEMV_BAR, (case, fmt, n, k, rows, norm_err(y, ref))
+
+
+def test_random_shapes_any_row_count_all_formats(jn):
+    """Eighty seeded linears - one to 80 activation rows, one to 700 weight rows, rows of whole 256-value columns up to 16128
+    values and of any whole number of blocks up to 8192, one activation row in four scaled by 1e5, with and without bias, all
+    ten block formats - against the oracle: every routing border (INT8 units up to four rows, matrix-core tiles to eight, the
+    one-pass kernel to 64, the many-row kernel beyond; the shapes each of them leaves to the plain kernels).  Bars: 1e-4 of the
+    largest output of each activation row up to 64 rows (of the whole output where a row has fewer than 32 outputs to take a
+    scale from), 2e-3 of the largest output beyond (the normalisation of GgufChecks.close, GgufChecks.java:110-120)."""
+    from oracle import oracle
+    rng = np.random.default_rng(20262)
+    fmts = ["Q4_K", "Q5_K", "Q6_K", "Q4_0", "Q4_1", "Q8_0", "Q5_1", "Q2_K", "Q5_0", "Q3_K"]
+    for case in range(80):
+        fmt = fmts[case % len(fmts)]
+        kq = BLOCK[fmt][0]
+        if case % 7 == 0:
+            k = 256 * int(rng.integers(1, 17))
+        elif case % 7 == 1:
+            k = 256 * int(rng.integers(17, 64))
+        else:
+            k = kq * int(rng.integers(1, 8192 // kq + 1))
+        n = int(rng.integers(1, 700)) if case % 3 else int(rng.integers(1, 40))
+        rows = int(rng.integers(1, 81))
+        raw = random_valid_blocks(rng, fmt, n, k)
+        w = weight(jn, fmt, raw, n, k)
+        x = rng.standard_normal((rows, k)).astype(np.float32)
+        if case % 4 == 0:
+            x[rng.integers(0, rows)] *= np.float32(1e5)
+        bias = rng.standard_normal(n).astype(np.float32) if case % 2 else None
+        ref = oracle.gguf_linear(GGML_ID[fmt], x, raw, bias, n, k).astype(np.float64)
+        y = jn.Gguf.linear(jn.Tensor.of(x), w, jn.Tensor.of(bias) if bias is not None else None).numpy().astype(np.float64)
+        if n >= 32 and rows <= 64:
+            err = max(float(np.abs(y[r] - ref[r]).max()) / max(float(np.abs(ref[r]).max()), 1e-30) for r in range(rows))
+        else:
+            err = float(np.abs(y - ref).max()) / max(float(np.abs(ref).max()), 1e-30)
+        assert err <= (MFMA_BAR if rows > 64 else GEMV_BAR), (case, fmt, n, k, rows, err)
 
 
 @pytest.mark.parametrize("fmt", ["Q5_1", "Q2_K"])
