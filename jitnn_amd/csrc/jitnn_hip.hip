@@ -291,13 +291,15 @@ int i8_args(const XregCall &c, I8Args &a) {
 }
 
 // workgroups and turns in flight for a launch of `groups` row groups (four rows each) of `waves`-wave workgroups
-void i8_shape(int groups, int waves, bool dual, int &blocks, int &pf) {
+void i8_shape(int fmt, int groups, int waves, bool dual, int &blocks, int &pf) {
     // Measured (us, pf / workgroups per CU): Q4_K 14336 x 4096 8.40 (1/2) 8.44 (2/1) 8.48 (3/1) 9.54 (1/4); Q4_K 4096 x 4096 4.75 (1/2)
     // 4.93 (1/1) 5.82 (1/4); Q6_K 128256 x 4096 71.9 (2/1) 72.9 (3/1) 73.6 (1/1) 74.5 (1/2); Q6_K 4096 x 14336 (14 waves) 12.9
     // (1/1) 14.3 (2/1) 16.2 (1/2).  Tall matrices: one workgroup per CU with two turns in flight behind the one being
     // multiplied; short ones: two workgroups with one; long rows: one with one.
     const int turns1 = (groups + g.cus - 1) / g.cus;
-    const int per_cu = waves > 4 ? 1 : turns1 >= 8 ? 1 : 2;
+    // (Q8_0, twice the bytes of a 4-bit format per turn: one workgroup per CU on short matrices too - 4096 x 4096 5.50 us (1/1) against
+    // 5.74 (1/2), 5.72 (2/1), 6.31 (2/2), 6.67 (1/3), 7.15 (1/4))
+    const int per_cu = waves > 4 ? 1 : turns1 >= 8 ? 1 : (fmt == F_Q8_0 && turns1 >= 4) ? 1 : 2;
     pf = waves > 4 ? 1 : turns1 >= 8 ? (dual ? 3 : 2) : 1;  // (gate + up of an 8B layer: 14.4 us with three turns in flight, 15.1 with two)
     blocks = groups < g.cus * per_cu ? groups : g.cus * per_cu;
 }
@@ -307,7 +309,7 @@ int launch_i8(const XregCall &c, hipStream_t stream) {
     const int n = i8_args(c, a);
     const int mode = c.w2 ? I8_DUAL : c.norm_w ? I8_NORM : c.bias ? I8_BIAS : I8_PLAIN;
     int blocks, pf;
-    i8_shape((n + 3) / 4, (a.k + 1023) / 1024, c.w2 != nullptr, blocks, pf);
+    i8_shape(c.w[0]->fmt, (n + 3) / 4, (a.k + 1023) / 1024, c.w2 != nullptr, blocks, pf);
     if (c.w[0]->fmt == F_Q5_K && pf > 2) pf = 2;  // (five loads per turn: a fourth buffer does not fit 128 registers)
     if (!gemv_i8_launch(c.w[0]->fmt, mode, pf, (unsigned)blocks, stream, a))
         return fail(JITNN_HIP_EDEVICE, "no INT8 GEMV kernel for format %d in mode %d, rows of %d values", c.w[0]->fmt, mode, a.k);
@@ -398,7 +400,7 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
         const int ga = (i8_args(ca, a) + 3) / 4, gb = (i8_args(cb, b) + 3) / 4;
         const double ba = (double)ga * ca.w[0]->nbytes / ca.w[0]->n, bb = (double)gb * cb.w[0]->nbytes / cb.w[0]->n;
         int total, pf;
-        i8_shape(ga + gb, (a.k + 1023) / 1024, false, total, pf);
+        i8_shape(ca.w[0]->fmt, ga + gb, (a.k + 1023) / 1024, false, total, pf);
         // (q, k | v of an 8B layer - 1536 row groups, six per CU -, us per launch by workgroups per CU / turns in flight: 6.7 (1 / 2)
         // 7.1 (1 / 1) 8.0 (2 / 1) 8.4 (2 / 2) 9.1 (3 / 1): the two formats' workgroups pace differently, one per CU keeps them apart)
         if (ga + gb >= 4 * g.cus) {
