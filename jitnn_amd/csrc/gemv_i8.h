@@ -634,24 +634,34 @@ __device__ __forceinline__ bool i8_stage(const float4 (&xv)[4], u32x4 *planes, i
     return nonfinite;
 }
 
+// what a wave needs before its first loads: the first matrix, the activations, (DUAL) the second matrix, (NORM) the norm weight,
+// the row length and the number of rows of all segments
+struct I8Lead {
+    const uint8_t *w0;
+    const float *x;
+    const uint8_t *w2;
+    const float *nw;
+    int k, n;
+};
+
 // -------------------------------------------------------------------------------------------------- the kernel body
 // rb: the first activation row of this workgroup (launches of more than B rows put the row groups of B along blockIdx.y:
 // their workgroups stream the same weight bytes at the same time, so one of them finds them in the cache)
 template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
-__device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, const int nblocks, const int rb = 0) {
+__device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, const int bid, const int nblocks, const int rb = 0) {
     constexpr int FMT = U::FMT, NB = PF + 1, FL = i8_flush(B);
     static_assert(FL % NB == 0 && FL % 2 == 0, "whole rings (and gate/up pairs) per flush window");
     static_assert(B == 1 || (!NORM && !DUAL), "the fused norm and the SwiGLU pair are batch-1 launches");
     extern __shared__ __align__(16) uint8_t i8_smem[];
     __shared__ float red[I8_MAX_WAVES];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = blockDim.x >> 6;
+    const int k = ld.k, chunks = k >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = (k + 1023) >> 10;  // (the launch has one wave per 1024 values of a row)
     constexpr size_t WAVE_LDS = gemv_i8_lds_per_wave(B);
     u32x4 *const planes = reinterpret_cast<u32x4 *>(i8_smem + (size_t)wave * WAVE_LDS);
     float *const mypart = reinterpret_cast<float *>(planes);  // after the staging: [2][FL][B][4 dpp rows][4 rows] partial sums of this wave
     const int b = lane >> 2, j = lane & 3;
-    const int k = a.k, chunks = k >> 6;
-    const int n = a.n[0] + a.n[1] + a.n[2];
+    const int n = ld.n;
     const int groups = (n + 3) >> 2;
     const size_t rowbytes = (size_t)(k / block_values(FMT)) * block_bytes(FMT);
     const bool inrow = wave * 16 + b < chunks;      // lanes past the end of the row: zero activations
@@ -667,11 +677,11 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
     for (int r = 0; r < B; ++r) {
         const bool have = inrow && (B == 1 || rb + r < a.rows);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) xv[r][i] = have ? reinterpret_cast<const float4 *>(a.x + (size_t)(rb + r) * k + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int i = 0; i < 4; ++i) xv[r][i] = have ? reinterpret_cast<const float4 *>(ld.x + (size_t)(rb + r) * k + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     if (NORM) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) nv[i] = inrow ? reinterpret_cast<const float4 *>(a.nw + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int i = 0; i < 4; ++i) nv[i] = inrow ? reinterpret_cast<const float4 *>(ld.nw + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 
     // ---- the ring of weight bytes
@@ -684,8 +694,8 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
     // Row segments (several matrices in one launch) exist only where the decode step uses them: with the fused norm.  Every other
     // launch has one matrix, and its per-turn scalar arithmetic - which a wave alone on its SIMD pays in full - stays short.
     constexpr bool SEGMENTS = NORM && !DUAL;
-    const uint8_t *const w0 = a.w[0], *const wd = a.w2;
-    const ptrdiff_t d01 = SEGMENTS ? a.w[1] - a.w[0] : 0, d12 = SEGMENTS ? a.w[2] - a.w[1] : 0;
+    const uint8_t *const w0 = ld.w0, *const wd = ld.w2;
+    const ptrdiff_t d01 = SEGMENTS ? a.w[1] - ld.w0 : 0, d12 = SEGMENTS ? a.w[2] - a.w[1] : 0;
     const int n0 = SEGMENTS ? a.n[0] : n, n01 = SEGMENTS ? a.n[0] + a.n[1] : n;
     auto fill = [&](typename U::Raw &dst, int t) {
         const int g = bid + (DUAL ? t >> 1 : t) * nblocks;
@@ -807,9 +817,9 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
                         for (int e = 0; e < 64; e += 4) {
                             const int p = U::x_pos(c, e);
                             const float4 w4 = dequant4<FMT>(rp, (size_t)p);
-                            float4 x4 = *reinterpret_cast<const float4 *>(a.x + (size_t)(rb + r) * k + p);
+                            float4 x4 = *reinterpret_cast<const float4 *>(ld.x + (size_t)(rb + r) * k + p);
                             if (NORM) {
-                                const float4 n4 = *reinterpret_cast<const float4 *>(a.nw + p);
+                                const float4 n4 = *reinterpret_cast<const float4 *>(ld.nw + p);
                                 x4 = make_float4(x4.x * n4.x, x4.y * n4.y, x4.z * n4.z, x4.w * n4.w);
                             }
                             acc = __builtin_fmaf(w4.x, x4.x, acc);
@@ -830,7 +840,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
             nscale = 1.f / sqrtf(tot / (float)k + a.eps);
         }
         const int outs = DUAL ? 2 * (tend - t0) : 4 * B * (tend - t0);
-        for (int o = tid; o < outs; o += (int)blockDim.x) {  // (a one-wave workgroup has fewer threads than a window has outputs)
+        for (int o = tid; o < outs; o += 64 * waves) {  // (a one-wave workgroup has fewer threads than a window has outputs)
             if (DUAL) {
                 const int pr = o >> 2, jj = o & 3;
                 const int g = group_of(t0 + 2 * pr), row = min(4 * g, n - 4) + jj;
@@ -856,17 +866,23 @@ __device__ __forceinline__ void gemv_i8_body(const I8Args &a, const int bid, con
     }
 }
 
+// The leading arguments are what a wave needs before its first loads can leave - the translation unit is built with kernel-argument
+// preloading, which hands them to the wave in scalar registers at its start; everything in `a` is fetched where it is needed (the
+// outputs, biases and segment bounds: at the first flush), off the path to the first weight load.
 template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
-__global__ void __launch_bounds__(64 * MAXW, (B > 1 ? 2 : 4)) gemv_i8_kernel(const I8Args a) {
-    gemv_i8_body<U, B, PF, BIAS, NORM, DUAL, MAXW>(a, blockIdx.x, gridDim.x, B * (int)blockIdx.y);
+__global__ void __launch_bounds__(64 * MAXW, (B > 1 ? 2 : 4)) gemv_i8_kernel(const uint8_t *w0, const float *x, const int k, const int n, const int nblocks,
+                                                                             const uint8_t *w2, const float *nw, const I8Args a) {
+    const I8Lead ld{w0, x, w2, nw, k, n};
+    gemv_i8_body<U, B, PF, BIAS, NORM, DUAL, MAXW>(ld, a, blockIdx.x, nblocks, B * (int)blockIdx.y);
 }
 
 // Two sets of matrices in two formats over the same (normalised) activations in one launch - the q / k and the v
 // projections of a Q4_K_M layer: workgroups below `split` run the first set, the others the second.
 template <class UA, class UB, int PF, int MAXW>
-__global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_pair_kernel(const I8Args a, const I8Args b, const int split) {
-    if ((int)blockIdx.x < split) gemv_i8_body<UA, 1, PF, false, true, false, MAXW>(a, blockIdx.x, split);
-    else gemv_i8_body<UB, 1, PF, false, true, false, MAXW>(b, blockIdx.x - split, gridDim.x - split);
+__global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_pair_kernel(const uint8_t *wa, const uint8_t *wb, const float *x, const float *nw, const int k, const int na,
+                                                                    const int nb, const int split, const int total, const I8Args a, const I8Args b) {
+    if ((int)blockIdx.x < split) gemv_i8_body<UA, 1, PF, false, true, false, MAXW>(I8Lead{wa, x, nullptr, nw, k, na}, a, blockIdx.x, split);
+    else gemv_i8_body<UB, 1, PF, false, true, false, MAXW>(I8Lead{wb, x, nullptr, nw, k, nb}, b, blockIdx.x - split, total - split);
 }
 
 }  // namespace jitnn

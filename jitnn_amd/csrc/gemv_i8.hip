@@ -11,7 +11,7 @@ bool gemv_i8_supported(int fmt, int k) {
     return (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K || fmt == F_Q2_K) && k % 256 == 0 && k >= 256 && k <= 1024 * I8_MAX_WAVES;
 }
 
-typedef void (*i8_fn)(const I8Args);
+typedef void (*i8_fn)(const uint8_t *, const float *, int, int, int, const uint8_t *, const float *, const I8Args);
 
 template <class U, int PF, int MAXW>
 static i8_fn pick_mode(int mode) {
@@ -88,11 +88,12 @@ bool gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, c
     }
     if (!fn) return false;
     const int bt = batch_of(rows);
-    hipLaunchKernelGGL(fn, dim3(blocks, (rows + bt - 1) / bt), dim3(64 * waves), gemv_i8_lds_bytes(waves, bt), s, a);
+    hipLaunchKernelGGL(fn, dim3(blocks, (rows + bt - 1) / bt), dim3(64 * waves), gemv_i8_lds_bytes(waves, bt), s, a.w[0], a.x, a.k, a.n[0] + a.n[1] + a.n[2], (int)blocks, a.w2,
+                       a.nw, a);
     return true;
 }
 
-typedef void (*i8_pair_fn)(const I8Args, const I8Args, int);
+typedef void (*i8_pair_fn)(const uint8_t *, const uint8_t *, const float *, const float *, int, int, int, int, int, const I8Args, const I8Args);
 
 template <int PF>
 static i8_pair_fn pick_pair(int fa, int fb, bool al) {
@@ -109,7 +110,8 @@ bool gemv_i8_pair_launch(int fmt_a, int fmt_b, int pf, unsigned blocks_a, unsign
     const bool al = fmt_b == F_Q6_K && q6_aligned(b);
     const i8_pair_fn fn = pf <= 1 ? pick_pair<1>(fmt_a, fmt_b, al) : pick_pair<2>(fmt_a, fmt_b, al);
     if (!fn || waves > 4) return false;
-    hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(64 * waves), gemv_i8_lds_bytes(waves), s, a, b, (int)blocks_a);
+    hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(64 * waves), gemv_i8_lds_bytes(waves), s, a.w[0], b.w[0], a.x, a.nw, a.k, a.n[0] + a.n[1] + a.n[2],
+                       b.n[0] + b.n[1] + b.n[2], (int)blocks_a, (int)(blocks_a + blocks_b), a, b);
     return true;
 }
 
