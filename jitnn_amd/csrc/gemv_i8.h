@@ -755,6 +755,15 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
         for (int r = 0; r < B; ++r) slow = i8_stage<U>(xv[r], planes, b, j, xa[r], sinv[r], sums[r]) || slow;  // an Inf or NaN in this wave's slice
     }
 
+    // What the flush needs of the argument block, asked for now: the round trip of the scalar cache runs while the wave would
+    // wait for its first weight bytes anyway - fetched where they are first used, it sits between the last product and the
+    // first store of every launch.
+    asm volatile("" ::"s"(a.y[0]));
+    if constexpr (BIAS) asm volatile("" ::"s"(a.bias[0]));
+    if constexpr (B > 1) asm volatile("" ::"s"(a.rows));
+    if constexpr (NORM) asm volatile("" ::"s"(a.eps));
+    if constexpr (SEGMENTS) asm volatile("" ::"s"(a.y[1]), "s"(a.y[2]), "s"(a.n[0]), "s"(a.n[1]));
+    if constexpr (SEGMENTS && BIAS) asm volatile("" ::"s"(a.bias[1]), "s"(a.bias[2]));
     auto group_of = [&](int t) { return bid + (DUAL ? t >> 1 : t) * nblocks; };
     // one output of a window: the partial sums of all waves in wave order
     // (all reads issued before the first addition - a loop over the workgroup's actual number of waves waits for every wave's four
