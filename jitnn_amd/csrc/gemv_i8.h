@@ -634,28 +634,34 @@ __device__ __forceinline__ bool i8_stage(const float4 (&xv)[4], u32x4 *planes, i
     return nonfinite;
 }
 
-// what a wave needs before its first loads: the first matrix, the activations, (DUAL) the second matrix, (NORM) the norm weight,
-// the row length and the number of rows of all segments
+// What a wave needs before its first loads, as the kernels take it in front of the argument block (fourteen dwords: as many as
+// the hardware preloads into scalar registers): the first matrix, the activations, a second matrix (DUAL: the up projection;
+// row segments: the second segment), the norm weight, the third segment's matrix, three packed numbers, the rows of all segments
+// and of the first two.
 struct I8Lead {
     const uint8_t *w0;
     const float *x;
-    const uint8_t *w2;
+    const uint8_t *wb;  // DUAL: w2; row segments: w[1]
     const float *nw;
-    int k, n;
+    const uint8_t *wc;  // row segments: w[2]
+    int k, nblocks, rows;
+    int n, n0, n1;
 };
+// k / 64 (9 bits: rows of at most 16384 values) | workgroups (20 bits) | activation rows - 1 (3 bits)
+__host__ __device__ constexpr uint32_t i8_pack(int k, int nblocks, int rows) { return (uint32_t)(k >> 6) | ((uint32_t)nblocks << 9) | ((uint32_t)(rows - 1) << 29); }
 
 // -------------------------------------------------------------------------------------------------- the kernel body
 // rb: the first activation row of this workgroup (launches of more than B rows put the row groups of B along blockIdx.y:
 // their workgroups stream the same weight bytes at the same time, so one of them finds them in the cache)
 template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
-__device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, const int bid, const int nblocks, const int rb = 0) {
+__device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, const int bid, const int rb = 0) {
     constexpr int FMT = U::FMT, NB = PF + 1, FL = i8_flush(B);
     static_assert(FL % NB == 0 && FL % 2 == 0, "whole rings (and gate/up pairs) per flush window");
     static_assert(B == 1 || (!NORM && !DUAL), "the fused norm and the SwiGLU pair are batch-1 launches");
     extern __shared__ __align__(16) uint8_t i8_smem[];
     __shared__ float red[I8_MAX_WAVES];
     const int tid = threadIdx.x, lane = tid & 63;
-    const int k = ld.k, chunks = k >> 6;
+    const int k = ld.k, chunks = k >> 6, nblocks = ld.nblocks;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), waves = (k + 1023) >> 10;  // (the launch has one wave per 1024 values of a row)
     constexpr size_t WAVE_LDS = gemv_i8_lds_per_wave(B);
     u32x4 *const planes = reinterpret_cast<u32x4 *>(i8_smem + (size_t)wave * WAVE_LDS);
@@ -675,7 +681,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
     float4 xv[B][4], nv[4];
 #pragma unroll
     for (int r = 0; r < B; ++r) {
-        const bool have = inrow && (B == 1 || rb + r < a.rows);
+        const bool have = inrow && (B == 1 || rb + r < ld.rows);
 #pragma unroll
         for (int i = 0; i < 4; ++i) xv[r][i] = have ? reinterpret_cast<const float4 *>(ld.x + (size_t)(rb + r) * k + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     }
@@ -694,9 +700,9 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
     // Row segments (several matrices in one launch) exist only where the decode step uses them: with the fused norm.  Every other
     // launch has one matrix, and its per-turn scalar arithmetic - which a wave alone on its SIMD pays in full - stays short.
     constexpr bool SEGMENTS = NORM && !DUAL;
-    const uint8_t *const w0 = ld.w0, *const wd = ld.w2;
-    const ptrdiff_t d01 = SEGMENTS ? a.w[1] - ld.w0 : 0, d12 = SEGMENTS ? a.w[2] - a.w[1] : 0;
-    const int n0 = SEGMENTS ? a.n[0] : n, n01 = SEGMENTS ? a.n[0] + a.n[1] : n;
+    const uint8_t *const w0 = ld.w0, *const wd = ld.wb;
+    const ptrdiff_t d01 = SEGMENTS ? ld.wb - ld.w0 : 0, d12 = SEGMENTS ? ld.wc - ld.wb : 0;
+    const int n0 = SEGMENTS ? ld.n0 : n, n01 = SEGMENTS ? ld.n0 + ld.n1 : n;
     auto fill = [&](typename U::Raw &dst, int t) {
         const int g = bid + (DUAL ? t >> 1 : t) * nblocks;
         // extent of the descriptor: everything for a group that exists, nothing past the last group (turns at or past
@@ -760,9 +766,8 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
     // first store of every launch.
     asm volatile("" ::"s"(a.y[0]));
     if constexpr (BIAS) asm volatile("" ::"s"(a.bias[0]));
-    if constexpr (B > 1) asm volatile("" ::"s"(a.rows));
     if constexpr (NORM) asm volatile("" ::"s"(a.eps));
-    if constexpr (SEGMENTS) asm volatile("" ::"s"(a.y[1]), "s"(a.y[2]), "s"(a.n[0]), "s"(a.n[1]));
+    if constexpr (SEGMENTS) asm volatile("" ::"s"(a.y[1]), "s"(a.y[2]));
     if constexpr (SEGMENTS && BIAS) asm volatile("" ::"s"(a.bias[1]), "s"(a.bias[2]));
     auto group_of = [&](int t) { return bid + (DUAL ? t >> 1 : t) * nblocks; };
     // one output of a window: the partial sums of all waves in wave order
@@ -821,7 +826,7 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
 #pragma unroll 1
                 for (int r = 0; r < B; ++r) {
                     float acc = 0.f;
-                    if (B == 1 || rb + r < a.rows) {
+                    if (B == 1 || rb + r < ld.rows) {
 #pragma unroll 1
                         for (int e = 0; e < 64; e += 4) {
                             const int p = U::x_pos(c, e);
@@ -860,10 +865,10 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
             } else {
                 const int jj = o & 3, r = (o >> 2) % B, tt = (o >> 2) / B;
                 const int g = group_of(t0 + tt), row = min(4 * g, n - 4) + jj;
-                if (g < groups && row >= 4 * g && (B == 1 || rb + r < a.rows)) {
+                if (g < groups && row >= 4 * g && (B == 1 || rb + r < ld.rows)) {
                     // (segment pointers by differences, as in fill: no dependent load from the argument block on the way out)
-                    const bool in1 = SEGMENTS && row >= a.n[0], in2 = SEGMENTS && row >= a.n[0] + a.n[1];
-                    const int local = row - (in1 ? a.n[0] : 0) - (in2 ? a.n[1] : 0);
+                    const bool in1 = SEGMENTS && row >= n0, in2 = SEGMENTS && row >= n01;
+                    const int local = row - (in1 ? n0 : 0) - (in2 ? n01 - n0 : 0);
                     float *const yp = a.y[0] + (in1 ? a.y[1] - a.y[0] : 0) + (in2 ? a.y[2] - a.y[1] : 0);
                     float bias = 0.f;
                     if (BIAS) bias = (a.bias[0] + (in1 ? a.bias[1] - a.bias[0] : 0) + (in2 ? a.bias[2] - a.bias[1] : 0))[local];
@@ -875,23 +880,33 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
     }
 }
 
-// The leading arguments are what a wave needs before its first loads can leave - the translation unit is built with kernel-argument
-// preloading, which hands them to the wave in scalar registers at its start; everything in `a` is fetched where it is needed (the
-// outputs, biases and segment bounds: at the first flush), off the path to the first weight load.
+// The leading arguments (I8Lead) are what a wave needs before its first loads can leave - the library is built with kernel-argument
+// preloading, which hands them to the wave in scalar registers at its start; what the flush needs of `a` (outputs, biases) is
+// fetched under the wait for the first weights.
+// (the fused forms - norm, SwiGLU pair, row segments - take all fourteen dwords; a plain or biased launch the six it uses: every
+// preloaded dword is written into every wave's registers at its start, and the headline launch ran 0.15 us longer with fourteen)
 template <class U, int B, int PF, bool BIAS, bool NORM, bool DUAL, int MAXW>
-__global__ void __launch_bounds__(64 * MAXW, (B > 1 ? 2 : 4)) gemv_i8_kernel(const uint8_t *w0, const float *x, const int k, const int n, const int nblocks,
-                                                                             const uint8_t *w2, const float *nw, const I8Args a) {
-    const I8Lead ld{w0, x, w2, nw, k, n};
-    gemv_i8_body<U, B, PF, BIAS, NORM, DUAL, MAXW>(ld, a, blockIdx.x, nblocks, B * (int)blockIdx.y);
+__global__ void __launch_bounds__(64 * MAXW, (B > 1 ? 2 : 4)) gemv_i8_kernel(const uint8_t *w0, const float *x, const uint8_t *wb, const float *nw, const uint8_t *wc,
+                                                                             const uint32_t packed, const int n, const int n0, const int n1, const I8Args a) {
+    static_assert(NORM, "the fused forms");
+    const I8Lead ld{w0, x, wb, nw, wc, (int)(packed & 511u) << 6, (int)((packed >> 9) & 0xfffffu), (int)(packed >> 29) + 1, n, n0, n1};
+    gemv_i8_body<U, B, PF, BIAS, NORM, DUAL, MAXW>(ld, a, blockIdx.x, B * (int)blockIdx.y);
+}
+template <class U, int B, int PF, bool BIAS, int MAXW>
+__global__ void __launch_bounds__(64 * MAXW, (B > 1 ? 2 : 4)) gemv_i8_plain_kernel(const uint8_t *w0, const float *x, const uint32_t packed, const int n, const I8Args a) {
+    const I8Lead ld{w0, x, w0, nullptr, w0, (int)(packed & 511u) << 6, (int)((packed >> 9) & 0xfffffu), (int)(packed >> 29) + 1, n, n, 0};
+    gemv_i8_body<U, B, PF, BIAS, false, false, MAXW>(ld, a, blockIdx.x, B * (int)blockIdx.y);
 }
 
 // Two sets of matrices in two formats over the same (normalised) activations in one launch - the q / k and the v
-// projections of a Q4_K_M layer: workgroups below `split` run the first set, the others the second.
+// projections of a Q4_K_M layer: workgroups below `split` run the first set (one or two row segments: wa, wa1 with na0 and
+// na - na0 rows), the others the second (one matrix).  packed: k / 64 (9 bits) | split (11 bits) | workgroups (12 bits).
 template <class UA, class UB, int PF, int MAXW>
-__global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_pair_kernel(const uint8_t *wa, const uint8_t *wb, const float *x, const float *nw, const int k, const int na,
-                                                                    const int nb, const int split, const int total, const I8Args a, const I8Args b) {
-    if ((int)blockIdx.x < split) gemv_i8_body<UA, 1, PF, false, true, false, MAXW>(I8Lead{wa, x, nullptr, nw, k, na}, a, blockIdx.x, split);
-    else gemv_i8_body<UB, 1, PF, false, true, false, MAXW>(I8Lead{wb, x, nullptr, nw, k, nb}, b, blockIdx.x - split, total - split);
+__global__ void __launch_bounds__(64 * MAXW, 4) gemv_i8_pair_kernel(const uint8_t *wa, const uint8_t *wa1, const uint8_t *wb, const float *x, const float *nw,
+                                                                    const uint32_t packed, const int na, const int na0, const int nb, const I8Args a, const I8Args b) {
+    const int k = (int)(packed & 511u) << 6, split = (int)((packed >> 9) & 2047u), total = (int)(packed >> 20);
+    if ((int)blockIdx.x < split) gemv_i8_body<UA, 1, PF, false, true, false, MAXW>(I8Lead{wa, x, wa1, nw, wa1, k, split, 1, na, na0, na - na0}, a, blockIdx.x);
+    else gemv_i8_body<UB, 1, PF, false, true, false, MAXW>(I8Lead{wb, x, wb, nw, wb, k, total - split, 1, nb, nb, 0}, b, blockIdx.x - split);
 }
 
 }  // namespace jitnn

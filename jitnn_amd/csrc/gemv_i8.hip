@@ -11,15 +11,23 @@ bool gemv_i8_supported(int fmt, int k) {
     return (fmt == F_Q4_K || fmt == F_Q5_K || fmt == F_Q6_K || fmt == F_Q2_K) && k % 256 == 0 && k >= 256 && k <= 1024 * I8_MAX_WAVES;
 }
 
-typedef void (*i8_fn)(const uint8_t *, const float *, int, int, int, const uint8_t *, const float *, const I8Args);
+typedef void (*i8_fused_fn)(const uint8_t *, const float *, const uint8_t *, const float *, const uint8_t *, uint32_t, int, int, int, const I8Args);
+typedef void (*i8_plain_fn)(const uint8_t *, const float *, uint32_t, int, const I8Args);
+struct i8_fn {  // one of the two is set
+    i8_plain_fn plain = nullptr;
+    i8_fused_fn fused = nullptr;
+    explicit operator bool() const { return plain || fused; }
+};
+static i8_fn plain_fn(i8_plain_fn f) { i8_fn r; r.plain = f; return r; }
+static i8_fn fused_fn(i8_fused_fn f) { i8_fn r; r.fused = f; return r; }
 
 template <class U, int PF, int MAXW>
 static i8_fn pick_mode(int mode) {
     switch (mode) {
-    case I8_BIAS: return gemv_i8_kernel<U, 1, PF, true, false, false, MAXW>;
-    case I8_NORM: return gemv_i8_kernel<U, 1, PF, false, true, false, MAXW>;
-    case I8_DUAL: return gemv_i8_kernel<U, 1, PF, false, true, true, MAXW>;
-    default: return gemv_i8_kernel<U, 1, PF, false, false, false, MAXW>;
+    case I8_BIAS: return plain_fn(gemv_i8_plain_kernel<U, 1, PF, true, MAXW>);
+    case I8_NORM: return fused_fn(gemv_i8_kernel<U, 1, PF, false, true, false, MAXW>);
+    case I8_DUAL: return fused_fn(gemv_i8_kernel<U, 1, PF, false, true, true, MAXW>);
+    default: return plain_fn(gemv_i8_plain_kernel<U, 1, PF, false, MAXW>);
     }
 }
 
@@ -33,33 +41,33 @@ static i8_fn pick_pf(int mode, int pf) {
 // its products multiply one activation row each: from five rows on the 16-row tiles of gemv_mfma_kernel are faster
 template <class U, int B>
 static i8_fn pick_batch(int mode, int pf) {
-    if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, B, 1, true, false, false, 4> : gemv_i8_kernel<U, B, 2, true, false, false, 4>;
-    return pf <= 1 ? gemv_i8_kernel<U, B, 1, false, false, false, 4> : gemv_i8_kernel<U, B, 2, false, false, false, 4>;
+    if (mode == I8_BIAS) return plain_fn(pf <= 1 ? gemv_i8_plain_kernel<U, B, 1, true, 4> : gemv_i8_plain_kernel<U, B, 2, true, 4>);
+    return plain_fn(pf <= 1 ? gemv_i8_plain_kernel<U, B, 1, false, 4> : gemv_i8_plain_kernel<U, B, 2, false, 4>);
 }
 
 // Q5_1 and Q2_K: formats no fused launch of the decode step is built for - with or without a bias, nothing else
 template <class U, int MAXW>
 static i8_fn pick_plain(int mode, int pf) {
+    if (mode != I8_BIAS && mode != I8_PLAIN) return i8_fn{};
     if constexpr (MAXW > 4) {  // (long rows: one turn in flight)
-        return mode == I8_BIAS ? gemv_i8_kernel<U, 1, 1, true, false, false, MAXW> : mode == I8_PLAIN ? gemv_i8_kernel<U, 1, 1, false, false, false, MAXW> : nullptr;
+        return plain_fn(mode == I8_BIAS ? gemv_i8_plain_kernel<U, 1, 1, true, MAXW> : gemv_i8_plain_kernel<U, 1, 1, false, MAXW>);
     } else {
-        if (mode == I8_BIAS) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, true, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, true, false, false, MAXW>;
-        if (mode == I8_PLAIN) return pf <= 1 ? gemv_i8_kernel<U, 1, 1, false, false, false, MAXW> : gemv_i8_kernel<U, 1, 2, false, false, false, MAXW>;
-        return nullptr;
+        if (mode == I8_BIAS) return plain_fn(pf <= 1 ? gemv_i8_plain_kernel<U, 1, 1, true, MAXW> : gemv_i8_plain_kernel<U, 1, 2, true, MAXW>);
+        return plain_fn(pf <= 1 ? gemv_i8_plain_kernel<U, 1, 1, false, MAXW> : gemv_i8_plain_kernel<U, 1, 2, false, MAXW>);
     }
 }
 
 template <class U>
 static i8_fn pick_rows(int rows, int waves, int mode, int pf) {
     if (rows == 1) return waves <= 4 ? pick_pf<U, 4>(mode, pf) : pick_plain<U, I8_MAX_WAVES>(mode, 1);  // (long rows: plain or biased, one turn in flight - the fused launches of the decode step have rows of at most 4096 values)
-    if (waves > 4 || rows > 8 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;  // (five to eight rows: two groups of four)
+    if (waves > 4 || rows > 8 || (mode != I8_PLAIN && mode != I8_BIAS)) return i8_fn{};  // (five to eight rows: two groups of four)
     return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }
 
 template <class U>
 static i8_fn pick_rows_plain(int rows, int waves, int mode, int pf) {
     if (rows == 1) return waves <= 4 ? pick_plain<U, 4>(mode, pf) : pick_plain<U, I8_MAX_WAVES>(mode, 1);
-    if (waves > 4 || rows > 4 || (mode != I8_PLAIN && mode != I8_BIAS)) return nullptr;
+    if (waves > 4 || rows > 4 || (mode != I8_PLAIN && mode != I8_BIAS)) return i8_fn{};
     return rows > 2 ? pick_batch<U, 4>(mode, pf) : pick_batch<U, 2>(mode, pf);
 }
 
@@ -74,7 +82,7 @@ static bool q6_aligned(const I8Args &a) {
 
 bool gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a) {
     const int waves = (a.k + 1023) / 1024, rows = a.rows < 1 ? 1 : a.rows;
-    i8_fn fn = nullptr;
+    i8_fn fn;
     switch (fmt) {
     case F_Q4_K: fn = pick_rows<U8<F_Q4_K>>(rows, waves, mode, pf); break;
     case F_Q5_K: fn = pick_rows<U8<F_Q5_K>>(rows, waves, mode, pf); break;
@@ -88,12 +96,17 @@ bool gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, c
     }
     if (!fn) return false;
     const int bt = batch_of(rows);
-    hipLaunchKernelGGL(fn, dim3(blocks, (rows + bt - 1) / bt), dim3(64 * waves), gemv_i8_lds_bytes(waves, bt), s, a.w[0], a.x, a.k, a.n[0] + a.n[1] + a.n[2], (int)blocks, a.w2,
-                       a.nw, a);
+    if (blocks >= (1u << 20) || rows > 8) return false;  // (what the packed argument holds)
+    const dim3 grid(blocks, (rows + bt - 1) / bt), block(64 * waves);
+    const size_t lds = gemv_i8_lds_bytes(waves, bt);
+    const uint32_t packed = i8_pack(a.k, (int)blocks, rows);
+    const int n = a.n[0] + a.n[1] + a.n[2];
+    if (fn.plain) hipLaunchKernelGGL(fn.plain, grid, block, lds, s, a.w[0], a.x, packed, n, a);
+    else hipLaunchKernelGGL(fn.fused, grid, block, lds, s, a.w[0], a.x, mode == I8_DUAL ? a.w2 : a.w[1], a.nw, a.w[2], packed, n, a.n[0], a.n[1], a);
     return true;
 }
 
-typedef void (*i8_pair_fn)(const uint8_t *, const uint8_t *, const float *, const float *, int, int, int, int, int, const I8Args, const I8Args);
+typedef void (*i8_pair_fn)(const uint8_t *, const uint8_t *, const uint8_t *, const float *, const float *, uint32_t, int, int, int, const I8Args, const I8Args);
 
 template <int PF>
 static i8_pair_fn pick_pair(int fa, int fb, bool al) {
@@ -109,9 +122,11 @@ bool gemv_i8_pair_launch(int fmt_a, int fmt_b, int pf, unsigned blocks_a, unsign
     const int waves = (a.k + 1023) / 1024;
     const bool al = fmt_b == F_Q6_K && q6_aligned(b);
     const i8_pair_fn fn = pf <= 1 ? pick_pair<1>(fmt_a, fmt_b, al) : pick_pair<2>(fmt_a, fmt_b, al);
-    if (!fn || waves > 4) return false;
-    hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(64 * waves), gemv_i8_lds_bytes(waves), s, a.w[0], b.w[0], a.x, a.nw, a.k, a.n[0] + a.n[1] + a.n[2],
-                       b.n[0] + b.n[1] + b.n[2], (int)blocks_a, (int)(blocks_a + blocks_b), a, b);
+    // (the first set: at most two row segments, the second one matrix; the split and the grid in 11 and 12 bits of the packed argument)
+    if (!fn || waves > 4 || a.n[2] != 0 || b.n[1] != 0 || b.n[2] != 0 || blocks_a >= 2048 || blocks_a + blocks_b >= 4096) return false;
+    const uint32_t packed = (uint32_t)(a.k >> 6) | (blocks_a << 9) | ((blocks_a + blocks_b) << 20);
+    hipLaunchKernelGGL(fn, dim3(blocks_a + blocks_b), dim3(64 * waves), gemv_i8_lds_bytes(waves), s, a.w[0], a.w[1], b.w[0], a.x, a.nw, packed, a.n[0] + a.n[1], a.n[0], b.n[0], a,
+                       b);
     return true;
 }
 

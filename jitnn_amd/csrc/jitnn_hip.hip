@@ -414,8 +414,11 @@ int launch_xreg2(const XregCall &c0, const XregCall &c1, hipStream_t stream) {
         if (blocks_a > ga) blocks_a = ga;
         int blocks_b = total - blocks_a;
         if (blocks_b > gb) blocks_b = gb;
-        if (!gemv_i8_pair_launch(ca.w[0]->fmt, cb.w[0]->fmt, pf > 2 ? 2 : pf, (unsigned)blocks_a, (unsigned)blocks_b, stream, a, b))
-            return fail(JITNN_HIP_EDEVICE, "no INT8 GEMV kernel for the formats %d and %d in one launch", ca.w[0]->fmt, cb.w[0]->fmt);
+        if (!gemv_i8_pair_launch(ca.w[0]->fmt, cb.w[0]->fmt, pf > 2 ? 2 : pf, (unsigned)blocks_a, (unsigned)blocks_b, stream, a, b)) {
+            // (a split the shared launch has no room for - three matrices of the first format, two of the second: a launch each)
+            if (int rc = launch_i8(ca, stream)) return rc;
+            return launch_i8(cb, stream);
+        }
         HIP_TRY(hipGetLastError());
         return JITNN_HIP_OK;
     }
