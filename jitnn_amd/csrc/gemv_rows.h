@@ -110,8 +110,8 @@ struct RowsPrepareOut {
     float *inv[3];
 };
 template <bool SWIGLU>
-__global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restrict__ x, const float *__restrict__ up, const RowsPrepareOut o, int rows,
-                                                           int k) {
+__global__ void __launch_bounds__(64) rows_prepare_kernel(const float *__restrict__ x, const float *__restrict__ up, int rows, int k,
+                                                           const RowsPrepareOut o) {  // (what the first loads need in front: preloaded with the wave)
     const int lane = threadIdx.x, b = lane >> 3, part = lane & 7;
     const int c = blockIdx.x, g = blockIdx.y, ncol = k >> 8;
     const int row = g * 8 + b;
@@ -518,9 +518,11 @@ __host__ __device__ constexpr size_t gemv_rows_stage_bytes(int tiles_per_wave) {
 // workgroup otherwise.
 template <int FMT, int T>
 __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ ops,
-                                                                const float *__restrict__ inv, const float *__restrict__ bias,
-                                                                const float *res, float *y, int n, int k, int rows,  // (res may be y)
-                                                                int groups) {
+                                                                const float *__restrict__ inv, int n, int k, int rows, int groups,
+                                                                const float *__restrict__ bias, const float *res, float *y) {  // (res may be y)
+    // (argument order: the first fourteen dwords arrive in scalar registers with the wave - everything the first loads need; y,
+    // which only the last lines use, is asked for here, not between the last product and the first store)
+    asm volatile("" ::"s"(y));
     typedef RTile<FMT> R;
     constexpr int NOPS = R::NOPS;
     extern __shared__ __attribute__((aligned(16))) uint8_t gr_smem[];

@@ -78,8 +78,8 @@ void gemv_rows_prepare_launch(hipStream_t s, const float *x, const float *swiglu
         o.inv[l] = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(scratch[l]) + gemv_rows_ops_bytes(groups, k));
     }
     const dim3 grid(ncol, groups);
-    if (swiglu_up) hipLaunchKernelGGL(rows_prepare_kernel<true>, grid, dim3(64), 0, s, x, swiglu_up, o, rows, k);
-    else hipLaunchKernelGGL(rows_prepare_kernel<false>, grid, dim3(64), 0, s, x, swiglu_up, o, rows, k);
+    if (swiglu_up) hipLaunchKernelGGL(rows_prepare_kernel<true>, grid, dim3(64), 0, s, x, swiglu_up, rows, k, o);
+    else hipLaunchKernelGGL(rows_prepare_kernel<false>, grid, dim3(64), 0, s, x, swiglu_up, rows, k, o);
 }
 
 template <int FMT>
@@ -98,8 +98,8 @@ static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const v
         const int cap = (int)(max_blocks / (unsigned)nbatch), gper = (groups + cap - 1) / cap;
         gy = (groups + gper - 1) / gper;
     }
-    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, bias, res, y, n, k, rows, groups);
-    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, bias, res, y, n, k, rows, groups);
+    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, n, k, rows, groups, bias, res, y);
+    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, n, k, rows, groups, bias, res, y);
 }
 
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,

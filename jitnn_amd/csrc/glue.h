@@ -42,20 +42,26 @@ struct AttCfg {
     static constexpr int CH = D <= 128 ? 32 : 16;  // keys per workgroup
 };
 
+// (Fourteen dwords of arguments, all preloaded into scalar registers with the wave: q, k and v of the new token are one buffer -
+// q [heads, D], k [kv_heads, D], v [kv_heads, D] -, the head counts share a dword, the position carries the rotary pairing in its
+// top bit, the scale is 1 / sqrt(D) and the number of chunks follows from the position.)
 template <int D>
-__global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restrict__ q_raw, const float *__restrict__ k_raw,
-                                                           const float *__restrict__ v_raw, float *__restrict__ kcache,
-                                                           float *__restrict__ vcache, const float *__restrict__ cosv,
-                                                           const float *__restrict__ sinv, float *__restrict__ part, int heads, int kv_heads,
-                                                           int pos, float scale, int interleaved) {
+__global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restrict__ qkv, const float *__restrict__ cosv, const float *__restrict__ sinv,
+                                                           float *__restrict__ kcache, float *__restrict__ vcache, float *__restrict__ part,
+                                                           const uint32_t head_counts, const uint32_t pos_pairing) {
     constexpr int CH = AttCfg<D>::CH, HALF = D / 2, DQ = D / 4;
     __shared__ float Ks[CH][D + 1];
     __shared__ float Vs[CH][D];
     __shared__ float Qs[ATT_GMAX][D];
     __shared__ float Sc[ATT_GMAX][CH];
+    const int heads = (int)(head_counts & 0xffffu), kv_heads = (int)(head_counts >> 16), pos = (int)(pos_pairing & 0x7fffffffu);
+    const bool interleaved = (pos_pairing >> 31) != 0;
+    const float scale = 1.0f / sqrtf((float)D);
+    const float *const q_raw = qkv, *const k_raw = qkv + (size_t)heads * D, *const v_raw = k_raw + (size_t)kv_heads * D;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int group = heads / kv_heads, g = blockIdx.y, c = blockIdx.x, chunks = gridDim.x;
+    const int group = heads / kv_heads, g = blockIdx.y, c = blockIdx.x;
     const int s = pos + 1, j0 = c * CH, nk = min(CH, s - j0);  // this chunk holds keys j0 .. j0 + nk - 1
+    const int chunks = (s + CH - 1) / CH;                      // (the grid's x extent)
     const float *cp = cosv + (size_t)pos * HALF, *sp = sinv + (size_t)pos * HALF;
 
     // ---- the group's query heads, rotated

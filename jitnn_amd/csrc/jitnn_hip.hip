@@ -1507,7 +1507,7 @@ struct jitnn_hip_llama {
     float *norms;                // [layers][2][d] then output norm [d]
     float *kc, *vc;              // [layers][max_ctx][kv][hd]
     float *cosv, *sinv;          // [max_ctx][hd/2]
-    float *xin, *xa, *xb, *xn, *q, *k, *v, *att, *gate, *up, *h, *part, *logits;
+    float *xin, *xa, *xb, *xn, *q, *k, *v, *att, *gate, *up, *h, *part, *logits;  // (k and v: inside the buffer of q, behind it)
     int chunks_max;
     // many-token (prefill) buffers, [pf_cap, ...] each, allocated by the first prefill call and grown when a longer one comes
     int pf_cap;
@@ -1526,8 +1526,9 @@ template <int D>
 void launch_attention(const jitnn_hip_llama *m, int layer, int pos, hipStream_t st) {
     const int chunks = (pos + 1 + AttCfg<D>::CH - 1) / AttCfg<D>::CH;
     const size_t lo = (size_t)layer * m->max_ctx * m->kv * m->hd;
-    hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->k, m->v, m->kc + lo, m->vc + lo, m->cosv, m->sinv,
-                       m->part, m->heads, m->kv, pos, 1.0f / sqrtf((float)D), m->rope_interleaved);
+    // (q, k, v: one buffer, see jitnn_hip_llama_create)
+    hipLaunchKernelGGL(attn_decode_kernel<D>, dim3(chunks, m->kv), dim3(256), 0, st, m->q, m->cosv, m->sinv, m->kc + lo, m->vc + lo, m->part,
+                       (uint32_t)m->heads | ((uint32_t)m->kv << 16), (uint32_t)pos | (m->rope_interleaved ? 0x80000000u : 0u));
     constexpr int NPL = 1024 / D < 8 ? 1024 / D : 8;  // long contexts: more threads per value share the chunks
     if (chunks > 32) hipLaunchKernelGGL((attn_merge_kernel<D, NPL>), dim3(m->heads), dim3(NPL * D), 0, st, m->part, m->att, chunks);
     else hipLaunchKernelGGL((attn_merge_kernel<D, 2>), dim3(m->heads), dim3(2 * D), 0, st, m->part, m->att, chunks);
@@ -1731,6 +1732,7 @@ int jitnn_hip_llama_create(int layers, int d_model, int heads, int kv_heads, int
     if (layers < 1 || d_model < 1 || heads < 1 || kv_heads < 1 || ffn < 1 || vocab < 1 || max_ctx < 1)
         return fail(JITNN_HIP_EINVAL, "non-positive model dimension");
     if (heads % kv_heads != 0) return fail(JITNN_HIP_EINVAL, "grouped-query attention: %d query heads over %d key/value heads", heads, kv_heads);
+    if (heads > 65535) return fail(JITNN_HIP_EINVAL, "%d query heads (the attention kernel's packed head counts hold 16 bits each)", heads);
     if (heads / kv_heads > ATT_GMAX) return fail(JITNN_HIP_EINVAL, "%d query heads per key/value head (at most %d are built)", heads / kv_heads, ATT_GMAX);
     if (head_dim != 64 && head_dim != 128 && head_dim != 192 && head_dim != 256)
         return fail(JITNN_HIP_EINVAL, "head_dim %d (64, 128, 192 and 256 are built)", head_dim);
@@ -1747,12 +1749,16 @@ int jitnn_hip_llama_create(int layers, int d_model, int heads, int kv_heads, int
     struct { float **p; size_t n; } bufs[] = {
         {&m->norms, ((size_t)layers * 2 + 1) * d_model}, {&m->kc, cache}, {&m->vc, cache}, {&m->cosv, (size_t)max_ctx * half},
         {&m->sinv, (size_t)max_ctx * half}, {&m->xin, (size_t)d_model}, {&m->xa, (size_t)d_model}, {&m->xb, (size_t)d_model}, {&m->xn, (size_t)d_model},
-        {&m->q, (size_t)qd}, {&m->k, (size_t)kd}, {&m->v, (size_t)kd}, {&m->att, (size_t)qd}, {&m->gate, (size_t)ffn}, {&m->up, (size_t)ffn},
+        {&m->q, (size_t)qd + 2 * (size_t)kd}, {&m->att, (size_t)qd}, {&m->gate, (size_t)ffn}, {&m->up, (size_t)ffn},
         {&m->h, (size_t)ffn}, {&m->part, (size_t)heads * m->chunks_max * (head_dim + 2)}, {&m->logits, (size_t)vocab}};
     bool ok = m->w != nullptr;
     for (auto &b : bufs) {
         if (!ok) break;
         ok = hipMalloc(b.p, b.n * sizeof(float)) == hipSuccess;
+    }
+    if (ok) {  // the projections of a decode step: q [heads, D], k [kv_heads, D], v [kv_heads, D] in one buffer (one pointer for the attention kernel)
+        m->k = m->q + qd;
+        m->v = m->k + kd;
     }
     if (ok) {
         // cos/sin of t * base^(-2i/D) in double, stored FP32: Rope.tables (core/ops/Rope.java:86-102)
@@ -1782,7 +1788,7 @@ int jitnn_hip_llama_create(int layers, int d_model, int heads, int kv_heads, int
 
 int jitnn_hip_llama_free(jitnn_hip_llama *m) {
     if (!m) return JITNN_HIP_OK;
-    float *bufs[] = {m->norms, m->kc, m->vc, m->cosv, m->sinv, m->xin, m->xa, m->xb, m->xn, m->q, m->k, m->v, m->att, m->gate, m->up, m->h, m->part, m->logits};
+    float *bufs[] = {m->norms, m->kc, m->vc, m->cosv, m->sinv, m->xin, m->xa, m->xb, m->xn, m->q, m->att, m->gate, m->up, m->h, m->part, m->logits};
     for (float *b : bufs)
         if (b) (void)hipFree(b);
     for (float *b : m->pf)
