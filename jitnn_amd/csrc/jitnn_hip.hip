@@ -319,11 +319,11 @@ int launch_i8(const XregCall &c, hipStream_t stream) {
 
 // Two to four activation rows, rows of at most 4096 values: the same kernel with the activations of all rows in registers - the
 // operands and scales of the weights are made once, every row runs its own chains of products.  us per launch against the FP32
-// two-row kernel / gemv_mfma_kernel - Q4_K 14336 x 4096: 9.2 (11.3) at two rows, 11.1 (13.9) at three, 11.5 (13.8) at four; Q4_0
-// 11008 x 4096 at four: 9.9 (11.8); Q8_0 4096 x 4096: 7.0 (10.1); Q6_K 14336 x 4096: 14.7 (23.0).  The number of its 4x4x4 products
+// two-row kernel / gemv_mfma_kernel - Q4_K 14336 x 4096: 8.9 (11.3) at two rows, 10.6 (13.9) at three, 11.3 (13.8) at four; Q4_0
+// 11008 x 4096 at four: 9.6 (11.8); Q8_0 4096 x 4096: 6.7 (10.1); Q6_K 14336 x 4096: 14.3 (23.0).  The number of its 4x4x4 products
 // grows with the rows (four rows: twelve digit planes in three products a step): eight rows (two groups of four along
 // blockIdx.y) stay behind gemv_mfma_kernel, whose 16-row tiles take 14.5 us whatever the rows - from five rows on those stay
-// ahead, except for Q6_K, whose tiles cost the most there (14336 x 4096 at eight rows: 23.1 against 28.4 us).
+// ahead, except for Q6_K, whose tiles cost the most there (14336 x 4096 at eight rows: 22.6 against 28.4 us).
 bool i8_batch_ok(const jitnn_hip_weight *w, int rows) {
     return g.gemv_i8 && rows >= 2 && rows <= (w->fmt == F_Q6_K ? 8 : 4) && gemv_i8_supported(w->fmt, w->k) && w->k <= 4096 && w->n >= 4 && w->nbytes < (1ll << 32) &&
            ((block_values(w->fmt) != 32 && w->fmt != F_Q2_K) || ((uintptr_t)w->dev & 3) == 0);
