@@ -413,7 +413,8 @@ __device__ __forceinline__ void mf_build_operands(const float4 (&v)[8], bool hav
 //   dynamic LDS gemv_mfma_lds_bytes<FMT>().
 template <int FMT>
 __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x,
-                                                                const float *__restrict__ bias, float *__restrict__ y, int n, int k, int rows) {
+                                                                const float *__restrict__ bias, float *__restrict__ y, int n, int k, int rows,
+                                                                int stride) {  // stride: the grid's workgroups (an argument, preloaded with the others: gridDim is fetched from a cold block)
     typedef MTile<FMT> T;
     constexpr int CH = T::BYTES / 16;           // whole 16-byte chunks of a tile row
     constexpr int TAIL = T::BYTES % 16;         // 0, or the 2 bytes of Q6_K's d after 13 chunks
@@ -428,7 +429,7 @@ __global__ void __launch_bounds__(MF_THREADS) gemv_mfma_kernel(const uint8_t *__
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint8_t *const reg = mf_smem + wave * NC * REGION;                                            // this wave's own regions
     float4 *const red = reinterpret_cast<float4 *>(mf_smem + MF_WAVES * NC * REGION);             // [wave][group][32 lanes]
-    const int tiles = k >> 8, ngroups = (n + 15) >> 4, stride = gridDim.x;
+    const int tiles = k >> 8, ngroups = (n + 15) >> 4;
     const size_t rowbytes = (size_t)tiles * T::BYTES;
 
     // this lane's share of a tile's bytes: chunk c = lane + 64 i -> (row c / CH, 16-byte chunk c % CH of that row's run)

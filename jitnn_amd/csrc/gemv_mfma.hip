@@ -18,12 +18,12 @@ KernelRef gemv_mfma_kernel_ref(int fmt) {
 
 void gemv_mfma_launch(int fmt, unsigned blocks, hipStream_t s, const uint8_t *W, const float *x, const float *bias, float *y, int n, int k, int rows) {
     switch (fmt) {
-    case F_Q4_0: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q4_0>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q4_0>(), s, W, x, bias, y, n, k, rows); break;
-    case F_Q4_1: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q4_1>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q4_1>(), s, W, x, bias, y, n, k, rows); break;
-    case F_Q8_0: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q8_0>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q8_0>(), s, W, x, bias, y, n, k, rows); break;
-    case F_Q4_K: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q4_K>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q4_K>(), s, W, x, bias, y, n, k, rows); break;
-    case F_Q5_K: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q5_K>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q5_K>(), s, W, x, bias, y, n, k, rows); break;
-    case F_Q6_K: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q6_K>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q6_K>(), s, W, x, bias, y, n, k, rows); break;
+    case F_Q4_0: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q4_0>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q4_0>(), s, W, x, bias, y, n, k, rows, (int)blocks); break;
+    case F_Q4_1: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q4_1>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q4_1>(), s, W, x, bias, y, n, k, rows, (int)blocks); break;
+    case F_Q8_0: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q8_0>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q8_0>(), s, W, x, bias, y, n, k, rows, (int)blocks); break;
+    case F_Q4_K: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q4_K>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q4_K>(), s, W, x, bias, y, n, k, rows, (int)blocks); break;
+    case F_Q5_K: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q5_K>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q5_K>(), s, W, x, bias, y, n, k, rows, (int)blocks); break;
+    case F_Q6_K: hipLaunchKernelGGL(gemv_mfma_kernel<F_Q6_K>, dim3(blocks), dim3(MF_THREADS), gemv_mfma_lds_bytes<F_Q6_K>(), s, W, x, bias, y, n, k, rows, (int)blocks); break;
     default: break;
     }
 }

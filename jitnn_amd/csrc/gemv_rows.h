@@ -519,10 +519,12 @@ __host__ __device__ constexpr size_t gemv_rows_stage_bytes(int tiles_per_wave) {
 template <int FMT, int T>
 __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ ops,
                                                                 const float *__restrict__ inv, int n, int k, int rows, int groups,
+                                                                const uint32_t grid,  // gridDim.x | gridDim.y << 16 (an argument, preloaded: gridDim is fetched from a cold block)
                                                                 const float *__restrict__ bias, const float *res, float *y) {  // (res may be y)
     // (argument order: the first fourteen dwords arrive in scalar registers with the wave - everything the first loads need; y,
     // which only the last lines use, is asked for here, not between the last product and the first store)
-    asm volatile("" ::"s"(y));
+    asm volatile("" ::"s"(y), "s"(res));
+    const int grid_x = (int)(grid & 0xffffu), grid_y = (int)(grid >> 16);
     typedef RTile<FMT> R;
     constexpr int NOPS = R::NOPS;
     extern __shared__ __attribute__((aligned(16))) uint8_t gr_smem[];
@@ -535,8 +537,8 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
     const size_t rowbytes = (size_t)ncol * R::BYTES;
     // gridDim.y > 1 (matrices with few tiles): workgroup y takes the groups [gper y, gper y + gper) of activation rows - it
     // decodes the same weights as its neighbours and writes whole outputs of its own rows, nothing meets across workgroups
-    if (gridDim.y > 1) {
-        const int gper = (groups + (int)gridDim.y - 1) / (int)gridDim.y, g0 = (int)blockIdx.y * gper;
+    if (grid_y > 1) {
+        const int gper = (groups + grid_y - 1) / grid_y, g0 = (int)blockIdx.y * gper;
         if (g0 >= groups) return;
         ops += (size_t)g0 * ncol * GR_OP_HALVES;
         inv += (size_t)g0 * ncol * 8;
@@ -567,7 +569,7 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
         point(blockIdx.x);
         fetch(wave);
     }
-    for (int tb = blockIdx.x; tb < nbatch; tb += gridDim.x) {
+    for (int tb = blockIdx.x; tb < nbatch; tb += grid_x) {
         if (!ACROSS) {
             point(tb);
             if (wave < ncol) fetch(wave);
@@ -594,8 +596,8 @@ __global__ void __launch_bounds__(GR_THREADS) gemv_rows_kernel(const uint8_t *__
             }
             if (c + GR_WAVES < ncol) {
                 fetch(c + GR_WAVES);
-            } else if (ACROSS && tb + (int)gridDim.x < nbatch) {  // this batch's last column: the first of the next batch
-                point(tb + gridDim.x);
+            } else if (ACROSS && tb + grid_x < nbatch) {  // this batch's last column: the first of the next batch
+                point(tb + grid_x);
                 fetch(wave);
             }
             for (int g = 0; g < groups; ++g) {

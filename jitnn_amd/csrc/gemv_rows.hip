@@ -98,8 +98,8 @@ static void launch(unsigned max_blocks, hipStream_t s, const uint8_t *W, const v
         const int cap = (int)(max_blocks / (unsigned)nbatch), gper = (groups + cap - 1) / cap;
         gy = (groups + gper - 1) / gper;
     }
-    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, n, k, rows, groups, bias, res, y);
-    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, n, k, rows, groups, bias, res, y);
+    if (T == 2) hipLaunchKernelGGL((gemv_rows_kernel<FMT, 2>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(2) + gemv_rows_stage_bytes<FMT>(2), s, W, ops, inv, n, k, rows, groups, blocks | ((unsigned)gy << 16), bias, res, y);
+    else hipLaunchKernelGGL((gemv_rows_kernel<FMT, 1>), dim3(blocks, gy), dim3(GR_THREADS), gemv_rows_lds_bytes(1) + gemv_rows_stage_bytes<FMT>(1), s, W, ops, inv, n, k, rows, groups, blocks | ((unsigned)gy << 16), bias, res, y);
 }
 
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,

@@ -94,8 +94,8 @@ __global__ void fp8_probe_kernel(float *out) {
 // Pure streaming read: every thread xors the 16-byte words it loads; the store can never happen for real data
 // but keeps the loads alive.  U loads in flight per lane (the workgroups stride the buffer together), NT: non-temporal loads.
 template <int U, bool NT>
-__global__ void __launch_bounds__(256) probe_read_kernel(const u32x4 *__restrict__ p, size_t n16, uint32_t *sink) {
-    const size_t stride = (size_t)gridDim.x * 256;
+__global__ void __launch_bounds__(256) probe_read_kernel(const u32x4 *__restrict__ p, size_t n16, uint32_t *sink, uint32_t threads) {
+    const size_t stride = threads;  // (the grid's threads as an argument: gridDim is fetched from a cold argument block by the wave's first instructions)
     u32x4 acc = {0, 0, 0, 0};
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     for (; i + (U - 1) * stride < n16; i += U * stride) {
@@ -1343,7 +1343,7 @@ int jitnn_hip_probe_read_shape_dev(const void *dev, long long nbytes, int workgr
     if (!dev || nbytes < 16 || ((uintptr_t)dev & 15) != 0) return fail(JITNN_HIP_EINVAL, "need a 16-byte aligned buffer of at least 16 bytes");
     if (workgroups_per_cu < 1 || workgroups_per_cu > 16) return fail(JITNN_HIP_EINVAL, "%d workgroups per CU", workgroups_per_cu);
     if (int rc = check_ready()) return rc;
-    typedef void (*fn_t)(const u32x4 *, size_t, uint32_t *);
+    typedef void (*fn_t)(const u32x4 *, size_t, uint32_t *, uint32_t);
     fn_t fn = nullptr;
     switch (loads_in_flight) {
     case 1: fn = nontemporal ? probe_read_kernel<1, true> : probe_read_kernel<1, false>; break;
@@ -1353,7 +1353,8 @@ int jitnn_hip_probe_read_shape_dev(const void *dev, long long nbytes, int workgr
     case 16: fn = nontemporal ? probe_read_kernel<16, true> : probe_read_kernel<16, false>; break;
     default: return fail(JITNN_HIP_EINVAL, "%d loads in flight (1, 2, 4, 8 or 16)", loads_in_flight);
     }
-    hipLaunchKernelGGL(fn, dim3(g.cus * workgroups_per_cu), dim3(256), 0, (hipStream_t)stream, (const u32x4 *)dev, (size_t)nbytes / 16, (uint32_t *)nullptr);
+    hipLaunchKernelGGL(fn, dim3(g.cus * workgroups_per_cu), dim3(256), 0, (hipStream_t)stream, (const u32x4 *)dev, (size_t)nbytes / 16, (uint32_t *)nullptr,
+                       (uint32_t)(g.cus * workgroups_per_cu * 256));
     HIP_TRY(hipGetLastError());
     return JITNN_HIP_OK;
 }
