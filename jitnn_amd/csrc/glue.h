@@ -64,16 +64,8 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
     const int chunks = (s + CH - 1) / CH;                      // (the grid's x extent)
     const float *cp = cosv + (size_t)pos * HALF, *sp = sinv + (size_t)pos * HALF;
 
-    // ---- the group's query heads, rotated
-    for (int i = tid; i < group * HALF; i += 256) {
-        const int h = i / HALF, p = i - h * HALF;
-        const float *r = q_raw + (size_t)(g * group + h) * D;
-        const int i0 = interleaved ? 2 * p : p, i1 = interleaved ? 2 * p + 1 : p + HALF;  // the pair rotated by angle p
-        const float a = r[i0], b = r[i1], cs = cp[p], sn = sp[p];
-        Qs[h][i0] = a * cs - b * sn;
-        Qs[h][i1] = a * sn + b * cs;
-    }
-    // ---- keys and values of the chunk: every load is issued before the first LDS write (one round trip to HBM);
+    // ---- keys and values of the chunk: every load is issued before the first LDS write (one round trip to HBM) - and before
+    // the query heads are fetched, whose wait would otherwise stand in front of these loads: two round trips in a row;
     // the new token's row comes from k_raw / v_raw, rotated, and is appended to the cache on the way
     constexpr int NI = CH * DQ / 256;
     static_assert(CH * DQ % 256 == 0, "whole passes");
@@ -88,6 +80,15 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
             kreg[it] = *reinterpret_cast<const float4 *>(kcache + row + e);
             vreg[it] = *reinterpret_cast<const float4 *>(vcache + row + e);
         }
+    }
+    // ---- the group's query heads, rotated
+    for (int i = tid; i < group * HALF; i += 256) {
+        const int h = i / HALF, p = i - h * HALF;
+        const float *r = q_raw + (size_t)(g * group + h) * D;
+        const int i0 = interleaved ? 2 * p : p, i1 = interleaved ? 2 * p + 1 : p + HALF;  // the pair rotated by angle p
+        const float a = r[i0], b = r[i1], cs = cp[p], sn = sp[p];
+        Qs[h][i0] = a * cs - b * sn;
+        Qs[h][i1] = a * sn + b * cs;
     }
 #pragma unroll
     for (int it = 0; it < NI; ++it) {
