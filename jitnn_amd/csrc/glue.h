@@ -81,6 +81,29 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
             vreg[it] = *reinterpret_cast<const float4 *>(vcache + row + e);
         }
     }
+    // ---- the new token's key and value row (the last chunk only; row jp, the thread that also writes that row's slot below):
+    // requested now, with everything else - fetched where the row is written, its round trip came after all the others, in
+    // the workgroup the launch ends with
+    const int jp = pos - j0, qp = (tid - jp * DQ) & 255;
+    const bool mine = jp >= 0 && jp < CH && qp < DQ;
+    const int ep = 4 * qp;
+    float4 na = make_float4(0.f, 0.f, 0.f, 0.f), nb = na, nc = na, ns = na, nvv = na;
+    if (mine) {
+        const float *r = k_raw + (size_t)g * D;
+        if (interleaved) {  // pairs (2i, 2i + 1): values e, e + 1 turn by angle e / 2, values e + 2, e + 3 by angle e / 2 + 1
+            na = *reinterpret_cast<const float4 *>(r + ep);
+            const float2 c2 = *reinterpret_cast<const float2 *>(cp + (ep >> 1)), s2 = *reinterpret_cast<const float2 *>(sp + (ep >> 1));
+            nc = make_float4(c2.x, c2.y, 0.f, 0.f);
+            ns = make_float4(s2.x, s2.y, 0.f, 0.f);
+        } else {
+            const int p = ep < HALF ? ep : ep - HALF;
+            na = *reinterpret_cast<const float4 *>(r + p);
+            nb = *reinterpret_cast<const float4 *>(r + p + HALF);
+            nc = *reinterpret_cast<const float4 *>(cp + p);
+            ns = *reinterpret_cast<const float4 *>(sp + p);
+        }
+        nvv = *reinterpret_cast<const float4 *>(v_raw + (size_t)g * D + ep);
+    }
     // ---- the group's query heads, rotated
     for (int i = tid; i < group * HALF; i += 256) {
         const int h = i / HALF, p = i - h * HALF;
@@ -93,26 +116,19 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const float *__restric
 #pragma unroll
     for (int it = 0; it < NI; ++it) {
         const int i = tid + it * 256, j = i / DQ, e = (i - j * DQ) * 4;
-        if (j < nk && j0 + j == pos) {
-            const size_t row = ((size_t)pos * kv_heads + g) * D;
-            const float *r = k_raw + (size_t)g * D;
-            if (interleaved) {  // pairs (2i, 2i + 1): values e, e + 1 turn by angle e / 2, values e + 2, e + 3 by angle e / 2 + 1
-                const float4 x = *reinterpret_cast<const float4 *>(r + e);
-                const float c0 = cp[e >> 1], s0 = sp[e >> 1], c1 = cp[(e >> 1) + 1], s1 = sp[(e >> 1) + 1];
-                kreg[it] = make_float4(x.x * c0 - x.y * s0, x.x * s0 + x.y * c0, x.z * c1 - x.w * s1, x.z * s1 + x.w * c1);
-            } else {
-                const int p = e < HALF ? e : e - HALF;
-                const float4 a = *reinterpret_cast<const float4 *>(r + p), b = *reinterpret_cast<const float4 *>(r + p + HALF);
-                const float4 cs = *reinterpret_cast<const float4 *>(cp + p), sn = *reinterpret_cast<const float4 *>(sp + p);
-                if (e < HALF) kreg[it] = make_float4(a.x * cs.x - b.x * sn.x, a.y * cs.y - b.y * sn.y, a.z * cs.z - b.z * sn.z, a.w * cs.w - b.w * sn.w);
-                else kreg[it] = make_float4(a.x * sn.x + b.x * cs.x, a.y * sn.y + b.y * cs.y, a.z * sn.z + b.z * cs.z, a.w * sn.w + b.w * cs.w);
-            }
-            vreg[it] = *reinterpret_cast<const float4 *>(v_raw + (size_t)g * D + e);
-            *reinterpret_cast<float4 *>(kcache + row + e) = kreg[it];
-            *reinterpret_cast<float4 *>(vcache + row + e) = vreg[it];
-        }
         Ks[j][e] = kreg[it].x; Ks[j][e + 1] = kreg[it].y; Ks[j][e + 2] = kreg[it].z; Ks[j][e + 3] = kreg[it].w;
         *reinterpret_cast<float4 *>(&Vs[j][e]) = vreg[it];
+    }
+    if (mine) {  // (the slot of row jp was written - with zeros - by this same thread in the loop above)
+        float4 kr;
+        if (interleaved) kr = make_float4(na.x * nc.x - na.y * ns.x, na.x * ns.x + na.y * nc.x, na.z * nc.y - na.w * ns.y, na.z * ns.y + na.w * nc.y);
+        else if (ep < HALF) kr = make_float4(na.x * nc.x - nb.x * ns.x, na.y * nc.y - nb.y * ns.y, na.z * nc.z - nb.z * ns.z, na.w * nc.w - nb.w * ns.w);
+        else kr = make_float4(na.x * ns.x + nb.x * nc.x, na.y * ns.y + nb.y * nc.y, na.z * ns.z + nb.z * nc.z, na.w * ns.w + nb.w * nc.w);
+        const size_t row = ((size_t)pos * kv_heads + g) * D;
+        *reinterpret_cast<float4 *>(kcache + row + ep) = kr;
+        *reinterpret_cast<float4 *>(vcache + row + ep) = nvv;
+        Ks[jp][ep] = kr.x; Ks[jp][ep + 1] = kr.y; Ks[jp][ep + 2] = kr.z; Ks[jp][ep + 3] = kr.w;
+        *reinterpret_cast<float4 *>(&Vs[jp][ep]) = nvv;
     }
     __syncthreads();
     // ---- scores: one (query head, key) pair per thread
