@@ -14,11 +14,13 @@
 //
 // Work decomposition: a workgroup has one wave per 1024 values of the row (four for K = 4096); a turn of the
 // workgroup is a group of four consecutive weight rows, wave w multiplying its 1024-value slice of them.  The slice's
-// partial sums of a turn leave the wave through a two-step DPP fold (16 floats to LDS); every I8_FLUSH turns the
+// partial sums of a turn leave the wave through a two-step DPP fold (16 floats to LDS); every i8_flush() turns the
 // workgroup meets at a barrier and one thread per output adds the partial sums in a fixed order - no atomics, the
 // result does not depend on the launch shape.  Weight bytes are prefetched PF turns ahead through a register ring with
 // unconditional loads (turns past the end get a descriptor of extent zero: zeros, no traffic) so the hardware's
-// in-order load counter is waited on exactly.
+// in-order load counter is waited on exactly.  What a wave needs before its first loads arrives in scalar registers with
+// the wave (leading kernel arguments, preloaded by the hardware: I8Lead); what the flush needs is fetched under the
+// wait for the first weights - a cold argument block is a round trip to memory wherever it is first touched.
 //
 // A slice that holds an activation that is not finite takes a slow path (every weight decoded by the bit-exact
 // expression of the dequantiser and multiplied in FP32) so that +-Inf and NaN come out as the reference's FP64 sum

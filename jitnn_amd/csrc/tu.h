@@ -93,8 +93,9 @@ void gemv_rows_prepare_launch(hipStream_t s, const float *x, const float *swiglu
 void gemv_rows_main_launch(int fmt, unsigned max_blocks, hipStream_t s, const uint8_t *W, const void *scratch, const float *bias, const float *res, float *y,
                            int n, int k, int rows);
 
-// ---- gemv_i8.hip: gemv_i8_kernel<unit>: GEMV of one to four activation rows with INT8 matrix-core products on the raw quants
-// Arguments of gemv_i8_kernel: up to three matrices of one format and row length share a launch and an activation vector (row segments
+// ---- gemv_i8.hip: gemv_i8_kernel / gemv_i8_plain_kernel<unit>: GEMV of one to four activation rows with INT8 matrix-core products on the
+// raw quants.  The argument block of the kernels (the launchers put what a wave's first loads need in front of it, as scalar
+// arguments the hardware preloads): up to three matrices of one format and row length share a launch and an activation vector (row segments
 // numbered one after the other).  DUAL: w2 is a second matrix of the shape of w[0]; y[0] = silu(w[0] x) * (w2 x).
 struct I8Args {
     const uint8_t *w[3];
@@ -111,7 +112,7 @@ struct I8Args {
 
 constexpr int I8_PLAIN = 0, I8_BIAS = 1, I8_NORM = 2, I8_DUAL = 3;  // DUAL: norm + the SwiGLU pair
 bool gemv_i8_supported(int fmt, int k);
-// blockDim = 64 * ceil(k / 1024); pf = turns of weight bytes in flight per wave beyond the one being multiplied (1..3; 1..2 for
+// One wave per 1024 values of a row (the launchers set the workgroup size); pf = turns of weight bytes in flight per wave beyond the one being multiplied (1..3; 1..2 for
 // two to four activation rows - a.rows in 2..4, rows of at most 4096 values, modes I8_PLAIN and I8_BIAS only)
 bool gemv_i8_launch(int fmt, int mode, int pf, unsigned blocks, hipStream_t s, const I8Args &a);  // false: no kernel for this call, nothing launched
 bool gemv_i8_pair_supported(int fmt_a, int fmt_b);
