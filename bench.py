@@ -125,6 +125,11 @@ class Workload:
             rc |= f(h, xp, b, None, yp, stream)
         if events:
             e1.record()
+        # (the host polls the stream until it is done, then synchronises: a host thread parked in the blocking wait takes some
+        # 10 us to wake up, half a microsecond per step of a 20-step region that is not the device's)
+        cur = torch.cuda.current_stream()
+        while not cur.query():
+            pass
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         if rc != 0:
