@@ -681,16 +681,19 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
     // ---- the activations this lane stages: 16 values of chunk c of every activation row
     const int xf = U::x_first(c, j);
     float4 xv[B][4], nv[4];
+    // (unconditional loads from clamped addresses - chunk c and the activation row exist -, zeroed afterwards where the lane has
+    // nothing to stage: a load behind a condition is a branch around it, eight of them stood in front of the first weight load)
 #pragma unroll
     for (int r = 0; r < B; ++r) {
-        const bool have = inrow && (B == 1 || rb + r < ld.rows);
+        const int xr = B == 1 ? rb + r : min(rb + r, ld.rows - 1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) xv[r][i] = have ? reinterpret_cast<const float4 *>(ld.x + (size_t)(rb + r) * k + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int i = 0; i < 4; ++i) xv[r][i] = reinterpret_cast<const float4 *>(ld.x + (size_t)xr * k + xf)[i];
     }
     if (NORM) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) nv[i] = inrow ? reinterpret_cast<const float4 *>(ld.nw + xf)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int i = 0; i < 4; ++i) nv[i] = reinterpret_cast<const float4 *>(ld.nw + xf)[i];
     }
+    __builtin_amdgcn_sched_barrier(0);  // (the activations' loads first: loads return in order, and the wait for them must not be one for weight bytes)
 
     // ---- the ring of weight bytes
     typename U::Raw buf[NB];
@@ -723,6 +726,22 @@ __device__ __forceinline__ void gemv_i8_body(const I8Lead &ld, const I8Args &a, 
 #pragma unroll
     for (int i = 0; i < NB; ++i) fill(buf[i], i);
     __builtin_amdgcn_sched_barrier(0);  // the weight loads leave before anything waits for the activations
+    {
+        auto keep = [](float4 &v, uint32_t m) {  // (a mask, not a branch)
+            v.x = __uint_as_float(__float_as_uint(v.x) & m); v.y = __uint_as_float(__float_as_uint(v.y) & m);
+            v.z = __uint_as_float(__float_as_uint(v.z) & m); v.w = __uint_as_float(__float_as_uint(v.w) & m);
+        };
+#pragma unroll
+        for (int r = 0; r < B; ++r) {
+            const uint32_t m = inrow && (B == 1 || rb + r < ld.rows) ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) keep(xv[r][i], m);
+        }
+        if (NORM) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) keep(nv[i], inrow ? 0xffffffffu : 0u);
+        }
+    }
 
     if (NORM) {
         // RMSNorm (ops/RowNorm.java:286-306): y = W (x * nw / sqrt(mean(x^2) + eps)).  The factor 1 / sqrt(...) is one number for the
